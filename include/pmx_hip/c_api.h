@@ -1,0 +1,300 @@
+/*
+ * C ABI of the MI355X (gfx950) int8-KV dynamic-batching attention path.
+ *
+ * The reference library has no C ABI: its boundary is the C++ class
+ * ppl::kernel::llm::cuda::pmx::dynamic_batching_multi_head_cache_attention
+ * (include/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention.h:25-159).  The
+ * entry points below are what that class bottoms out in -- one per kernel launch
+ * site of src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/kernel.cu -- with
+ * plain pointers and sizes only, so that any FFI can bind them.  The C++ class in
+ * multi_head_cache_attention.h (this directory) marshals its cfg into these.
+ *
+ * Conventions shared by every entry point:
+ *   - all pointers are device pointers unless stated otherwise; the caller owns
+ *     every buffer; nothing is allocated, freed or synchronised by the library;
+ *   - work is enqueued on `stream` (a hipStream_t; NULL = the null stream);
+ *   - half tensors are IEEE binary16; index arrays are int64;
+ *   - cache element (token t, layer l, K/V plane kv, kv head h, channel d) lives at
+ *       t*cache_stride_s + l*cache_stride_l + kv*cache_stride_kv + h*cache_stride_h + d
+ *     in the int8 cache, and its group-of-8 scale at that index / 8 in the scale
+ *     tensor (kernel.cu:117-126); all four strides must be multiples of 8;
+ *   - cache_mode 0: token t of sequence b is row cachestarts[b] + t;
+ *     cache_mode 1: row cachestarts[b*cachestarts_stride_b + t/128] + t%128
+ *     (kernel.cu:97-100, 365-368);
+ *   - return value: a pmxhip_status_t (0 = success).
+ */
+#ifndef PMX_HIP_C_API_H_
+#define PMX_HIP_C_API_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define PMXHIP_API __attribute__((visibility("default")))
+#else
+#define PMXHIP_API
+#endif
+
+/* Same numeric values as ppl::common::RetCode (ppl.common retcode.h, not part of
+ * the reference tree; only these four are used on this path). */
+typedef enum pmxhip_status_t {
+    PMXHIP_SUCCESS = 0,
+    PMXHIP_OTHER_ERROR = 1,
+    PMXHIP_UNSUPPORTED = 2,
+    PMXHIP_INVALID_VALUE = 4
+} pmxhip_status_t;
+
+typedef struct ihipStream_t* pmxhip_stream_t; /* == hipStream_t */
+
+#define PMXHIP_PAGE_SIZE 128 /* UNIFORM_PAGE_SIZE, kernel.cu:31 */
+
+/* ---- quantise/append ------------------------------------------------------
+ * Replaces dynamic_batching_kv_cache_quantize_kernel_param (kernel.cu:64-84) and
+ * the launch in forward_kvstore (kernel.cu:2013-2057).  Fields up to `scale` are
+ * the reference's, in the reference's order; the rest are what the launch site
+ * reads from cfg. */
+typedef struct pmxhip_kvstore_params {
+    const void* current_key;   /* half (S, KVH, D) */
+    const void* current_value; /* half (S, KVH, D) */
+    const int64_t* seqstarts;  /* (B + 1) */
+    const int64_t* cachestarts; /* (B) or (B, MaxP) */
+    const int64_t* start_pos;  /* (B) */
+    int64_t num_layer;
+    int64_t layer_idx;
+    int64_t num_kv_heads;
+    int64_t head_dim;
+    int32_t page_size; /* used when cache_mode == 1; must be 128 */
+    int64_t current_key_stride_s;
+    int64_t current_value_stride_s;
+    int64_t cache_stride_s;
+    int64_t cache_stride_l;
+    int64_t cache_stride_h;
+    int64_t cache_stride_kv;
+    int64_t cachestarts_stride_b;
+    void* cache; /* int8 */
+    void* scale; /* half */
+    /* launch-site values (cfg.batch, cfg.max_seqlen, cfg.cache_mode) */
+    int64_t batch;
+    int64_t max_seqlen; /* upper bound of seqstarts[b+1]-seqstarts[b] */
+    int32_t cache_mode; /* 0 contiguous, 1 paged */
+} pmxhip_kvstore_params;
+
+PMXHIP_API int pmxhip_kv_cache_quantize(const pmxhip_kvstore_params* p, pmxhip_stream_t stream);
+
+/* ---- decode attention (one query token per sequence) -----------------------
+ * Replaces dynamic_batching_decoding_cache_attention_kernel_param
+ * (kernel.cu:35-62) and forward_decode (kernel.cu:2059-2125), including the
+ * split-KV partials and their combine (kernel.cu:600-678).  The split is not a
+ * fixed block count: the kv tokens of all decode sequences form one stream that
+ * is cut into `num_token_ranges` equal ranges, one workgroup each, and a second
+ * kernel merges the pieces of every sequence that spans more than one range. */
+typedef struct pmxhip_decode_params {
+    const void* query;     /* half (B_dec, Hq, D); row = sequence index */
+    const void* attn_mask; /* half, optional (NULL = none) */
+    void* output;          /* half (B_dec, Hq, D) */
+    const void* cache;     /* int8 */
+    const void* scale;     /* half */
+    const int64_t* cachestarts;
+    const int64_t* kvstarts; /* (B_dec + 1) */
+    float attn_scale;
+    int64_t layer_idx;
+    int64_t num_kv_repeats; /* Hq / KVH */
+    int64_t page_size;
+    int64_t query_stride_s;
+    int64_t output_stride_s;
+    int64_t mask_stride_s;
+    int64_t mask_stride_h;
+    int64_t cache_stride_s;
+    int64_t cache_stride_l;
+    int64_t cache_stride_h;
+    int64_t cache_stride_kv;
+    int64_t cachestarts_stride_b;
+    /* launch-site values */
+    int64_t decoding_batches;
+    int64_t num_heads;
+    int64_t num_kv_heads;
+    int64_t head_dim;
+    int32_t cache_mode;
+    /* split-KV plan: from pmxhip_decode_plan(); workspace >= plan.workspace_size */
+    int32_t num_token_ranges;
+    void* workspace;
+    int64_t workspace_size;
+} pmxhip_decode_params;
+
+typedef struct pmxhip_decode_plan {
+    int32_t num_token_ranges;   /* workgroups along the kv-token stream */
+    int32_t kv_heads_per_group; /* kv heads one workgroup serves */
+    int32_t q_heads_per_pass;   /* query heads per kv head held in registers at once */
+    int32_t num_passes;         /* ceil(num_kv_repeats / q_heads_per_pass) */
+    int64_t partial_out_size;   /* bytes: float32 partial outputs */
+    int64_t partial_ml_size;    /* bytes: float32 (running max, exp-sum) pairs */
+    int64_t workspace_size;     /* total bytes */
+} pmxhip_decode_plan;
+
+/* Host-only.  `compute_units` is hipDeviceProp_t::multiProcessorCount.
+ * `num_token_ranges_hint` 0 = choose; > 0 = use exactly this many ranges. */
+PMXHIP_API int pmxhip_decode_plan_make(int64_t decoding_batches, int64_t num_heads, int64_t num_kv_heads,
+                                       int64_t head_dim, int64_t max_kvlen, int32_t compute_units,
+                                       int32_t num_token_ranges_hint, pmxhip_decode_plan* plan);
+
+PMXHIP_API int pmxhip_decode_attention(const pmxhip_decode_params* p, pmxhip_stream_t stream);
+
+/* ---- split-KV combine on caller-supplied pieces ----------------------------
+ * The merge of kernel.cu:617-665 as a stand-alone kernel: for each of `rows`
+ * (sequence, head) pairs, merges pieces [piece_begin[r], piece_end[r]) of
+ *   partial_out float32 (pieces, D)   normalised partial outputs
+ *   partial_ml  float32 (pieces, 2)   (running max in log2 units, exp-sum)
+ * into output row r (half, D).  Rows with no pieces produce zeros. */
+PMXHIP_API int pmxhip_splitkv_combine(const float* partial_out, const float* partial_ml,
+                                      const int64_t* piece_begin, const int64_t* piece_end,
+                                      int64_t rows, int64_t head_dim, void* output,
+                                      pmxhip_stream_t stream);
+
+/* ---- multi-query-token (chunked prefill) attention over the int8 cache -----
+ * Replaces the flash_attn2_paged_fmha call of forward_prefill
+ * (kernel.cu:2127-2179; include/ppl/kernel/llm/cuda/flash_attn2/fmha.h:73).
+ * Sequences [decoding_batches, batch) are prefill; query/output rows are
+ * addressed through seqstarts, kv length through kvstarts, cache rows through
+ * cachestarts; causal masking is bottom-right aligned (mask.h:186). */
+typedef struct pmxhip_prefill_params {
+    const void* query; /* half (S, Hq, D) */
+    void* output;      /* half (S, Hq, D) */
+    const void* cache;
+    const void* scale;
+    const int64_t* seqstarts;   /* (B + 1), whole batch */
+    const int64_t* kvstarts;    /* (B + 1), whole batch */
+    const int64_t* cachestarts; /* whole batch */
+    float attn_scale;
+    int32_t is_causal;
+    int64_t batch;
+    int64_t decoding_batches;
+    int64_t max_seqlen;
+    int64_t max_kvlen;
+    int64_t layer_idx;
+    int64_t num_heads;
+    int64_t num_kv_heads;
+    int64_t head_dim;
+    int32_t cache_mode;
+    int64_t page_size;
+    int64_t query_stride_s;
+    int64_t output_stride_s;
+    int64_t cache_stride_s;
+    int64_t cache_stride_l;
+    int64_t cache_stride_h;
+    int64_t cache_stride_kv;
+    int64_t cachestarts_stride_b;
+} pmxhip_prefill_params;
+
+PMXHIP_API int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t stream);
+
+/* ---- the operator class behind a C handle -----------------------------------
+ * Drives the C++ class (heuristic_prepare / forward_*) so that a non-C++ host
+ * can use the reference's operator interface unchanged.  Argument meaning and
+ * order follow multi_head_cache_attention.h:107-148 of the reference. */
+typedef struct pmxhip_tensor_shape {
+    int32_t dim_count;
+    int32_t data_type; /* pmxhip DATATYPE_* value; 5 = float16 */
+    int64_t dims[4];
+} pmxhip_tensor_shape;
+
+typedef struct pmxhip_mhca_prepare_args {
+    int32_t compute_units;              /* device_prop.multiProcessorCount */
+    int64_t shared_mem_per_block_optin; /* device_prop.sharedMemPerBlockOptin */
+    pmxhip_tensor_shape query_shape;
+    const void* query;
+    pmxhip_tensor_shape current_key_shape;
+    const void* current_key;
+    pmxhip_tensor_shape current_value_shape;
+    const void* current_value;
+    pmxhip_tensor_shape attn_mask_shape;
+    const void* attn_mask;
+    const void* seqstarts;
+    const void* kvstarts;
+    const void* cachestarts;
+    const void* start_pos;
+    const void* alibi_slopes;
+    int32_t is_causal;
+    int64_t batch;
+    int64_t decoding_batches;
+    int64_t max_seqlen;
+    int64_t max_kvlen;
+    int64_t layer_idx;
+    int64_t num_layer;
+    int64_t num_heads;
+    int64_t num_kv_heads;
+    int64_t head_dim;
+    int32_t cache_mode;
+    int64_t page_size;
+    int64_t cache_stride_s;
+    int64_t cache_stride_l;
+    int64_t cache_stride_h;
+    int64_t cache_stride_kv;
+    int64_t cachestarts_stride_b;
+    int32_t enable_cache_prefill;
+    int32_t enable_sharemem_mhca;
+    int32_t enable_infinity_mhca;
+    int32_t enable_infinity_gqca;
+    int32_t specify_decoding_multi_block;
+    int32_t specify_decoding_tpb;
+    void* cache;
+    void* scale;
+    pmxhip_tensor_shape output_shape;
+    void* output;
+} pmxhip_mhca_prepare_args;
+
+/* What heuristic_prepare derived (the "produce by prepare function" block of the
+ * reference's config, multi_head_cache_attention.h:76-98). */
+typedef struct pmxhip_mhca_derived {
+    int64_t prefill_batches;
+    int64_t q_stride_s, k_stride_s, v_stride_s, o_stride_s;
+    int64_t mask_stride_s, mask_stride_h;
+    float attn_scale;
+    int64_t num_kv_repeats;
+    int32_t decoding_algo;
+    int64_t decoding_threads_per_block;
+    int64_t decoding_multi_block_size;
+    int64_t decoding_multi_block_partial_out_size;
+    int64_t decoding_multi_block_partial_log_sum_exp_size;
+    int64_t decoding_multi_block_counter_size;
+    int64_t workspace_size;
+} pmxhip_mhca_derived;
+
+typedef struct pmxhip_mhca* pmxhip_mhca_t;
+
+PMXHIP_API pmxhip_mhca_t pmxhip_mhca_create(void);
+PMXHIP_API void pmxhip_mhca_destroy(pmxhip_mhca_t op);
+PMXHIP_API int pmxhip_mhca_heuristic_prepare(pmxhip_mhca_t op, const pmxhip_mhca_prepare_args* args);
+PMXHIP_API int pmxhip_mhca_get_derived(pmxhip_mhca_t op, pmxhip_mhca_derived* out);
+PMXHIP_API int pmxhip_mhca_set_workspace(pmxhip_mhca_t op, void* workspace);
+PMXHIP_API int pmxhip_mhca_forward_kvstore(pmxhip_mhca_t op, pmxhip_stream_t stream);
+PMXHIP_API int pmxhip_mhca_forward_decode(pmxhip_mhca_t op, pmxhip_stream_t stream);
+PMXHIP_API int pmxhip_mhca_forward_prefill(pmxhip_mhca_t op, pmxhip_stream_t stream);
+PMXHIP_API int pmxhip_mhca_forward(pmxhip_mhca_t op, pmxhip_stream_t stream);
+
+/* ---- key_value_cache -------------------------------------------------------
+ * The append step under the operator name the serving stack uses for it
+ * (pmx op KeyValueCache); same arguments as pmxhip_kvstore_params, flattened.
+ * In the reference tree the step is forward_kvstore (kernel.cu:2013-2057). */
+PMXHIP_API int pmxhip_key_value_cache(
+    pmxhip_stream_t stream,
+    const void* current_key, const void* current_value,
+    const int64_t* seqstarts, const int64_t* cachestarts, const int64_t* start_pos,
+    int64_t batch, int64_t max_seqlen, int64_t num_layer, int64_t layer_idx,
+    int64_t num_kv_heads, int64_t head_dim,
+    int32_t cache_mode, int64_t page_size,
+    int64_t cache_stride_s, int64_t cache_stride_l, int64_t cache_stride_h, int64_t cache_stride_kv,
+    int64_t cachestarts_stride_b,
+    void* cache, void* scale);
+
+/* Library identity / build check (host only). */
+PMXHIP_API const char* pmxhip_version(void);
+PMXHIP_API const char* pmxhip_last_error(void); /* thread-local text of the last failure */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PMX_HIP_C_API_H_ */

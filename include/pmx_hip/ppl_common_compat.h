@@ -1,0 +1,82 @@
+/*
+ * Minimal stand-ins for the ppl.common types the operator interface names.
+ * ppl.common is an external dependency of the reference (cmake/deps.cmake:90)
+ * and is not in its tree; only what
+ * include/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention.h and
+ * src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/utils.cu:68-131,269
+ * touch is provided: RetCode, datatype_t, and TensorShape's GetDim /
+ * GetDimCount / GetDataType / CalcElementsExcludingPadding.
+ * When building inside a tree that has the real ppl.common, define
+ * PMX_HIP_USE_PPL_COMMON and these are taken from there instead.
+ */
+#ifndef PMX_HIP_PPL_COMMON_COMPAT_H_
+#define PMX_HIP_PPL_COMMON_COMPAT_H_
+
+#ifdef PMX_HIP_USE_PPL_COMMON
+#include "ppl/common/retcode.h"
+#include "ppl/common/tensor_shape.h"
+#else
+
+#include <cstdint>
+#include <initializer_list>
+
+namespace ppl { namespace common {
+
+typedef uint32_t RetCode;
+enum {
+    RC_SUCCESS = 0,
+    RC_OTHER_ERROR = 1,
+    RC_UNSUPPORTED = 2,
+    RC_OUT_OF_MEMORY = 3,
+    RC_INVALID_VALUE = 4,
+};
+
+typedef uint32_t datatype_t;
+enum {
+    DATATYPE_UNKNOWN = 0,
+    DATATYPE_FLOAT16 = 5,
+    DATATYPE_FLOAT32 = 6,
+    DATATYPE_INT8 = 10,
+    DATATYPE_INT64 = 13,
+};
+
+class TensorShape final {
+public:
+    static constexpr uint32_t kMaxDims = 8;
+
+    TensorShape() : dim_count_(0), data_type_(DATATYPE_UNKNOWN) {
+        for (uint32_t i = 0; i < kMaxDims; ++i) dims_[i] = 0;
+    }
+    TensorShape(datatype_t dt, std::initializer_list<int64_t> dims) : TensorShape() {
+        data_type_ = dt;
+        for (int64_t d : dims) {
+            if (dim_count_ < kMaxDims) dims_[dim_count_++] = d;
+        }
+    }
+
+    void SetDataType(datatype_t dt) { data_type_ = dt; }
+    datatype_t GetDataType() const { return data_type_; }
+
+    void SetDimCount(uint32_t n) { dim_count_ = n < kMaxDims ? n : kMaxDims; }
+    uint32_t GetDimCount() const { return dim_count_; }
+
+    void SetDim(uint32_t i, int64_t v) { if (i < kMaxDims) dims_[i] = v; }
+    int64_t GetDim(uint32_t i) const { return i < kMaxDims ? dims_[i] : 0; }
+
+    uint64_t CalcElementsExcludingPadding() const {
+        if (dim_count_ == 0) return 0;
+        uint64_t n = 1;
+        for (uint32_t i = 0; i < dim_count_; ++i) n *= (uint64_t)dims_[i];
+        return n;
+    }
+
+private:
+    uint32_t dim_count_;
+    datatype_t data_type_;
+    int64_t dims_[kMaxDims];
+};
+
+}} // namespace ppl::common
+
+#endif // PMX_HIP_USE_PPL_COMMON
+#endif // PMX_HIP_PPL_COMMON_COMPAT_H_

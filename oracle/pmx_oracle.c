@@ -1,0 +1,415 @@
+/*
+ * TEST INFRASTRUCTURE ONLY -- CPU oracle for the int8-KV dynamic-batching path.
+ *
+ * This file restates, in plain C, the arithmetic of the reference's
+ *   src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/kernel.cu   (KC below)
+ *   src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/utils.cu    (UC below)
+ *   src/ppl/kernel/llm/cuda/flash_attn2/src/mask.h                      (causal alignment)
+ * so that the HIP kernels can be checked against it.  Nothing in the shipped
+ * library links, loads or calls this file: only tests, the smoke check and the
+ * cpu_baseline leg of the benchmark do.
+ *
+ * Pinning status of each function (what independent evidence fixes its result):
+ *   pmx_oracle_kv_cache_quantize   pinned: hand-derived known answers, exhaustive
+ *                                  fp16 sweep against an independent numpy
+ *                                  restatement, invariants (tests/test_oracle_*).
+ *                                  The reference holds no golden vectors for it.
+ *   pmx_oracle_decode_attention    pinned: closed forms (kvlen=1, zero query,
+ *                                  dominant key), torch SDPA on the dequantised
+ *                                  cache, naive python loops on tiny inputs.
+ *   pmx_oracle_prefill_attention   pinned: torch SDPA with explicit bottom-right
+ *                                  causal mask, qlen=1 rows equal decode.
+ *   pmx_oracle_splitkv_combine     pinned: any split of the kv range equals the
+ *                                  single pass (log-sum-exp associativity).
+ *   The reference itself cannot be compiled here (CUDA, inline PTX, CUTLASS, and
+ *   dependencies fetched at configure time), so bit patterns of its fp16
+ *   attention output are "parity unpinned"; the contract is the fp32
+ *   dequantised attention within 2e-3 abs / 1e-2 rel.
+ *
+ * All half-precision values travel as uint16_t bit patterns.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* ------------------------------------------------------------------------- */
+/* IEEE binary16 <-> binary32, bit level, round-to-nearest-even, subnormals   */
+/* kept (no flush-to-zero).                                                   */
+/* ------------------------------------------------------------------------- */
+
+static inline float bits_to_float(uint32_t u)
+{
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+static inline uint32_t float_to_bits(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+
+float pmx_oracle_half_to_float(uint16_t h)
+{
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    const uint32_t exp = (h >> 10) & 0x1fu;
+    uint32_t man = h & 0x3ffu;
+    if (exp == 0) {
+        if (man == 0)
+            return bits_to_float(sign);
+        /* subnormal: value = man * 2^-24, exactly representable in binary32 */
+        float v = (float)man * (1.0f / 16777216.0f);
+        return bits_to_float(float_to_bits(v) | sign);
+    }
+    if (exp == 31)
+        return bits_to_float(sign | 0x7f800000u | (man << 13));
+    return bits_to_float(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+uint16_t pmx_oracle_float_to_half(float f)
+{
+    const uint32_t x = float_to_bits(f);
+    const uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    const uint32_t ax = x & 0x7fffffffu;
+    if (ax >= 0x7f800000u) /* inf / nan */
+        return (uint16_t)(sign | 0x7c00u | ((ax > 0x7f800000u) ? 0x200u : 0u));
+    if (ax >= 0x477ff000u) /* >= 65520 rounds to inf */
+        return (uint16_t)(sign | 0x7c00u);
+    if (ax < 0x33000001u) /* <= 2^-25 rounds to zero (tie at 2^-25 goes to even = 0) */
+        return sign;
+    int32_t e = (int32_t)(ax >> 23) - 127; /* unbiased exponent */
+    uint32_t m = (ax & 0x7fffffu) | 0x800000u; /* 24-bit significand */
+    int shift; /* bits dropped from the 24-bit significand */
+    uint32_t base;
+    if (e < -14) { /* subnormal half: unit = 2^-24 */
+        shift = 13 + (-14 - e);
+        base = 0;
+    } else {
+        shift = 13;
+        base = (uint32_t)(e + 15) << 10;
+    }
+    uint32_t q = m >> shift;
+    const uint32_t rem = m & ((1u << shift) - 1u);
+    const uint32_t half_ulp = 1u << (shift - 1);
+    if (rem > half_ulp || (rem == half_ulp && (q & 1u)))
+        q += 1; /* may carry into the exponent field, which is the right result */
+    if (e >= -14)
+        q -= 0x400u; /* drop the implicit bit: base already holds the exponent */
+    return (uint16_t)(sign | (base + q));
+}
+
+/* ------------------------------------------------------------------------- */
+/* Token addressing shared by every stage.  KC:97-100 (store), KC:365-368     */
+/* (decode), flash_fwd_kernel.h:621-632 (prefill: table entries are token      */
+/* offsets, multiplied by the token stride).                                   */
+/* ------------------------------------------------------------------------- */
+
+static inline int64_t cache_token_index(const int64_t* cachestarts, int64_t cachestarts_stride_b,
+                                        int64_t batch_id, int64_t pos, int32_t page_size)
+{
+    if (page_size <= 0)
+        return cachestarts[batch_id] + pos;
+    return cachestarts[batch_id * cachestarts_stride_b + pos / page_size] + pos % page_size;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Quantise/append.  KC:86-157 (kernel), KC:2013-2057 (launch).                */
+/*   absmax in half (KC:133-137), scale = half(float(absmax)/127) (KC:139),    */
+/*   clamp to eps = half(1e-5f) (KC:129,141-142), q = rint_even(half(x/scale)) */
+/*   (KC:146), 8 channels per group, scale index = element index / 8           */
+/*   (KC:125-126).  The half division is the correctly rounded quotient.       */
+/* ------------------------------------------------------------------------- */
+
+void pmx_oracle_quantize_group8(const uint16_t* x, int8_t* q, uint16_t* scale_out)
+{
+    const uint16_t eps_bits = pmx_oracle_float_to_half(1e-5f); /* 0x00A8 */
+    const float eps = pmx_oracle_half_to_float(eps_bits);
+    float amax = 0.0f;
+    for (int i = 0; i < 8; ++i) {
+        const float a = fabsf(pmx_oracle_half_to_float(x[i]));
+        amax = amax > a ? amax : a; /* same select form as KC:135 */
+    }
+    uint16_t s_bits = pmx_oracle_float_to_half(amax / 127.0f);
+    float s = pmx_oracle_half_to_float(s_bits);
+    if (!(s > eps)) {
+        s = eps;
+        s_bits = eps_bits;
+    }
+    for (int i = 0; i < 8; ++i) {
+        /* half / half: exact quotient rounded once to binary16.  Going through a
+         * correctly rounded binary32 quotient is equivalent (24 >= 2*11+2). */
+        const float quo = pmx_oracle_half_to_float(x[i]) / s;
+        const float quo_h = pmx_oracle_half_to_float(pmx_oracle_float_to_half(quo));
+        q[i] = (int8_t)(int)nearbyintf(quo_h); /* default mode: ties to even */
+    }
+    *scale_out = s_bits;
+}
+
+int pmx_oracle_kv_cache_quantize(
+    const uint16_t* current_key, const uint16_t* current_value,
+    const int64_t* seqstarts, const int64_t* cachestarts, const int64_t* start_pos,
+    int64_t batch, int64_t layer_idx, int64_t num_kv_heads, int64_t head_dim,
+    int32_t page_size, /* 0 = contiguous (cache_mode 0), 128 = paged (cache_mode 1) */
+    int64_t current_key_stride_s, int64_t current_value_stride_s,
+    int64_t cache_stride_s, int64_t cache_stride_l, int64_t cache_stride_h, int64_t cache_stride_kv,
+    int64_t cachestarts_stride_b,
+    int8_t* cache, uint16_t* scale)
+{
+    if (head_dim % 8 != 0)
+        return 2;
+    for (int64_t b = 0; b < batch; ++b) {
+        const int64_t seqlen = seqstarts[b + 1] - seqstarts[b];
+#pragma omp parallel for schedule(static)
+        for (int64_t i = 0; i < seqlen; ++i) {
+            const int64_t tok = cache_token_index(cachestarts, cachestarts_stride_b, b, start_pos[b] + i, page_size);
+            const int64_t in_tok = seqstarts[b] + i;
+            for (int64_t h = 0; h < num_kv_heads; ++h) {
+                for (int64_t d0 = 0; d0 < head_dim; d0 += 8) {
+                    const int64_t in_idx = h * head_dim + d0;
+                    const int64_t k_out = tok * cache_stride_s + layer_idx * cache_stride_l + h * cache_stride_h + d0;
+                    const int64_t v_out = k_out + cache_stride_kv;
+                    pmx_oracle_quantize_group8(current_key + in_tok * current_key_stride_s + in_idx,
+                                               cache + k_out, scale + k_out / 8);
+                    pmx_oracle_quantize_group8(current_value + in_tok * current_value_stride_s + in_idx,
+                                               cache + v_out, scale + v_out / 8);
+                }
+            }
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Attention over the dequantised cache.                                       */
+/*   dequant: float(int8) * float(scale) -- exact in binary32.  (KC:404,509    */
+/*   round this product to half; the contract here is the unrounded product.)  */
+/*   logit = attn_scale * dot(q, k^) (+ mask)  KC:410-415                      */
+/*   kv head = q head / num_kv_repeats          KC:299                          */
+/*   kv length = kvstarts[b+1]-kvstarts[b]      KC:347                          */
+/*   softmax and PV accumulate in double; result written as binary32.          */
+/* ------------------------------------------------------------------------- */
+
+static void attend_one_row(
+    const uint16_t* q_row, /* head_dim halves */
+    const uint16_t* mask_row, /* may be NULL; indexed by kv position */
+    const int8_t* cache, const uint16_t* scale,
+    const int64_t* cachestarts, int64_t cachestarts_stride_b, int64_t b, int32_t page_size,
+    int64_t kv_begin, int64_t kv_end, /* positions attended: [kv_begin, kv_end) */
+    int64_t head_base, /* layer_idx*stride_l + kvh*stride_h */
+    int64_t cache_stride_s, int64_t cache_stride_kv, int64_t head_dim, float attn_scale,
+    double* logits, /* scratch, >= kv_end-kv_begin */
+    float* out, /* head_dim floats */
+    float* out_max, float* out_sum) /* optional: running max and exp-sum (for split tests) */
+{
+    float qf[256];
+    for (int64_t d = 0; d < head_dim; ++d)
+        qf[d] = pmx_oracle_half_to_float(q_row[d]);
+    const int64_t n = kv_end - kv_begin;
+    double mx = -INFINITY;
+    for (int64_t t = 0; t < n; ++t) {
+        const int64_t tok = cache_token_index(cachestarts, cachestarts_stride_b, b, kv_begin + t, page_size);
+        const int64_t k_off = tok * cache_stride_s + head_base;
+        double acc = 0.0;
+        for (int64_t d0 = 0; d0 < head_dim; d0 += 8) {
+            const float s = pmx_oracle_half_to_float(scale[(k_off + d0) >> 3]);
+            for (int64_t d = d0; d < d0 + 8; ++d)
+                acc += (double)qf[d] * (double)((float)cache[k_off + d] * s);
+        }
+        double l = (double)attn_scale * acc;
+        if (mask_row)
+            l += (double)pmx_oracle_half_to_float(mask_row[kv_begin + t]);
+        logits[t] = l;
+        if (l > mx)
+            mx = l;
+    }
+    double o[256];
+    for (int64_t d = 0; d < head_dim; ++d)
+        o[d] = 0.0;
+    double sum = 0.0;
+    for (int64_t t = 0; t < n; ++t) {
+        const double p = (mx == -INFINITY) ? 0.0 : exp(logits[t] - mx);
+        sum += p;
+        const int64_t tok = cache_token_index(cachestarts, cachestarts_stride_b, b, kv_begin + t, page_size);
+        const int64_t v_off = tok * cache_stride_s + head_base + cache_stride_kv;
+        for (int64_t d0 = 0; d0 < head_dim; d0 += 8) {
+            const float s = pmx_oracle_half_to_float(scale[(v_off + d0) >> 3]);
+            for (int64_t d = d0; d < d0 + 8; ++d)
+                o[d] += p * (double)((float)cache[v_off + d] * s);
+        }
+    }
+    const double inv = sum > 0.0 ? 1.0 / sum : 0.0;
+    for (int64_t d = 0; d < head_dim; ++d)
+        out[d] = (float)(o[d] * inv);
+    if (out_max)
+        *out_max = (float)mx;
+    if (out_sum)
+        *out_sum = (float)sum;
+}
+
+/* Decode: sequences [0, decoding_batches), one query row each, row index = batch
+ * index (KC:333), output row likewise (KC:589).  Mask row for sequence b starts at
+ * attn_mask + h*mask_stride_h + b*mask_stride_s + kvstarts[b] (KC:320-324). */
+int pmx_oracle_decode_attention(
+    const uint16_t* query, const uint16_t* attn_mask, /* mask may be NULL */
+    const int8_t* cache, const uint16_t* scale,
+    const int64_t* cachestarts, const int64_t* kvstarts,
+    int64_t decoding_batches, int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+    float attn_scale, int64_t layer_idx, int32_t page_size,
+    int64_t query_stride_s, int64_t output_stride_s, int64_t mask_stride_s, int64_t mask_stride_h,
+    int64_t cache_stride_s, int64_t cache_stride_l, int64_t cache_stride_h, int64_t cache_stride_kv,
+    int64_t cachestarts_stride_b,
+    float* output) /* [decoding_batches, output_stride_s] binary32 */
+{
+    if (num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || head_dim % 8 != 0 || head_dim > 256)
+        return 2;
+    const int64_t repeats = num_heads / num_kv_heads;
+    int64_t max_len = 0;
+    for (int64_t b = 0; b < decoding_batches; ++b) {
+        const int64_t l = kvstarts[b + 1] - kvstarts[b];
+        if (l > max_len)
+            max_len = l;
+    }
+    const int64_t work = decoding_batches * num_heads;
+#pragma omp parallel
+    {
+        double* logits = (double*)malloc(sizeof(double) * (size_t)(max_len > 0 ? max_len : 1));
+#pragma omp for schedule(dynamic, 1)
+        for (int64_t w = 0; w < work; ++w) {
+            const int64_t b = w / num_heads, h = w % num_heads;
+            const int64_t kvh = h / repeats;
+            const int64_t len = kvstarts[b + 1] - kvstarts[b];
+            const uint16_t* mrow = attn_mask ? attn_mask + h * mask_stride_h + b * mask_stride_s + kvstarts[b] : NULL;
+            attend_one_row(query + b * query_stride_s + h * head_dim, mrow, cache, scale,
+                           cachestarts, cachestarts_stride_b, b, page_size, 0, len,
+                           layer_idx * cache_stride_l + kvh * cache_stride_h,
+                           cache_stride_s, cache_stride_kv, head_dim, attn_scale, logits,
+                           output + b * output_stride_s + h * head_dim, NULL, NULL);
+        }
+        free(logits);
+    }
+    return 0;
+}
+
+/* Prefill over the int8 cache: sequences [decoding_batches, batch).  Query rows
+ * seqstarts[b]..seqstarts[b+1] (KC:2131), kv length from kvstarts (KC:2132),
+ * cache rows through cachestarts (KC:2142).  Causal mask is bottom-right aligned:
+ * row i sees columns < i + 1 + kvlen - qlen (flash_attn2/src/mask.h:186). */
+int pmx_oracle_prefill_attention(
+    const uint16_t* query,
+    const int8_t* cache, const uint16_t* scale,
+    const int64_t* seqstarts, const int64_t* kvstarts, const int64_t* cachestarts,
+    int64_t batch, int64_t decoding_batches, int32_t is_causal,
+    int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+    float attn_scale, int64_t layer_idx, int32_t page_size,
+    int64_t query_stride_s, int64_t output_stride_s,
+    int64_t cache_stride_s, int64_t cache_stride_l, int64_t cache_stride_h, int64_t cache_stride_kv,
+    int64_t cachestarts_stride_b,
+    float* output) /* indexed by absolute query row like the query */
+{
+    if (num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || head_dim % 8 != 0 || head_dim > 256)
+        return 2;
+    const int64_t repeats = num_heads / num_kv_heads;
+    for (int64_t b = decoding_batches; b < batch; ++b) {
+        const int64_t qlen = seqstarts[b + 1] - seqstarts[b];
+        const int64_t kvlen = kvstarts[b + 1] - kvstarts[b];
+        const int64_t work = qlen * num_heads;
+#pragma omp parallel
+        {
+            double* logits = (double*)malloc(sizeof(double) * (size_t)(kvlen > 0 ? kvlen : 1));
+#pragma omp for schedule(dynamic, 8)
+            for (int64_t w = 0; w < work; ++w) {
+                const int64_t i = w / num_heads, h = w % num_heads;
+                const int64_t kvh = h / repeats;
+                int64_t limit = kvlen;
+                if (is_causal) {
+                    limit = i + 1 + kvlen - qlen;
+                    if (limit > kvlen)
+                        limit = kvlen;
+                    if (limit < 0)
+                        limit = 0;
+                }
+                const int64_t row = seqstarts[b] + i;
+                attend_one_row(query + row * query_stride_s + h * head_dim, NULL, cache, scale,
+                               cachestarts, cachestarts_stride_b, b, page_size, 0, limit,
+                               layer_idx * cache_stride_l + kvh * cache_stride_h,
+                               cache_stride_s, cache_stride_kv, head_dim, attn_scale, logits,
+                               output + row * output_stride_s + h * head_dim, NULL, NULL);
+            }
+            free(logits);
+        }
+    }
+    return 0;
+}
+
+/* One piece of one sequence: attention over kv positions [kv_begin, kv_end) of
+ * sequence b for query head h, returning the normalised partial output plus the
+ * piece's running max and exp-sum.  Used to check split-KV partials. */
+int pmx_oracle_decode_partial(
+    const uint16_t* query, const int8_t* cache, const uint16_t* scale,
+    const int64_t* cachestarts,
+    int64_t b, int64_t h, int64_t kv_begin, int64_t kv_end,
+    int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+    float attn_scale, int64_t layer_idx, int32_t page_size,
+    int64_t query_stride_s,
+    int64_t cache_stride_s, int64_t cache_stride_l, int64_t cache_stride_h, int64_t cache_stride_kv,
+    int64_t cachestarts_stride_b,
+    float* out, float* out_max, float* out_sum)
+{
+    const int64_t repeats = num_heads / num_kv_heads;
+    const int64_t n = kv_end - kv_begin;
+    double* logits = (double*)malloc(sizeof(double) * (size_t)(n > 0 ? n : 1));
+    attend_one_row(query + b * query_stride_s + h * head_dim, NULL, cache, scale,
+                   cachestarts, cachestarts_stride_b, b, page_size, kv_begin, kv_end,
+                   layer_idx * cache_stride_l + (h / repeats) * cache_stride_h,
+                   cache_stride_s, cache_stride_kv, head_dim, attn_scale, logits,
+                   out, out_max, out_sum);
+    free(logits);
+    return 0;
+}
+
+/* Split-KV combine.  KC:617-665: weights exp(lse_i - max lse) / sum, with
+ * lse_i = m_i + log(l_i) (KC:450).  Here each piece carries (m_i, l_i) and a
+ * normalised partial o_i; an empty piece has l_i = 0 and contributes nothing. */
+int pmx_oracle_splitkv_combine(
+    const float* partial_out, /* [n_pieces, head_dim] */
+    const float* partial_max, const float* partial_sum, /* [n_pieces] */
+    int64_t n_pieces, int64_t head_dim,
+    float* out) /* [head_dim] */
+{
+    double mx = -INFINITY;
+    for (int64_t i = 0; i < n_pieces; ++i)
+        if (partial_sum[i] > 0.0f && (double)partial_max[i] > mx)
+            mx = (double)partial_max[i];
+    double den = 0.0;
+    double o[256];
+    for (int64_t d = 0; d < head_dim; ++d)
+        o[d] = 0.0;
+    for (int64_t i = 0; i < n_pieces; ++i) {
+        if (!(partial_sum[i] > 0.0f))
+            continue;
+        const double w = (double)partial_sum[i] * exp((double)partial_max[i] - mx);
+        den += w;
+        for (int64_t d = 0; d < head_dim; ++d)
+            o[d] += w * (double)partial_out[i * head_dim + d];
+    }
+    for (int64_t d = 0; d < head_dim; ++d)
+        out[d] = den > 0.0 ? (float)(o[d] / den) : 0.0f;
+    return 0;
+}
+
+/* Host threads the OpenMP loops above will use (reported beside CPU timings). */
+int pmx_oracle_num_threads(void)
+{
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}

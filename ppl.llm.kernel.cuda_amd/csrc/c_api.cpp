@@ -1,0 +1,316 @@
+// Host side of the C ABI: argument checks, the split plan, and kernel launches.
+// No allocation, no synchronisation; errors are reported by return code plus a
+// thread-local message (pmxhip_last_error).
+#include "pmx_hip/c_api.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "launch_params.h"
+
+namespace {
+
+thread_local char g_last_error[512] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+    fprintf(stderr, "[pmx_hip] error: %s\n", g_last_error);
+    return code;
+}
+
+bool head_dim_supported(int64_t d) { return d == 64 || d == 96 || d == 128 || d == 256; }
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_cache_layout(const char* who, int32_t cache_mode, int64_t page_size, int64_t s, int64_t l, int64_t h,
+                       int64_t kv, int64_t multiple)
+{
+    if (cache_mode != 0 && cache_mode != 1) return fail(PMXHIP_UNSUPPORTED, "%s: invalid cache_mode %d", who, cache_mode);
+    if (cache_mode == 1 && page_size != PMXHIP_PAGE_SIZE)
+        return fail(PMXHIP_UNSUPPORTED, "%s: cache_mode 1 needs page_size == %d, got %lld", who, PMXHIP_PAGE_SIZE,
+                    (long long)page_size);
+    if (s % multiple || l % multiple || h % multiple || kv % multiple)
+        return fail(PMXHIP_UNSUPPORTED, "%s: cache strides must be multiples of %lld (s=%lld l=%lld h=%lld kv=%lld)", who,
+                    (long long)multiple, (long long)s, (long long)l, (long long)h, (long long)kv);
+    return PMXHIP_SUCCESS;
+}
+
+int launch_status(const char* who)
+{
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(PMXHIP_OTHER_ERROR, "%s: launch failed: %s", who, hipGetErrorString(e));
+    return PMXHIP_SUCCESS;
+}
+
+int largest_pow2_divisor_upto(int64_t n, int cap)
+{
+    int r = 1;
+    while (r * 2 <= cap && n % (r * 2) == 0) r *= 2;
+    return r;
+}
+
+} // namespace
+
+extern "C" {
+
+const char* pmxhip_version(void) { return "pmx_hip 0.1 (gfx950)"; }
+
+const char* pmxhip_last_error(void) { return g_last_error; }
+
+int pmxhip_kv_cache_quantize(const pmxhip_kvstore_params* p, pmxhip_stream_t stream)
+{
+    if (!p) return fail(PMXHIP_INVALID_VALUE, "kv_cache_quantize: null params");
+    if (p->head_dim <= 0 || p->head_dim % 8 != 0) // kernel.cu:2040-2043
+        return fail(PMXHIP_UNSUPPORTED, "kv_cache_quantize: head_dim must be aligned with 8, currently get %lld",
+                    (long long)p->head_dim);
+    if (int rc = check_cache_layout("kv_cache_quantize", p->cache_mode, p->page_size, p->cache_stride_s, p->cache_stride_l,
+                                    p->cache_stride_h, p->cache_stride_kv, 8))
+        return rc;
+    if (p->batch < 0 || p->max_seqlen < 0 || p->num_kv_heads <= 0)
+        return fail(PMXHIP_INVALID_VALUE, "kv_cache_quantize: bad batch/max_seqlen/num_kv_heads");
+    if (p->batch == 0 || p->max_seqlen == 0) return PMXHIP_SUCCESS;
+    if (!p->current_key || !p->current_value || !p->seqstarts || !p->cachestarts || !p->start_pos || !p->cache || !p->scale)
+        return fail(PMXHIP_INVALID_VALUE, "kv_cache_quantize: null device pointer");
+    if (p->current_key_stride_s % 8 || p->current_value_stride_s % 8 || !aligned16(p->current_key) ||
+        !aligned16(p->current_value) || (reinterpret_cast<uintptr_t>(p->cache) & 7u))
+        return fail(PMXHIP_UNSUPPORTED, "kv_cache_quantize: current_key/value need 16-byte aligned rows, cache 8-byte alignment");
+
+    pmxhip::QuantLaunch a{};
+    a.current_key = p->current_key;
+    a.current_value = p->current_value;
+    a.seqstarts = p->seqstarts;
+    a.cachestarts = p->cachestarts;
+    a.start_pos = p->start_pos;
+    a.cache = static_cast<int8_t*>(p->cache);
+    a.scale = p->scale;
+    a.batch = p->batch;
+    a.layer_idx = p->layer_idx;
+    a.num_kv_heads = (int32_t)p->num_kv_heads;
+    a.head_dim = (int32_t)p->head_dim;
+    a.current_key_stride_s = p->current_key_stride_s;
+    a.current_value_stride_s = p->current_value_stride_s;
+    a.cache_stride_s = p->cache_stride_s;
+    a.cache_stride_l = p->cache_stride_l;
+    a.cache_stride_h = p->cache_stride_h;
+    a.cache_stride_kv = p->cache_stride_kv;
+    a.cachestarts_stride_b = p->cachestarts_stride_b;
+    a.max_tokens = p->batch * p->max_seqlen;
+    a.cache_mode = p->cache_mode;
+    pmxhip::launch_kv_quantize(a, stream);
+    return launch_status("kv_cache_quantize");
+}
+
+int pmxhip_key_value_cache(pmxhip_stream_t stream, const void* current_key, const void* current_value,
+                           const int64_t* seqstarts, const int64_t* cachestarts, const int64_t* start_pos, int64_t batch,
+                           int64_t max_seqlen, int64_t num_layer, int64_t layer_idx, int64_t num_kv_heads,
+                           int64_t head_dim, int32_t cache_mode, int64_t page_size, int64_t cache_stride_s,
+                           int64_t cache_stride_l, int64_t cache_stride_h, int64_t cache_stride_kv,
+                           int64_t cachestarts_stride_b, void* cache, void* scale)
+{
+    pmxhip_kvstore_params p;
+    memset(&p, 0, sizeof(p));
+    p.current_key = current_key;
+    p.current_value = current_value;
+    p.seqstarts = seqstarts;
+    p.cachestarts = cachestarts;
+    p.start_pos = start_pos;
+    p.num_layer = num_layer;
+    p.layer_idx = layer_idx;
+    p.num_kv_heads = num_kv_heads;
+    p.head_dim = head_dim;
+    p.page_size = (int32_t)page_size;
+    p.current_key_stride_s = num_kv_heads * head_dim;
+    p.current_value_stride_s = num_kv_heads * head_dim;
+    p.cache_stride_s = cache_stride_s;
+    p.cache_stride_l = cache_stride_l;
+    p.cache_stride_h = cache_stride_h;
+    p.cache_stride_kv = cache_stride_kv;
+    p.cachestarts_stride_b = cachestarts_stride_b;
+    p.cache = cache;
+    p.scale = scale;
+    p.batch = batch;
+    p.max_seqlen = max_seqlen;
+    p.cache_mode = cache_mode;
+    return pmxhip_kv_cache_quantize(&p, stream);
+}
+
+int pmxhip_decode_plan_make(int64_t decoding_batches, int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                            int64_t max_kvlen, int32_t compute_units, int32_t num_token_ranges_hint,
+                            pmxhip_decode_plan* plan)
+{
+    if (!plan) return fail(PMXHIP_INVALID_VALUE, "decode_plan: null plan");
+    memset(plan, 0, sizeof(*plan));
+    if (!head_dim_supported(head_dim))
+        return fail(PMXHIP_UNSUPPORTED, "cache flash decoding attention do not support head dim %lld", (long long)head_dim);
+    if (num_kv_heads <= 0 || num_heads <= 0 || num_heads % num_kv_heads != 0)
+        return fail(PMXHIP_UNSUPPORTED, "only support num_heads %% num_kv_heads == 0.");
+    if (num_token_ranges_hint < 0) return fail(PMXHIP_INVALID_VALUE, "decode_plan: negative range hint");
+    const int64_t repeats = num_heads / num_kv_heads;
+    const int lanes_per_slot = head_dim == 64 ? 4 : (head_dim == 256 ? 16 : 8);
+    const int slots_per_wave = 64 / lanes_per_slot;
+    const int kvhb = largest_pow2_divisor_upto(num_kv_heads, slots_per_wave < 8 ? slots_per_wave : 8);
+    int gt = 1;
+    while (gt < repeats && gt < 8) gt *= 2;
+    const int passes = (int)((repeats + gt - 1) / gt);
+    const int wg_tokens = pmxhip::decode_wg_tokens((int)head_dim, kvhb);
+    const int min_tokens = wg_tokens > 128 ? wg_tokens : 128;
+
+    int64_t ranges = num_token_ranges_hint;
+    if (ranges == 0) {
+        const int64_t groups = (num_kv_heads / kvhb) * passes;
+        const int cus = compute_units > 0 ? compute_units : 256;
+        ranges = ((int64_t)cus * 2 + groups - 1) / groups;
+        const int64_t max_tokens = decoding_batches * (max_kvlen > 0 ? max_kvlen : 1);
+        const int64_t useful = (max_tokens + min_tokens - 1) / min_tokens;
+        if (ranges > useful) ranges = useful;
+        if (ranges < 1) ranges = 1;
+    }
+    plan->num_token_ranges = (int32_t)ranges;
+    plan->kv_heads_per_group = kvhb;
+    plan->q_heads_per_pass = gt;
+    plan->num_passes = passes;
+    if (ranges > 1) {
+        const int64_t pieces = ranges + decoding_batches;
+        plan->partial_out_size = pieces * num_heads * head_dim * (int64_t)sizeof(float);
+        plan->partial_ml_size = pieces * num_heads * 2 * (int64_t)sizeof(float);
+    }
+    plan->workspace_size = plan->partial_out_size + plan->partial_ml_size;
+    return PMXHIP_SUCCESS;
+}
+
+int pmxhip_decode_attention(const pmxhip_decode_params* p, pmxhip_stream_t stream)
+{
+    if (!p) return fail(PMXHIP_INVALID_VALUE, "decode_attention: null params");
+    if (p->decoding_batches < 0) return fail(PMXHIP_INVALID_VALUE, "decode_attention: negative decoding_batches");
+    if (p->decoding_batches == 0) return PMXHIP_SUCCESS; // kernel.cu:2084
+    if (!head_dim_supported(p->head_dim))
+        return fail(PMXHIP_UNSUPPORTED, "cache flash decoding attention do not support head dim %lld", (long long)p->head_dim);
+    if (p->num_kv_heads <= 0 || p->num_heads % p->num_kv_heads != 0 || p->num_kv_repeats != p->num_heads / p->num_kv_heads)
+        return fail(PMXHIP_UNSUPPORTED, "only support num_heads %% num_kv_heads == 0.");
+    if (int rc = check_cache_layout("decode_attention", p->cache_mode, p->page_size, p->cache_stride_s, p->cache_stride_l,
+                                    p->cache_stride_h, p->cache_stride_kv, 16))
+        return rc;
+    if (!p->query || !p->output || !p->cache || !p->scale || !p->cachestarts || !p->kvstarts)
+        return fail(PMXHIP_INVALID_VALUE, "decode_attention: null device pointer");
+    if (!aligned16(p->query) || !aligned16(p->cache) || (reinterpret_cast<uintptr_t>(p->scale) & 3u) ||
+        p->query_stride_s % 8 != 0)
+        return fail(PMXHIP_UNSUPPORTED, "decode_attention: query/cache must be 16-byte aligned, scale 4-byte aligned");
+    if (p->attn_mask && p->mask_stride_s % 8 != 0) // utils.cu:127-130
+        return fail(PMXHIP_UNSUPPORTED, "last dimension of attn_mask must be aligned with 8");
+
+    pmxhip_decode_plan plan;
+    if (p->num_token_ranges <= 0) return fail(PMXHIP_INVALID_VALUE, "decode_attention: num_token_ranges must be >= 1");
+    if (int rc = pmxhip_decode_plan_make(p->decoding_batches, p->num_heads, p->num_kv_heads, p->head_dim, 0, 0,
+                                         p->num_token_ranges, &plan))
+        return rc;
+    if (plan.workspace_size > 0) {
+        if (!p->workspace || p->workspace_size < plan.workspace_size)
+            return fail(PMXHIP_INVALID_VALUE, "decode_attention: workspace too small (%lld < %lld)",
+                        (long long)p->workspace_size, (long long)plan.workspace_size);
+        if (!aligned16(p->workspace)) return fail(PMXHIP_INVALID_VALUE, "decode_attention: workspace must be 16-byte aligned");
+    }
+
+    pmxhip::DecodeLaunch a{};
+    a.query = p->query;
+    a.attn_mask = p->attn_mask;
+    a.output = p->output;
+    a.cache = p->cache;
+    a.scale = p->scale;
+    a.cachestarts = p->cachestarts;
+    a.kvstarts = p->kvstarts;
+    a.partial_out = static_cast<float*>(p->workspace);
+    a.partial_ml = reinterpret_cast<float*>(static_cast<char*>(p->workspace) + plan.partial_out_size);
+    a.attn_scale = p->attn_scale;
+    a.cache_mode = p->cache_mode;
+    a.layer_idx = p->layer_idx;
+    a.num_kv_repeats = p->num_kv_repeats;
+    a.query_stride_s = p->query_stride_s;
+    a.output_stride_s = p->output_stride_s;
+    a.mask_stride_s = p->mask_stride_s;
+    a.mask_stride_h = p->mask_stride_h;
+    a.cache_stride_s = p->cache_stride_s;
+    a.cache_stride_l = p->cache_stride_l;
+    a.cache_stride_h = p->cache_stride_h;
+    a.cache_stride_kv = p->cache_stride_kv;
+    a.cachestarts_stride_b = p->cachestarts_stride_b;
+    a.decoding_batches = p->decoding_batches;
+    a.num_heads = p->num_heads;
+    a.num_kv_heads = p->num_kv_heads;
+    a.head_dim = (int32_t)p->head_dim;
+    a.ranges = plan.num_token_ranges;
+    a.kv_heads_per_group = plan.kv_heads_per_group;
+    a.q_heads_per_pass = plan.q_heads_per_pass;
+    a.num_passes = plan.num_passes;
+    a.wg_tokens = pmxhip::decode_wg_tokens((int)p->head_dim, plan.kv_heads_per_group);
+    a.min_tokens_per_range = a.wg_tokens > 128 ? a.wg_tokens : 128;
+    if (pmxhip::launch_decode(a, stream) != 0) return fail(PMXHIP_UNSUPPORTED, "decode_attention: no kernel for this shape");
+    return launch_status("decode_attention");
+}
+
+int pmxhip_splitkv_combine(const float* partial_out, const float* partial_ml, const int64_t* piece_begin,
+                           const int64_t* piece_end, int64_t rows, int64_t head_dim, void* output,
+                           pmxhip_stream_t stream)
+{
+    if (rows < 0 || head_dim <= 0) return fail(PMXHIP_INVALID_VALUE, "splitkv_combine: bad rows/head_dim");
+    if (rows == 0) return PMXHIP_SUCCESS;
+    if (!partial_out || !partial_ml || !piece_begin || !piece_end || !output)
+        return fail(PMXHIP_INVALID_VALUE, "splitkv_combine: null device pointer");
+    pmxhip::launch_splitkv_combine_rows(partial_out, partial_ml, piece_begin, piece_end, rows, head_dim, output, stream);
+    return launch_status("splitkv_combine");
+}
+
+int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t stream)
+{
+    if (!p) return fail(PMXHIP_INVALID_VALUE, "prefill_attention: null params");
+    const int64_t prefill_batches = p->batch - p->decoding_batches;
+    if (prefill_batches < 0 || p->decoding_batches < 0)
+        return fail(PMXHIP_INVALID_VALUE, "prefill_attention: decoding_batches out of range");
+    if (prefill_batches == 0 || p->max_seqlen == 0) return PMXHIP_SUCCESS; // kernel.cu:2130, 2214-2216
+    if (p->head_dim != 64 && p->head_dim != 128)
+        return fail(PMXHIP_UNSUPPORTED, "prefill_attention: head dim %lld not supported (64, 128)", (long long)p->head_dim);
+    if (p->num_kv_heads <= 0 || p->num_heads % p->num_kv_heads != 0)
+        return fail(PMXHIP_UNSUPPORTED, "only support num_heads %% num_kv_heads == 0.");
+    if (int rc = check_cache_layout("prefill_attention", p->cache_mode, p->page_size, p->cache_stride_s, p->cache_stride_l,
+                                    p->cache_stride_h, p->cache_stride_kv, 8))
+        return rc;
+    if (!p->query || !p->output || !p->cache || !p->scale || !p->seqstarts || !p->kvstarts || !p->cachestarts)
+        return fail(PMXHIP_INVALID_VALUE, "prefill_attention: null device pointer");
+    if (!aligned16(p->query) || p->query_stride_s % 8 != 0 || (reinterpret_cast<uintptr_t>(p->cache) & 7u))
+        return fail(PMXHIP_UNSUPPORTED, "prefill_attention: query must be 16-byte aligned, cache 8-byte aligned");
+
+    pmxhip::PrefillLaunch a{};
+    a.query = p->query;
+    a.output = p->output;
+    a.cache = p->cache;
+    a.scale = p->scale;
+    a.seqstarts = p->seqstarts + p->decoding_batches;                          // kernel.cu:2131
+    a.kvstarts = p->kvstarts + p->decoding_batches;                            // kernel.cu:2132
+    a.cachestarts = p->cachestarts + p->decoding_batches * p->cachestarts_stride_b; // kernel.cu:2142
+    a.attn_scale = p->attn_scale;
+    a.is_causal = p->is_causal;
+    a.cache_mode = p->cache_mode;
+    a.prefill_batches = prefill_batches;
+    a.max_seqlen = p->max_seqlen;
+    a.layer_idx = p->layer_idx;
+    a.num_heads = p->num_heads;
+    a.num_kv_heads = p->num_kv_heads;
+    a.head_dim = (int32_t)p->head_dim;
+    a.query_stride_s = p->query_stride_s;
+    a.output_stride_s = p->output_stride_s;
+    a.cache_stride_s = p->cache_stride_s;
+    a.cache_stride_l = p->cache_stride_l;
+    a.cache_stride_h = p->cache_stride_h;
+    a.cache_stride_kv = p->cache_stride_kv;
+    a.cachestarts_stride_b = p->cachestarts_stride_b;
+    if (pmxhip::launch_prefill(a, stream) != 0) return fail(PMXHIP_UNSUPPORTED, "prefill_attention: no kernel for this shape");
+    return launch_status("prefill_attention");
+}
+
+} // extern "C"

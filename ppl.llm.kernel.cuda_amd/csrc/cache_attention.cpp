@@ -1,0 +1,489 @@
+// The pmx operator class over the C ABI, the key_value_cache free function, and
+// the C handle that lets a non-C++ host drive the class.
+//
+// heuristic_prepare keeps the reference's checks and derived values
+// (src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/utils.cu:68-131,
+// 162-165, 210-214, 318-324) and replaces its launch heuristics (utils.cu:136-264)
+// with the token-range plan of this implementation.
+#include "pmx_hip/cache_attention.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "pmx_hip/c_api.h"
+#include "pmx_hip/key_value_cache.h"
+
+namespace ppl { namespace kernel { namespace llm { namespace cuda { namespace pmx {
+
+namespace {
+
+constexpr int32_t UNIFORM_PAGE_SIZE = PMXHIP_PAGE_SIZE;
+
+#define PMX_LOG_ERROR(...)                         \
+    do {                                           \
+        fprintf(stderr, "[pmx_hip] error: ");      \
+        fprintf(stderr, __VA_ARGS__);              \
+        fprintf(stderr, "\n");                     \
+    } while (0)
+
+ppl::common::RetCode to_retcode(int status)
+{
+    switch (status) {
+        case PMXHIP_SUCCESS: return ppl::common::RC_SUCCESS;
+        case PMXHIP_UNSUPPORTED: return ppl::common::RC_UNSUPPORTED;
+        case PMXHIP_INVALID_VALUE: return ppl::common::RC_INVALID_VALUE;
+        default: return ppl::common::RC_OTHER_ERROR;
+    }
+}
+
+} // namespace
+
+ppl::common::RetCode dynamic_batching_multi_head_cache_attention::heuristic_prepare(
+    const hipDeviceProp_t& device_prop,
+    const ppl::common::TensorShape* query_shape, const void* query,
+    const ppl::common::TensorShape* current_key_shape, const void* current_key,
+    const ppl::common::TensorShape* current_value_shape, const void* current_value,
+    const ppl::common::TensorShape* attn_mask_shape, const void* attn_mask,
+    const void* seqstarts, const void* kvstarts,
+    const void* cachestarts, const void* start_pos,
+    const void* alibi_slopes,
+    const bool is_causal,
+    const int64_t batch, const int64_t decoding_batches,
+    const int64_t max_seqlen, const int64_t max_kvlen,
+    const int64_t layer_idx, const int64_t num_layer,
+    const int64_t num_heads, const int64_t num_kv_heads, const int64_t head_dim,
+    const int32_t cache_mode, const int64_t page_size,
+    const int64_t cache_stride_s, const int64_t cache_stride_l,
+    const int64_t cache_stride_h, const int64_t cache_stride_kv,
+    const int64_t cachestarts_stride_b,
+    const bool enable_cache_prefill,
+    const bool enable_sharemem_mhca, const bool enable_infinity_mhca, const bool enable_infinity_gqca,
+    const int32_t specify_decoding_multi_block,
+    const int32_t specify_decoding_tpb,
+    void* cache, void* scale,
+    const ppl::common::TensorShape* output_shape, void* output)
+{
+    // ---- shape checks, in the reference's order (utils.cu:68-95) ----
+    if (query_shape->GetDim(1) != num_heads) {
+        PMX_LOG_ERROR("currently do not support leading dim on query's num_heads");
+        return ppl::common::RC_UNSUPPORTED;
+    }
+    if (output_shape->GetDim(1) != num_heads) {
+        PMX_LOG_ERROR("currently do not support leading dim on output's num_heads");
+        return ppl::common::RC_UNSUPPORTED;
+    }
+    if (current_key_shape->GetDim(1) != num_kv_heads) {
+        PMX_LOG_ERROR("currently do not support leading dim on current_key's num_kv_heads");
+        return ppl::common::RC_UNSUPPORTED;
+    }
+    if (current_value_shape->GetDim(1) != num_kv_heads) {
+        PMX_LOG_ERROR("currently do not support leading dim on current_value's num_kv_heads");
+        return ppl::common::RC_UNSUPPORTED;
+    }
+    if (cache_mode == 1 && page_size != UNIFORM_PAGE_SIZE) {
+        PMX_LOG_ERROR("currently only support page_size == %d", UNIFORM_PAGE_SIZE);
+        return ppl::common::RC_UNSUPPORTED;
+    }
+
+    constexpr int64_t VPT = 8;
+    const int64_t num_kv_repeats = num_kv_heads > 0 ? num_heads / num_kv_heads : 0;
+    if (num_kv_heads <= 0 || num_kv_heads * num_kv_repeats != num_heads) { // utils.cu:101-105
+        PMX_LOG_ERROR("only support num_heads %% num_kv_heads == 0.");
+        return ppl::common::RC_UNSUPPORTED;
+    }
+
+    // ---- derived values (utils.cu:107-131) ----
+    const int64_t prefill_batches = batch - decoding_batches;
+    const float attn_scale = float(1.0 / std::sqrt(float(head_dim)));
+    const int64_t q_stride_s = query_shape->GetDim(1) * head_dim;
+    const int64_t k_stride_s = current_key_shape->GetDim(1) * head_dim;
+    const int64_t v_stride_s = current_value_shape->GetDim(1) * head_dim;
+    const int64_t o_stride_s = output_shape->GetDim(1) * head_dim;
+
+    int64_t mask_stride_s = 0, mask_stride_h = 0;
+    if (attn_mask && attn_mask_shape && attn_mask_shape->CalcElementsExcludingPadding() > 0) {
+        if (attn_mask_shape->GetDimCount() == 3) {
+            mask_stride_h = attn_mask_shape->GetDim(1) * attn_mask_shape->GetDim(2);
+            mask_stride_s = attn_mask_shape->GetDim(2);
+        } else if (attn_mask_shape->GetDimCount() == 2) {
+            mask_stride_s = attn_mask_shape->GetDim(1);
+        } else {
+            PMX_LOG_ERROR("attn_mask must be 2d or 3d");
+            return ppl::common::RC_UNSUPPORTED;
+        }
+        if (mask_stride_s % VPT != 0) {
+            PMX_LOG_ERROR("last dimension of attn_mask must be aligned with %lld", (long long)VPT);
+            return ppl::common::RC_UNSUPPORTED;
+        }
+    }
+
+    // ---- knob checks (utils.cu:162-165, 210-214) ----
+    if (specify_decoding_multi_block < 0 || specify_decoding_multi_block > 2) {
+        PMX_LOG_ERROR("specify_decoding_multi_block only accept 0/1/2");
+        return ppl::common::RC_INVALID_VALUE;
+    }
+    int64_t decoding_threads_per_block = 256;
+    if (specify_decoding_tpb) {
+        if (specify_decoding_tpb != 256 && specify_decoding_tpb != 512) {
+            PMX_LOG_ERROR("only support decoding tpb 256 or 512");
+            return ppl::common::RC_INVALID_VALUE;
+        }
+        decoding_threads_per_block = specify_decoding_tpb; // recorded; the kernels here always run 256 threads
+    }
+
+    // ---- algorithm selection as the reference reports it (utils.cu:193-203, 244-264, 318-331).
+    // Exactly one of the three must come out enabled; which one does not change the kernel here.
+    const bool use_infinity_gqca = enable_infinity_gqca && decoding_batches > 0 &&
+        (num_kv_repeats == 4 || num_kv_repeats == 6 || num_kv_repeats == 8 || num_kv_repeats == 16);
+    bool use_sharemem_mhca = enable_sharemem_mhca && !use_infinity_gqca;
+    bool use_infinity_mhca = false;
+    if (enable_infinity_mhca && !use_infinity_gqca && decoding_batches > 0 && !use_sharemem_mhca) use_infinity_mhca = true;
+    if ((use_infinity_gqca ? 1 : 0) + (use_infinity_mhca ? 1 : 0) + (use_sharemem_mhca ? 1 : 0) != 1) {
+        PMX_LOG_ERROR("No algo to be used or more than one algo is selected, sharemem_mhca=%d, infinity_mhca=%d, infinity_gqca=%d",
+                      (int)use_sharemem_mhca, (int)use_infinity_mhca, (int)use_infinity_gqca);
+        return ppl::common::RC_OTHER_ERROR;
+    }
+
+    // ---- split plan of this implementation ----
+    pmxhip_decode_plan plan;
+    memset(&plan, 0, sizeof(plan));
+    if (decoding_batches > 0) {
+        const int32_t hint = specify_decoding_multi_block == 0 ? 1 : 0;
+        const int rc = pmxhip_decode_plan_make(decoding_batches, num_heads, num_kv_heads, head_dim, max_kvlen,
+                                               device_prop.multiProcessorCount, hint, &plan);
+        // an unsupported head_dim is reported by forward_decode, as in the reference (kernel.cu:1975-2006)
+        if (rc != PMXHIP_SUCCESS) memset(&plan, 0, sizeof(plan));
+    }
+
+    cfg.device_prop = const_cast<hipDeviceProp_t*>(&device_prop);
+    cfg.datatype = query_shape->GetDataType();
+    cfg.query = const_cast<void*>(query);
+    cfg.current_key = const_cast<void*>(current_key);
+    cfg.current_value = const_cast<void*>(current_value);
+    cfg.attn_mask = const_cast<void*>(attn_mask);
+    cfg.seqstarts = const_cast<void*>(seqstarts);
+    cfg.kvstarts = const_cast<void*>(kvstarts);
+    cfg.cachestarts = const_cast<void*>(cachestarts);
+    cfg.start_pos = const_cast<void*>(start_pos);
+    cfg.alibi_slopes = const_cast<void*>(alibi_slopes);
+    cfg.cache = cache;
+    cfg.scale = scale;
+    cfg.output = output;
+    cfg.is_causal = is_causal;
+    cfg.batch = batch;
+    cfg.decoding_batches = decoding_batches;
+    cfg.max_seqlen = max_seqlen;
+    cfg.max_kvlen = max_kvlen;
+    cfg.layer_idx = layer_idx;
+    cfg.num_layer = num_layer;
+    cfg.num_heads = num_heads;
+    cfg.num_kv_heads = num_kv_heads;
+    cfg.head_dim = head_dim;
+    cfg.cache_mode = cache_mode;
+    cfg.page_size = (int32_t)page_size;
+    cfg.cache_stride_s = cache_stride_s;
+    cfg.cache_stride_l = cache_stride_l;
+    cfg.cache_stride_h = cache_stride_h;
+    cfg.cache_stride_kv = cache_stride_kv;
+    cfg.cachestarts_stride_b = cachestarts_stride_b;
+
+    cfg.prefill_batches = prefill_batches;
+    cfg.q_stride_s = q_stride_s;
+    cfg.k_stride_s = k_stride_s;
+    cfg.v_stride_s = v_stride_s;
+    cfg.o_stride_s = o_stride_s;
+    cfg.mask_stride_s = mask_stride_s;
+    cfg.mask_stride_h = mask_stride_h;
+    cfg.attn_scale = attn_scale;
+    cfg.num_kv_repeats = num_kv_repeats;
+    cfg.decoding_algo = use_infinity_gqca ? decoding_algo::INFINITY_GQCA
+                                          : (use_infinity_mhca ? decoding_algo::INFINITY_MHCA : decoding_algo::SHAREMEM_MHCA);
+    cfg.decoding_threads_per_block = decoding_threads_per_block;
+    cfg.decoding_multi_block_size = plan.num_token_ranges > 0 ? plan.num_token_ranges : 1;
+    cfg.decoding_multi_block_partial_out_size = plan.partial_out_size;
+    cfg.decoding_multi_block_partial_log_sum_exp_size = plan.partial_ml_size;
+    cfg.decoding_multi_block_counter_size = 0;
+    cfg.workspace_size = plan.workspace_size;
+    cfg.enable_cache_prefill = enable_cache_prefill;
+    return ppl::common::RC_SUCCESS;
+}
+
+ppl::common::RetCode dynamic_batching_multi_head_cache_attention::forward_kvstore(const hipStream_t stream)
+{
+    pmxhip_kvstore_params p;
+    memset(&p, 0, sizeof(p));
+    p.current_key = cfg.current_key;
+    p.current_value = cfg.current_value;
+    p.seqstarts = static_cast<const int64_t*>(cfg.seqstarts);
+    p.cachestarts = static_cast<const int64_t*>(cfg.cachestarts);
+    p.start_pos = static_cast<const int64_t*>(cfg.start_pos);
+    p.num_layer = cfg.num_layer;
+    p.layer_idx = cfg.layer_idx;
+    p.num_kv_heads = cfg.num_kv_heads;
+    p.head_dim = cfg.head_dim;
+    p.page_size = cfg.page_size;
+    p.current_key_stride_s = cfg.k_stride_s;
+    p.current_value_stride_s = cfg.v_stride_s;
+    p.cache_stride_s = cfg.cache_stride_s;
+    p.cache_stride_l = cfg.cache_stride_l;
+    p.cache_stride_h = cfg.cache_stride_h;
+    p.cache_stride_kv = cfg.cache_stride_kv;
+    p.cachestarts_stride_b = cfg.cachestarts_stride_b;
+    p.cache = cfg.cache;
+    p.scale = cfg.scale;
+    p.batch = cfg.batch;
+    p.max_seqlen = cfg.max_seqlen;
+    p.cache_mode = cfg.cache_mode;
+    return to_retcode(pmxhip_kv_cache_quantize(&p, stream));
+}
+
+ppl::common::RetCode dynamic_batching_multi_head_cache_attention::forward_decode(const hipStream_t stream)
+{
+    if (cfg.decoding_batches <= 0) return ppl::common::RC_SUCCESS;
+    pmxhip_decode_params p;
+    memset(&p, 0, sizeof(p));
+    p.query = cfg.query;
+    p.attn_mask = cfg.attn_mask;
+    p.output = cfg.output;
+    p.cache = cfg.cache;
+    p.scale = cfg.scale;
+    p.cachestarts = static_cast<const int64_t*>(cfg.cachestarts);
+    p.kvstarts = static_cast<const int64_t*>(cfg.kvstarts);
+    p.attn_scale = cfg.attn_scale;
+    p.layer_idx = cfg.layer_idx;
+    p.num_kv_repeats = cfg.num_kv_repeats;
+    p.page_size = cfg.page_size;
+    p.query_stride_s = cfg.q_stride_s;
+    p.output_stride_s = cfg.o_stride_s;
+    p.mask_stride_s = cfg.mask_stride_s;
+    p.mask_stride_h = cfg.mask_stride_h;
+    p.cache_stride_s = cfg.cache_stride_s;
+    p.cache_stride_l = cfg.cache_stride_l;
+    p.cache_stride_h = cfg.cache_stride_h;
+    p.cache_stride_kv = cfg.cache_stride_kv;
+    p.cachestarts_stride_b = cfg.cachestarts_stride_b;
+    p.decoding_batches = cfg.decoding_batches;
+    p.num_heads = cfg.num_heads;
+    p.num_kv_heads = cfg.num_kv_heads;
+    p.head_dim = cfg.head_dim;
+    p.cache_mode = cfg.cache_mode;
+    p.num_token_ranges = (int32_t)cfg.decoding_multi_block_size;
+    p.workspace = cfg.workspace;
+    p.workspace_size = cfg.workspace_size;
+    const int rc = pmxhip_decode_attention(&p, stream);
+    if (rc != PMXHIP_SUCCESS) {
+        // the reference folds every decode dispatch failure into RC_UNSUPPORTED (kernel.cu:2118-2121)
+        PMX_LOG_ERROR("decode stage rejected the configuration");
+        return rc == PMXHIP_INVALID_VALUE ? ppl::common::RC_INVALID_VALUE : ppl::common::RC_UNSUPPORTED;
+    }
+    return ppl::common::RC_SUCCESS;
+}
+
+ppl::common::RetCode dynamic_batching_multi_head_cache_attention::forward_prefill(const hipStream_t stream)
+{
+    if (cfg.prefill_batches <= 0) return ppl::common::RC_SUCCESS;
+    if (cfg.datatype != ppl::common::DATATYPE_FLOAT16) { // flash_attn2/fmha.cu:75
+        PMX_LOG_ERROR("prefill attention only supports fp16");
+        return ppl::common::RC_UNSUPPORTED;
+    }
+    if (!cfg.enable_cache_prefill) {
+        // kernel.cu:2181-2212: attention over the fp16 current_key/value only, no cache read
+        PMX_LOG_ERROR("prefill over fp16 current_key/value (enable_cache_prefill = false) is not built; "
+                      "use enable_cache_prefill = true");
+        return ppl::common::RC_UNSUPPORTED;
+    }
+    if (cfg.attn_mask || cfg.alibi_slopes) {
+        PMX_LOG_ERROR("prefill attention: attn_mask / alibi_slopes are not built on this path");
+        return ppl::common::RC_UNSUPPORTED;
+    }
+    pmxhip_prefill_params p;
+    memset(&p, 0, sizeof(p));
+    p.query = cfg.query;
+    p.output = cfg.output;
+    p.cache = cfg.cache;
+    p.scale = cfg.scale;
+    p.seqstarts = static_cast<const int64_t*>(cfg.seqstarts);
+    p.kvstarts = static_cast<const int64_t*>(cfg.kvstarts);
+    p.cachestarts = static_cast<const int64_t*>(cfg.cachestarts);
+    p.attn_scale = cfg.attn_scale;
+    p.is_causal = cfg.is_causal ? 1 : 0;
+    p.batch = cfg.batch;
+    p.decoding_batches = cfg.decoding_batches;
+    p.max_seqlen = cfg.max_seqlen;
+    p.max_kvlen = cfg.max_kvlen;
+    p.layer_idx = cfg.layer_idx;
+    p.num_heads = cfg.num_heads;
+    p.num_kv_heads = cfg.num_kv_heads;
+    p.head_dim = cfg.head_dim;
+    p.cache_mode = cfg.cache_mode;
+    p.page_size = cfg.page_size;
+    p.query_stride_s = cfg.q_stride_s;
+    p.output_stride_s = cfg.o_stride_s;
+    p.cache_stride_s = cfg.cache_stride_s;
+    p.cache_stride_l = cfg.cache_stride_l;
+    p.cache_stride_h = cfg.cache_stride_h;
+    p.cache_stride_kv = cfg.cache_stride_kv;
+    p.cachestarts_stride_b = cfg.cachestarts_stride_b;
+    return to_retcode(pmxhip_prefill_attention(&p, stream));
+}
+
+ppl::common::RetCode dynamic_batching_multi_head_cache_attention::forward(const hipStream_t stream)
+{
+    // First failure wins (the reference keeps only the last stage's status, kernel.cu:2219-2240).
+    ppl::common::RetCode ret = forward_kvstore(stream);
+    if (ret != ppl::common::RC_SUCCESS) {
+        PMX_LOG_ERROR("kv_store stage failed.");
+        return ret;
+    }
+    ret = forward_decode(stream);
+    if (ret != ppl::common::RC_SUCCESS) {
+        PMX_LOG_ERROR("decode stage failed.");
+        return ret;
+    }
+    ret = forward_prefill(stream);
+    if (ret != ppl::common::RC_SUCCESS) PMX_LOG_ERROR("prefill stage failed.");
+    return ret;
+}
+
+ppl::common::RetCode dynamic_batching_key_value_cache(
+    const hipStream_t stream,
+    const ppl::common::TensorShape* current_key_shape, const void* current_key,
+    const ppl::common::TensorShape* current_value_shape, const void* current_value,
+    const void* seqstarts, const void* cachestarts, const void* start_pos,
+    const int64_t batch, const int64_t max_seqlen,
+    const int64_t num_layer, const int64_t layer_idx,
+    const int64_t num_kv_heads, const int64_t head_dim,
+    const int32_t cache_mode, const int64_t page_size,
+    const int64_t cache_stride_s, const int64_t cache_stride_l,
+    const int64_t cache_stride_h, const int64_t cache_stride_kv,
+    const int64_t cachestarts_stride_b,
+    void* cache, void* scale)
+{
+    if (current_key_shape->GetDim(1) != num_kv_heads || current_value_shape->GetDim(1) != num_kv_heads) {
+        PMX_LOG_ERROR("currently do not support leading dim on current_key/value's num_kv_heads");
+        return ppl::common::RC_UNSUPPORTED;
+    }
+    return to_retcode(pmxhip_key_value_cache(
+        stream, current_key, current_value, static_cast<const int64_t*>(seqstarts),
+        static_cast<const int64_t*>(cachestarts), static_cast<const int64_t*>(start_pos), batch, max_seqlen, num_layer,
+        layer_idx, num_kv_heads, head_dim, cache_mode, page_size, cache_stride_s, cache_stride_l, cache_stride_h,
+        cache_stride_kv, cachestarts_stride_b, cache, scale));
+}
+
+}}}}} // namespace ppl::kernel::llm::cuda::pmx
+
+// ---- C handle over the class ---------------------------------------------------
+
+using mhca_class = ppl::kernel::llm::cuda::pmx::dynamic_batching_multi_head_cache_attention;
+
+struct pmxhip_mhca {
+    mhca_class op;
+    hipDeviceProp_t prop; // heuristic_prepare keeps a pointer to it
+    bool prepared;
+};
+
+namespace {
+
+ppl::common::TensorShape to_shape(const pmxhip_tensor_shape& s)
+{
+    ppl::common::TensorShape t;
+    t.SetDataType((ppl::common::datatype_t)s.data_type);
+    const int n = s.dim_count < 0 ? 0 : (s.dim_count > 4 ? 4 : s.dim_count);
+    t.SetDimCount((uint32_t)n);
+    for (int i = 0; i < n; ++i) t.SetDim((uint32_t)i, s.dims[i]);
+    return t;
+}
+
+} // namespace
+
+extern "C" {
+
+pmxhip_mhca_t pmxhip_mhca_create(void)
+{
+    pmxhip_mhca* h = new (std::nothrow) pmxhip_mhca();
+    if (h) {
+        memset(&h->prop, 0, sizeof(h->prop));
+        h->prepared = false;
+    }
+    return h;
+}
+
+void pmxhip_mhca_destroy(pmxhip_mhca_t op) { delete op; }
+
+int pmxhip_mhca_heuristic_prepare(pmxhip_mhca_t h, const pmxhip_mhca_prepare_args* a)
+{
+    if (!h || !a) return PMXHIP_INVALID_VALUE;
+    h->prop.multiProcessorCount = a->compute_units;
+    h->prop.sharedMemPerBlockOptin = (size_t)a->shared_mem_per_block_optin;
+    const ppl::common::TensorShape qs = to_shape(a->query_shape), ks = to_shape(a->current_key_shape),
+                                   vs = to_shape(a->current_value_shape), ms = to_shape(a->attn_mask_shape),
+                                   os = to_shape(a->output_shape);
+    const ppl::common::RetCode rc = h->op.heuristic_prepare(
+        h->prop, &qs, a->query, &ks, a->current_key, &vs, a->current_value, &ms, a->attn_mask, a->seqstarts, a->kvstarts,
+        a->cachestarts, a->start_pos, a->alibi_slopes, a->is_causal != 0, a->batch, a->decoding_batches, a->max_seqlen,
+        a->max_kvlen, a->layer_idx, a->num_layer, a->num_heads, a->num_kv_heads, a->head_dim, a->cache_mode, a->page_size,
+        a->cache_stride_s, a->cache_stride_l, a->cache_stride_h, a->cache_stride_kv, a->cachestarts_stride_b,
+        a->enable_cache_prefill != 0, a->enable_sharemem_mhca != 0, a->enable_infinity_mhca != 0,
+        a->enable_infinity_gqca != 0, a->specify_decoding_multi_block, a->specify_decoding_tpb, a->cache, a->scale, &os,
+        a->output);
+    h->prepared = rc == ppl::common::RC_SUCCESS;
+    return (int)rc;
+}
+
+int pmxhip_mhca_get_derived(pmxhip_mhca_t h, pmxhip_mhca_derived* out)
+{
+    if (!h || !out || !h->prepared) return PMXHIP_INVALID_VALUE;
+    const mhca_class::config& c = h->op.cfg;
+    out->prefill_batches = c.prefill_batches;
+    out->q_stride_s = c.q_stride_s;
+    out->k_stride_s = c.k_stride_s;
+    out->v_stride_s = c.v_stride_s;
+    out->o_stride_s = c.o_stride_s;
+    out->mask_stride_s = c.mask_stride_s;
+    out->mask_stride_h = c.mask_stride_h;
+    out->attn_scale = c.attn_scale;
+    out->num_kv_repeats = c.num_kv_repeats;
+    out->decoding_algo = c.decoding_algo;
+    out->decoding_threads_per_block = c.decoding_threads_per_block;
+    out->decoding_multi_block_size = c.decoding_multi_block_size;
+    out->decoding_multi_block_partial_out_size = c.decoding_multi_block_partial_out_size;
+    out->decoding_multi_block_partial_log_sum_exp_size = c.decoding_multi_block_partial_log_sum_exp_size;
+    out->decoding_multi_block_counter_size = c.decoding_multi_block_counter_size;
+    out->workspace_size = c.workspace_size;
+    return PMXHIP_SUCCESS;
+}
+
+int pmxhip_mhca_set_workspace(pmxhip_mhca_t h, void* workspace)
+{
+    if (!h || !h->prepared) return PMXHIP_INVALID_VALUE;
+    h->op.cfg.workspace = workspace;
+    return PMXHIP_SUCCESS;
+}
+
+int pmxhip_mhca_forward_kvstore(pmxhip_mhca_t h, pmxhip_stream_t stream)
+{
+    if (!h || !h->prepared) return PMXHIP_INVALID_VALUE;
+    return (int)h->op.forward_kvstore(stream);
+}
+
+int pmxhip_mhca_forward_decode(pmxhip_mhca_t h, pmxhip_stream_t stream)
+{
+    if (!h || !h->prepared) return PMXHIP_INVALID_VALUE;
+    return (int)h->op.forward_decode(stream);
+}
+
+int pmxhip_mhca_forward_prefill(pmxhip_mhca_t h, pmxhip_stream_t stream)
+{
+    if (!h || !h->prepared) return PMXHIP_INVALID_VALUE;
+    return (int)h->op.forward_prefill(stream);
+}
+
+int pmxhip_mhca_forward(pmxhip_mhca_t h, pmxhip_stream_t stream)
+{
+    if (!h || !h->prepared) return PMXHIP_INVALID_VALUE;
+    return (int)h->op.forward(stream);
+}
+
+} // extern "C"

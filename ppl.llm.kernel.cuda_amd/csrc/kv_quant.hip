@@ -1,0 +1,129 @@
+// KV-cache quantise/append for gfx950: fp16 K/V -> symmetric int8 in groups of 8
+// channels with one fp16 scale per group, scattered into the cache.
+//
+// Arithmetic restated from the reference kernel
+// (src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/kernel.cu:128-154):
+//   absmax over the group in half; scale = half(float(absmax) / 127.0f);
+//   scale = scale > eps ? scale : eps with eps = half(1e-5f) (a half subnormal);
+//   q = (int8) round-half-even( half(x / scale) ).
+// The half quotient is formed as the correctly rounded binary32 quotient rounded
+// once more to binary16, which equals the correctly rounded half quotient
+// (24 >= 2*11 + 2), and the integer rounding is v_rndne -- HIP's __half2short_rn
+// truncates, so it is not used.
+//
+// Decomposition (this file's own): a flat grid over (new token, group of 8
+// channels); one lane owns one group of K and the same group of V: two 128-bit
+// loads, two 64-bit int8 stores, two 16-bit scale stores.  The sequence of a
+// token is found by bisection over seqstarts, so no workgroup is launched per
+// (position, sequence) pair that does not exist.
+#include "device_common.h"
+#include "launch_params.h"
+
+namespace pmxhip {
+
+namespace {
+
+constexpr int kQuantThreads = 256;
+
+struct Quantised {
+    u32x2 q;
+    half_t scale;
+};
+
+__device__ __forceinline__ Quantised quantise_group(const u32x4 raw)
+{
+    half_t x[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const half2_t h = bitcast<half2_t>(raw[i]);
+        x[2 * i] = h.x;
+        x[2 * i + 1] = h.y;
+    }
+    half_t amax = (half_t)0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const half_t ax = __builtin_fabsf16(x[i]);
+        amax = amax > ax ? amax : ax;
+    }
+    const half_t eps = (half_t)1e-5f;
+    half_t s = (half_t)((float)amax / 127.0f);
+    s = s > eps ? s : eps;
+    const float sf = (float)s;
+    uint32_t packed[2] = {0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const half_t quo = (half_t)((float)x[i] / sf);
+        const int qi = (int)__builtin_rintf((float)quo);
+        packed[i >> 2] |= ((uint32_t)qi & 0xffu) << (8 * (i & 3));
+    }
+    Quantised r;
+    r.q = u32x2{packed[0], packed[1]};
+    r.scale = s;
+    return r;
+}
+
+// largest b in [0, n) with starts[b] <= v   (starts non-decreasing, starts[0] <= v < starts[n]);
+// being the largest, it is never an empty sequence
+__device__ __forceinline__ int sequence_of(const int64_t* __restrict__ starts, int n, int64_t v)
+{
+    int lo = 0, hi = n - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (starts[mid] <= v) lo = mid;
+        else hi = mid - 1;
+    }
+    return lo;
+}
+
+} // namespace
+
+template <bool PAGED>
+__global__ __launch_bounds__(kQuantThreads) void kv_quantize_kernel(const QuantLaunch a)
+{
+    const int groups_per_head = a.head_dim >> 3;
+    const int groups_per_token = a.num_kv_heads * groups_per_head;
+    const int64_t first = a.seqstarts[0];
+    const int64_t n_tokens = a.seqstarts[a.batch] - first;
+    const int64_t n_units = n_tokens * groups_per_token;
+    const int64_t stride = (int64_t)gridDim.x * kQuantThreads;
+    for (int64_t u = (int64_t)blockIdx.x * kQuantThreads + threadIdx.x; u < n_units; u += stride) {
+        const int64_t tok = u / groups_per_token;
+        const int gi = (int)(u - tok * groups_per_token);
+        const int h = gi / groups_per_head;
+        const int d0 = (gi - h * groups_per_head) << 3;
+        const int64_t in_tok = first + tok;
+        const int b = sequence_of(a.seqstarts, (int)a.batch, in_tok);
+        const int64_t pos = a.start_pos[b] + (in_tok - a.seqstarts[b]);
+        const int64_t row = token_row<PAGED>(a.cachestarts, PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b, pos);
+
+        const int64_t in_idx = (int64_t)h * a.head_dim + d0;
+        const u32x4 kraw = *(const u32x4*)((const half_t*)a.current_key + in_tok * a.current_key_stride_s + in_idx);
+        const u32x4 vraw = *(const u32x4*)((const half_t*)a.current_value + in_tok * a.current_value_stride_s + in_idx);
+        const Quantised kq = quantise_group(kraw);
+        const Quantised vq = quantise_group(vraw);
+
+        const int64_t k_out = row * a.cache_stride_s + a.layer_idx * a.cache_stride_l + (int64_t)h * a.cache_stride_h + d0;
+        const int64_t v_out = k_out + a.cache_stride_kv;
+        *(u32x2*)(a.cache + k_out) = kq.q;
+        *(u32x2*)(a.cache + v_out) = vq.q;
+        ((half_t*)a.scale)[k_out >> 3] = kq.scale;
+        ((half_t*)a.scale)[v_out >> 3] = vq.scale;
+    }
+}
+
+int launch_kv_quantize(const QuantLaunch& a, hipStream_t stream)
+{
+    const int64_t groups_per_token = (int64_t)a.num_kv_heads * (a.head_dim >> 3);
+    const int64_t max_units = a.max_tokens * groups_per_token;
+    if (max_units <= 0) return 0;
+    int64_t blocks = (max_units + kQuantThreads - 1) / kQuantThreads;
+    const int64_t cap = 256 * 32; // grid-stride beyond this: enough waves to fill 256 CUs
+    if (blocks > cap) blocks = cap;
+    if (a.cache_mode == 1)
+        hipLaunchKernelGGL(kv_quantize_kernel<true>, dim3((unsigned)blocks), dim3(kQuantThreads), 0, stream, a);
+    else
+        hipLaunchKernelGGL(kv_quantize_kernel<false>, dim3((unsigned)blocks), dim3(kQuantThreads), 0, stream, a);
+    return 0;
+}
+
+} // namespace pmxhip

@@ -1,0 +1,105 @@
+// Kernel argument blocks and launcher prototypes shared between the host layer
+// (c_api.cpp) and the .hip translation units.
+#ifndef PMX_HIP_LAUNCH_PARAMS_H_
+#define PMX_HIP_LAUNCH_PARAMS_H_
+
+#include <hip/hip_runtime_api.h>
+#include <stdint.h>
+
+namespace pmxhip {
+
+struct QuantLaunch {
+    const void* current_key;
+    const void* current_value;
+    const int64_t* seqstarts;
+    const int64_t* cachestarts;
+    const int64_t* start_pos;
+    int8_t* cache;
+    void* scale;
+    int64_t batch;
+    int64_t layer_idx;
+    int32_t num_kv_heads;
+    int32_t head_dim;
+    int64_t current_key_stride_s;
+    int64_t current_value_stride_s;
+    int64_t cache_stride_s;
+    int64_t cache_stride_l;
+    int64_t cache_stride_h;
+    int64_t cache_stride_kv;
+    int64_t cachestarts_stride_b;
+    int64_t max_tokens; // batch * max_seqlen: upper bound of the new-token count
+    int32_t cache_mode;
+};
+
+struct DecodeLaunch {
+    const void* query;
+    const void* attn_mask;
+    void* output;
+    const void* cache;
+    const void* scale;
+    const int64_t* cachestarts;
+    const int64_t* kvstarts;
+    float* partial_out; // (ranges + batches, Hq, D)
+    float* partial_ml;  // (ranges + batches, Hq, 2)
+    float attn_scale;
+    int32_t cache_mode;
+    int64_t layer_idx;
+    int64_t num_kv_repeats;
+    int64_t query_stride_s;
+    int64_t output_stride_s;
+    int64_t mask_stride_s;
+    int64_t mask_stride_h;
+    int64_t cache_stride_s;
+    int64_t cache_stride_l;
+    int64_t cache_stride_h;
+    int64_t cache_stride_kv;
+    int64_t cachestarts_stride_b;
+    int64_t decoding_batches;
+    int64_t num_heads;
+    int64_t num_kv_heads;
+    int32_t head_dim;
+    int32_t ranges;               // workgroups along the kv-token stream
+    int32_t kv_heads_per_group;   // kv heads per workgroup (power of two)
+    int32_t q_heads_per_pass;     // GT
+    int32_t num_passes;           // ceil(num_kv_repeats / GT)
+    int32_t wg_tokens;            // tokens one workgroup iteration covers
+    int32_t min_tokens_per_range;
+};
+
+struct PrefillLaunch {
+    const void* query;
+    void* output;
+    const void* cache;
+    const void* scale;
+    const int64_t* seqstarts;   // already offset to the first prefill sequence
+    const int64_t* kvstarts;    // likewise
+    const int64_t* cachestarts; // likewise
+    float attn_scale;
+    int32_t is_causal;
+    int32_t cache_mode;
+    int64_t prefill_batches;
+    int64_t max_seqlen;
+    int64_t layer_idx;
+    int64_t num_heads;
+    int64_t num_kv_heads;
+    int32_t head_dim;
+    int64_t query_stride_s;
+    int64_t output_stride_s;
+    int64_t cache_stride_s;
+    int64_t cache_stride_l;
+    int64_t cache_stride_h;
+    int64_t cache_stride_kv;
+    int64_t cachestarts_stride_b;
+};
+
+int launch_kv_quantize(const QuantLaunch& a, hipStream_t stream);
+int launch_decode(const DecodeLaunch& a, hipStream_t stream);
+int decode_wg_tokens(int head_dim, int kv_heads_per_group);
+void launch_splitkv_combine_rows(const float* partial_out, const float* partial_ml, const int64_t* piece_begin,
+                                 const int64_t* piece_end, int64_t rows, int64_t head_dim, void* output,
+                                 hipStream_t stream);
+int launch_prefill(const PrefillLaunch& a, hipStream_t stream);
+
+} // namespace pmxhip
+
+#endif // PMX_HIP_LAUNCH_PARAMS_H_

@@ -1,0 +1,287 @@
+"""Host-side mirror of the pmx operator interface over the C ABI.
+
+Tensors are torch tensors that live in GPU memory; torch is used for nothing but
+allocation and the current stream.  Every function goes through
+libpmx_hip.so -- there is no PyTorch or CPU implementation behind these names.
+
+Names follow the reference operator
+(include/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention.h:25-159):
+``DynamicBatchingMultiHeadCacheAttention.heuristic_prepare / forward_kvstore /
+forward_decode / forward_prefill / forward``; ``key_value_cache`` is the append
+step as a free function.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import (DATATYPE_FLOAT16, DecodeParams, DecodePlan, KvstoreParams, MhcaDerived,
+                   MhcaPrepareArgs, PrefillParams, TensorShape)
+
+RC_SUCCESS = _lib.PMXHIP_SUCCESS
+RC_OTHER_ERROR = _lib.PMXHIP_OTHER_ERROR
+RC_UNSUPPORTED = _lib.PMXHIP_UNSUPPORTED
+RC_INVALID_VALUE = _lib.PMXHIP_INVALID_VALUE
+
+
+class PmxError(RuntimeError):
+    def __init__(self, code, where):
+        self.code = code
+        super().__init__("%s failed with status %d: %s" % (where, code, _lib.last_error()))
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    if isinstance(t, int):
+        return t
+    if not t.is_cuda:
+        raise ValueError("device tensor expected (got a CPU tensor)")
+    return t.data_ptr()
+
+
+def _stream(stream=None):
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return ctypes.c_void_p(stream.cuda_stream)
+
+
+def compute_units(device=None):
+    return torch.cuda.get_device_properties(device if device is not None else torch.cuda.current_device()).multi_processor_count
+
+
+def key_value_cache(current_key, current_value, seqstarts, cachestarts, start_pos, cache, scale, *,
+                    batch, max_seqlen, num_layer, layer_idx, num_kv_heads, head_dim, cache_mode, page_size,
+                    cache_stride_s, cache_stride_l, cache_stride_h, cache_stride_kv, cachestarts_stride_b,
+                    stream=None, check=True):
+    """Quantise/append `current_key`/`current_value` (fp16 [S, KVH, D]) into the int8 cache."""
+    p = KvstoreParams()
+    p.current_key = _ptr(current_key)
+    p.current_value = _ptr(current_value)
+    p.seqstarts = _ptr(seqstarts)
+    p.cachestarts = _ptr(cachestarts)
+    p.start_pos = _ptr(start_pos)
+    p.num_layer = num_layer
+    p.layer_idx = layer_idx
+    p.num_kv_heads = num_kv_heads
+    p.head_dim = head_dim
+    p.page_size = page_size
+    p.current_key_stride_s = num_kv_heads * head_dim
+    p.current_value_stride_s = num_kv_heads * head_dim
+    p.cache_stride_s = cache_stride_s
+    p.cache_stride_l = cache_stride_l
+    p.cache_stride_h = cache_stride_h
+    p.cache_stride_kv = cache_stride_kv
+    p.cachestarts_stride_b = cachestarts_stride_b
+    p.cache = _ptr(cache)
+    p.scale = _ptr(scale)
+    p.batch = batch
+    p.max_seqlen = max_seqlen
+    p.cache_mode = cache_mode
+    rc = _lib.lib().pmxhip_kv_cache_quantize(ctypes.byref(p), _stream(stream))
+    if check and rc != RC_SUCCESS:
+        raise PmxError(rc, "key_value_cache")
+    return rc
+
+
+def decode_plan(decoding_batches, num_heads, num_kv_heads, head_dim, max_kvlen, cus=None, ranges_hint=0):
+    plan = DecodePlan()
+    rc = _lib.lib().pmxhip_decode_plan_make(decoding_batches, num_heads, num_kv_heads, head_dim, max_kvlen,
+                                            compute_units() if cus is None else cus, ranges_hint, ctypes.byref(plan))
+    if rc != RC_SUCCESS:
+        raise PmxError(rc, "decode_plan")
+    return plan
+
+
+def decode_attention(query, output, cache, scale, cachestarts, kvstarts, *, attn_scale, layer_idx,
+                     decoding_batches, num_heads, num_kv_heads, head_dim, cache_mode, page_size,
+                     cache_stride_s, cache_stride_l, cache_stride_h, cache_stride_kv, cachestarts_stride_b,
+                     num_token_ranges, workspace=None, attn_mask=None, mask_stride_s=0, mask_stride_h=0,
+                     stream=None, check=True):
+    """Decode attention of sequences [0, decoding_batches); output fp16 [B_dec, Hq, D]."""
+    p = DecodeParams()
+    p.query = _ptr(query)
+    p.attn_mask = _ptr(attn_mask)
+    p.output = _ptr(output)
+    p.cache = _ptr(cache)
+    p.scale = _ptr(scale)
+    p.cachestarts = _ptr(cachestarts)
+    p.kvstarts = _ptr(kvstarts)
+    p.attn_scale = attn_scale
+    p.layer_idx = layer_idx
+    p.num_kv_repeats = num_heads // num_kv_heads if num_kv_heads else 0
+    p.page_size = page_size
+    p.query_stride_s = num_heads * head_dim
+    p.output_stride_s = num_heads * head_dim
+    p.mask_stride_s = mask_stride_s
+    p.mask_stride_h = mask_stride_h
+    p.cache_stride_s = cache_stride_s
+    p.cache_stride_l = cache_stride_l
+    p.cache_stride_h = cache_stride_h
+    p.cache_stride_kv = cache_stride_kv
+    p.cachestarts_stride_b = cachestarts_stride_b
+    p.decoding_batches = decoding_batches
+    p.num_heads = num_heads
+    p.num_kv_heads = num_kv_heads
+    p.head_dim = head_dim
+    p.cache_mode = cache_mode
+    p.num_token_ranges = num_token_ranges
+    p.workspace = _ptr(workspace)
+    p.workspace_size = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    rc = _lib.lib().pmxhip_decode_attention(ctypes.byref(p), _stream(stream))
+    if check and rc != RC_SUCCESS:
+        raise PmxError(rc, "decode_attention")
+    return rc
+
+
+def splitkv_combine(partial_out, partial_ml, piece_begin, piece_end, output, *, head_dim, stream=None):
+    rows = piece_begin.numel()
+    rc = _lib.lib().pmxhip_splitkv_combine(_ptr(partial_out), _ptr(partial_ml), _ptr(piece_begin), _ptr(piece_end),
+                                           rows, head_dim, _ptr(output), _stream(stream))
+    if rc != RC_SUCCESS:
+        raise PmxError(rc, "splitkv_combine")
+    return rc
+
+
+def prefill_attention(query, output, cache, scale, seqstarts, kvstarts, cachestarts, *, attn_scale, is_causal,
+                      batch, decoding_batches, max_seqlen, max_kvlen, layer_idx, num_heads, num_kv_heads,
+                      head_dim, cache_mode, page_size, cache_stride_s, cache_stride_l, cache_stride_h,
+                      cache_stride_kv, cachestarts_stride_b, stream=None, check=True):
+    p = PrefillParams()
+    p.query = _ptr(query)
+    p.output = _ptr(output)
+    p.cache = _ptr(cache)
+    p.scale = _ptr(scale)
+    p.seqstarts = _ptr(seqstarts)
+    p.kvstarts = _ptr(kvstarts)
+    p.cachestarts = _ptr(cachestarts)
+    p.attn_scale = attn_scale
+    p.is_causal = 1 if is_causal else 0
+    p.batch = batch
+    p.decoding_batches = decoding_batches
+    p.max_seqlen = max_seqlen
+    p.max_kvlen = max_kvlen
+    p.layer_idx = layer_idx
+    p.num_heads = num_heads
+    p.num_kv_heads = num_kv_heads
+    p.head_dim = head_dim
+    p.cache_mode = cache_mode
+    p.page_size = page_size
+    p.query_stride_s = num_heads * head_dim
+    p.output_stride_s = num_heads * head_dim
+    p.cache_stride_s = cache_stride_s
+    p.cache_stride_l = cache_stride_l
+    p.cache_stride_h = cache_stride_h
+    p.cache_stride_kv = cache_stride_kv
+    p.cachestarts_stride_b = cachestarts_stride_b
+    rc = _lib.lib().pmxhip_prefill_attention(ctypes.byref(p), _stream(stream))
+    if check and rc != RC_SUCCESS:
+        raise PmxError(rc, "prefill_attention")
+    return rc
+
+
+class DynamicBatchingMultiHeadCacheAttention:
+    """The operator class (C++ `dynamic_batching_multi_head_cache_attention`) behind its C handle."""
+
+    def __init__(self):
+        self._h = _lib.lib().pmxhip_mhca_create()
+        if not self._h:
+            raise MemoryError("pmxhip_mhca_create failed")
+        self._keep = None
+        self.workspace = None
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            _lib.lib().pmxhip_mhca_destroy(h)
+
+    def heuristic_prepare(self, *, query=None, query_shape, current_key=None, current_key_shape,
+                          current_value=None, current_value_shape, attn_mask=None, attn_mask_shape=(),
+                          seqstarts=None, kvstarts=None, cachestarts=None, start_pos=None, alibi_slopes=None,
+                          is_causal=True, batch, decoding_batches, max_seqlen, max_kvlen, layer_idx, num_layer,
+                          num_heads, num_kv_heads, head_dim, cache_mode, page_size, cache_stride_s,
+                          cache_stride_l, cache_stride_h, cache_stride_kv, cachestarts_stride_b,
+                          enable_cache_prefill=True, enable_sharemem_mhca=True, enable_infinity_mhca=True,
+                          enable_infinity_gqca=True, specify_decoding_multi_block=1, specify_decoding_tpb=0,
+                          cache=None, scale=None, output=None, output_shape, datatype=DATATYPE_FLOAT16,
+                          compute_units_override=None, shared_mem_per_block_optin=65536):
+        """Same arguments, in the same order of meaning, as the reference's heuristic_prepare
+        (multi_head_cache_attention.h:107-148).  Returns the status code; pointers may be None
+        for host-only validation runs."""
+        a = MhcaPrepareArgs()
+        a.compute_units = compute_units_override if compute_units_override is not None else compute_units()
+        a.shared_mem_per_block_optin = shared_mem_per_block_optin
+        a.query_shape = TensorShape.of(query_shape, datatype)
+        a.query = _ptr(query)
+        a.current_key_shape = TensorShape.of(current_key_shape, datatype)
+        a.current_key = _ptr(current_key)
+        a.current_value_shape = TensorShape.of(current_value_shape, datatype)
+        a.current_value = _ptr(current_value)
+        a.attn_mask_shape = TensorShape.of(attn_mask_shape, datatype)
+        a.attn_mask = _ptr(attn_mask)
+        a.seqstarts = _ptr(seqstarts)
+        a.kvstarts = _ptr(kvstarts)
+        a.cachestarts = _ptr(cachestarts)
+        a.start_pos = _ptr(start_pos)
+        a.alibi_slopes = _ptr(alibi_slopes)
+        a.is_causal = 1 if is_causal else 0
+        a.batch = batch
+        a.decoding_batches = decoding_batches
+        a.max_seqlen = max_seqlen
+        a.max_kvlen = max_kvlen
+        a.layer_idx = layer_idx
+        a.num_layer = num_layer
+        a.num_heads = num_heads
+        a.num_kv_heads = num_kv_heads
+        a.head_dim = head_dim
+        a.cache_mode = cache_mode
+        a.page_size = page_size
+        a.cache_stride_s = cache_stride_s
+        a.cache_stride_l = cache_stride_l
+        a.cache_stride_h = cache_stride_h
+        a.cache_stride_kv = cache_stride_kv
+        a.cachestarts_stride_b = cachestarts_stride_b
+        a.enable_cache_prefill = int(enable_cache_prefill)
+        a.enable_sharemem_mhca = int(enable_sharemem_mhca)
+        a.enable_infinity_mhca = int(enable_infinity_mhca)
+        a.enable_infinity_gqca = int(enable_infinity_gqca)
+        a.specify_decoding_multi_block = specify_decoding_multi_block
+        a.specify_decoding_tpb = specify_decoding_tpb
+        a.cache = _ptr(cache)
+        a.scale = _ptr(scale)
+        a.output_shape = TensorShape.of(output_shape, datatype)
+        a.output = _ptr(output)
+        # keep the tensors alive for as long as the operator may launch on them
+        self._keep = (query, current_key, current_value, attn_mask, seqstarts, kvstarts, cachestarts, start_pos,
+                      alibi_slopes, cache, scale, output)
+        return _lib.lib().pmxhip_mhca_heuristic_prepare(self._h, ctypes.byref(a))
+
+    @property
+    def cfg(self):
+        d = MhcaDerived()
+        rc = _lib.lib().pmxhip_mhca_get_derived(self._h, ctypes.byref(d))
+        if rc != RC_SUCCESS:
+            raise PmxError(rc, "cfg (heuristic_prepare has not succeeded)")
+        return d
+
+    def set_workspace(self, workspace):
+        self.workspace = workspace
+        return _lib.lib().pmxhip_mhca_set_workspace(self._h, _ptr(workspace))
+
+    def allocate_workspace(self, device="cuda"):
+        n = int(self.cfg.workspace_size)
+        ws = torch.empty(max(n, 16), dtype=torch.uint8, device=device) if n > 0 else None
+        self.set_workspace(ws)
+        return ws
+
+    def forward_kvstore(self, stream=None):
+        return _lib.lib().pmxhip_mhca_forward_kvstore(self._h, _stream(stream))
+
+    def forward_decode(self, stream=None):
+        return _lib.lib().pmxhip_mhca_forward_decode(self._h, _stream(stream))
+
+    def forward_prefill(self, stream=None):
+        return _lib.lib().pmxhip_mhca_forward_prefill(self._h, _stream(stream))
+
+    def forward(self, stream=None):
+        return _lib.lib().pmxhip_mhca_forward(self._h, _stream(stream))

@@ -1,0 +1,178 @@
+"""GPU parity of decode attention (and its split-KV combine) against the CPU
+oracle, through the C ABI.  Tolerance: |got - ref| <= 2e-3 + 1e-2 * |ref| against
+the fp32 dequantised reference."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import (assert_attention_close, host_cache, oracle_append_step, oracle_decode, oracle_fill_history,
+                      oracle_layout_kwargs)
+
+pytestmark = pytest.mark.gpu
+
+
+def make_case(pkg, oracle, seed, **kw):
+    """Cache quantised by the oracle on the host, uploaded as-is: decode parity is then
+    independent of the append kernel."""
+    bt, rng = pkg.workloads.custom_batch(seed, **kw)
+    cache, scale = host_cache(bt)
+    oracle_fill_history(oracle, pkg, bt, rng, cache, scale)
+    q, k, v = pkg.workloads.step_inputs(bt, rng)
+    oracle_append_step(oracle, bt, k, v, cache, scale)
+    dev = pkg.harness.DeviceBatch(bt)
+    dev.cache.copy_(torch.from_numpy(cache))
+    dev.scale.copy_(torch.from_numpy(scale))
+    dev.set_step_inputs(q, k, v)
+    return bt, dev, q, cache, scale
+
+
+def run_decode(dev, ranges=0, **kw):
+    dev.output.fill_(float("nan"))
+    plan, ws = dev.decode_only(num_token_ranges=ranges, **kw)
+    torch.cuda.synchronize()
+    return dev.output[:dev.bt.decoding_batches].float().cpu().numpy(), plan
+
+
+SHAPES = [
+    # (Hq, KVH, D)
+    (8, 8, 64), (4, 4, 128), (32, 8, 128), (16, 2, 128), (12, 2, 128), (6, 2, 96), (4, 2, 256), (32, 2, 64),
+    (3, 3, 128), (24, 8, 128), (2, 1, 128),
+]
+
+
+@pytest.mark.parametrize("cache_mode", [0, 1])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_decode_matches_oracle(pkg, oracle, shape, cache_mode):
+    hq, hkv, d = shape
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 200 + hq + d, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                         cache_mode=cache_mode, dec_kv_lens=[1, 300, 17, 129, 640, 2, 128],
+                                         outliers=True)
+    ref = oracle_decode(oracle, bt, q, cache, scale)
+    for ranges in (1, 0, 3, 11):
+        got, plan = run_decode(dev, ranges)
+        assert_attention_close(got, ref, "shape %s mode %d ranges %d" % (shape, cache_mode, plan.num_token_ranges))
+
+
+def test_decode_c1_golden_shape(pkg, oracle):
+    bt, rng = pkg.workloads.make_batch("C1")
+    cache, scale = host_cache(bt)
+    oracle_fill_history(oracle, pkg, bt, rng, cache, scale)
+    q, k, v = pkg.workloads.step_inputs(bt, rng)
+    oracle_append_step(oracle, bt, k, v, cache, scale)
+    dev = pkg.harness.DeviceBatch(bt)
+    dev.cache.copy_(torch.from_numpy(cache))
+    dev.scale.copy_(torch.from_numpy(scale))
+    dev.set_step_inputs(q, k, v)
+    ref = oracle_decode(oracle, bt, q, cache, scale)
+    got, _ = run_decode(dev)
+    assert_attention_close(got, ref, "C1")
+
+
+def test_decode_empty_sequence_and_closed_forms(pkg, oracle):
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 77, num_heads=8, num_kv_heads=2, head_dim=128, cache_mode=1,
+                                         dec_kv_lens=[1, 40, 1, 9])
+    # make sequence 1 empty: kv length 0 -> zeros (the reference's 0/(0+1e-6))
+    bt.kv_lens[1] = 0
+    bt.kvstarts = np.concatenate([[0], np.cumsum(bt.kv_lens)]).astype(np.int64)
+    dev.kvstarts.copy_(torch.from_numpy(bt.kvstarts))
+    ref = oracle_decode(oracle, bt, q, cache, scale)
+    assert (ref[1] == 0).all()
+    for ranges in (1, 2):
+        got, _ = run_decode(dev, ranges)
+        assert_attention_close(got, ref, "empty seq")
+        assert (got[1] == 0).all()
+        # kvlen = 1: the output is the dequantised V row, exactly representable -> fp16 rounding only
+        for b in (0, 2):
+            tok = int(bt.cachestarts[b, 0])
+            vrow = cache[0, 1, tok].astype(np.float32) * np.repeat(scale[0, 1, tok].astype(np.float32), 8, -1)
+            want = np.repeat(vrow, 4, axis=0).astype(np.float16).astype(np.float32)
+            np.testing.assert_allclose(got[b], want, rtol=2e-3, atol=1e-6)
+
+
+def test_decode_gqa_identical_queries_and_mha_equivalence(pkg, oracle):
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 78, num_heads=8, num_kv_heads=2, head_dim=128, cache_mode=0,
+                                         dec_kv_lens=[333, 64])
+    q2 = q.copy()
+    q2[:, 1:4] = q2[:, 0:1]
+    dev.query.copy_(torch.from_numpy(q2))
+    got, _ = run_decode(dev, 2)
+    for g in range(1, 4):
+        assert np.array_equal(got[:, g], got[:, 0])
+
+
+def test_decode_with_mask(pkg, oracle):
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 79, num_heads=8, num_kv_heads=4, head_dim=128, cache_mode=1,
+                                         dec_kv_lens=[70, 300, 5])
+    total = int(bt.kvstarts[-1])
+    width = (total + 7) // 8 * 8
+    rng = np.random.default_rng(3)
+    for per_head in (True, False):
+        shape = (bt.num_heads, bt.batch, width) if per_head else (bt.batch, width)
+        mask = rng.standard_normal(shape).astype(np.float16)
+        mask[..., 1, 5:9] = -np.inf
+        msh = bt.batch * width if per_head else 0
+        ref = oracle_decode(oracle, bt, q, cache, scale, attn_mask=mask, mask_stride_s=width, mask_stride_h=msh)
+        md = torch.from_numpy(mask).cuda()
+        for ranges in (1, 4):
+            got, _ = run_decode(dev, ranges, attn_mask=md, mask_stride_s=width, mask_stride_h=msh)
+            assert_attention_close(got, ref, "mask per_head=%s ranges=%d" % (per_head, ranges))
+
+
+def test_combine_entry_point_against_oracle_pieces(pkg, oracle):
+    """pmxhip_splitkv_combine on pieces produced by the oracle: any cut of the kv range gives the single-pass result."""
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 80, num_heads=4, num_kv_heads=2, head_dim=128, cache_mode=1,
+                                         dec_kv_lens=[97, 260])
+    ref = oracle_decode(oracle, bt, q, cache, scale)
+    kw = oracle_layout_kwargs(bt)
+    log2e = 1.4426950408889634
+    po, pml, begin, end = [], [], [], []
+    rng = np.random.default_rng(4)
+    for b in range(2):
+        n = int(bt.kv_lens[b])
+        for h in range(4):
+            cuts = sorted(rng.choice(np.arange(1, n), size=int(rng.integers(0, 6)), replace=False).tolist())
+            edges = [0] + cuts + [n]
+            if h == 2:
+                edges.insert(1, edges[1])  # an empty piece
+            begin.append(len(po))
+            for a, e in zip(edges[:-1], edges[1:]):
+                o, m, s = oracle.decode_partial(q[b:], cache, scale, bt.cachestarts[b:], 0, h, a, e, 4, 2, 128,
+                                                bt.attn_scale, 0, bt.page_size, **kw)
+                po.append(o)
+                # the kernel keeps the running max in log2 units; an empty piece carries sum 0
+                pml.append([m * log2e if s > 0 else -1e30, s])
+            end.append(len(po))
+    out = torch.zeros(8, 128, dtype=torch.float16, device="cuda")
+    pkg.ops.splitkv_combine(torch.tensor(np.stack(po), dtype=torch.float32, device="cuda"),
+                            torch.tensor(pml, dtype=torch.float32, device="cuda"),
+                            torch.tensor(begin, dtype=torch.int64, device="cuda"),
+                            torch.tensor(end, dtype=torch.int64, device="cuda"), out, head_dim=128)
+    torch.cuda.synchronize()
+    assert_attention_close(out.float().cpu().numpy().reshape(2, 4, 128), ref, "combine")
+
+
+@pytest.mark.parametrize("name", ["C2", "C3", "C4"])
+def test_decode_full_size_properties(pkg, oracle, name):
+    """At the benchmark's full sizes the oracle is too slow for every row, so: (1) the split count
+    does not change the result (1 range vs the planned hundreds), (2) sampled rows match the oracle."""
+    bt, rng = pkg.workloads.make_batch(name)
+    dev = pkg.harness.DeviceBatch(bt)
+    dev.fill_history_random_bytes(seed=bt.seed)
+    q, k, v = pkg.workloads.step_inputs(bt, rng)
+    dev.set_step_inputs(q, k, v)
+    got_many, plan = run_decode(dev, 0)
+    assert plan.num_token_ranges > 1
+    got_few, _ = run_decode(dev, 7)
+    assert not np.isnan(got_many).any()
+    np.testing.assert_allclose(got_many, got_few, rtol=2e-2, atol=4e-3)
+    # sampled rows against the oracle (host copy of the whole cache)
+    cache = dev.cache.cpu().numpy()
+    scale = dev.scale.cpu().numpy()
+    kw = oracle_layout_kwargs(bt)
+    pick = np.random.default_rng(0)
+    for b in pick.choice(bt.decoding_batches, size=3, replace=False):
+        for h in pick.choice(bt.num_heads, size=2, replace=False):
+            o, _, _ = oracle.decode_partial(q[b:], cache, scale, bt.cachestarts[b:], 0, int(h), 0, int(bt.kv_lens[b]),
+                                            bt.num_heads, bt.num_kv_heads, bt.head_dim, bt.attn_scale, 0,
+                                            bt.page_size, **kw)
+            assert_attention_close(got_many[b, h], o, "%s b=%d h=%d" % (name, b, h))
