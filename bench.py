@@ -1,0 +1,195 @@
+#!/usr/bin/env python3
+"""Benchmark of the int8-KV decode layer call on one MI355X.
+
+One step = one layer call of the hot path over one synthetic dynamic batch:
+quantise/append of the step's new K/V rows, decode attention over the int8 cache
+(token-range kernel + combine) and, for the mixed workload, the chunked-prefill
+tile.  Inputs are resident in HBM before the timed region.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3]
+
+Prints one JSON line.  `value` = algorithmic decode bytes of the batch divided by
+the whole step time (GB/s); `roofline` prices the dominant kernel alone (the
+token-range decode kernel), timed with events on the stream it is launched on;
+`cpu_baseline` is the CPU oracle on a bounded sample of the same batch.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def read_traffic(workload):
+    """HBM bytes per launch of the decode kernel from the committed rocprofv3 --pmc summary, or None."""
+    path = os.path.join(ROOT, "profiles", "decode_attention_%s_traffic.txt" % workload)
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return float(line.split(":", 1)[1])
+    except OSError:
+        pass
+    return None
+
+
+def cpu_baseline(oracle, bt, q, cache_host, scale_host, budget_s=12.0):
+    """The oracle's decode attention over the first sequences of the batch, sized to the time budget."""
+    lay = bt.layout
+    kw = dict(cache_stride_s=lay.stride_s, cache_stride_l=lay.stride_l, cache_stride_h=lay.stride_h,
+              cache_stride_kv=lay.stride_kv, cachestarts_stride_b=bt.cachestarts_stride_b)
+    d = bt.head_dim
+    per_tok = bt.num_kv_heads * (2 * d + 2 * (d // 8) * 2)
+
+    def run(nseq):
+        kvstarts = bt.kvstarts[:nseq + 1]
+        t0 = time.perf_counter()
+        oracle.decode_attention(q, cache_host, scale_host, bt.cachestarts, kvstarts, nseq, bt.num_heads,
+                                bt.num_kv_heads, d, bt.attn_scale, bt.layer_idx, bt.page_size, **kw)
+        dt = time.perf_counter() - t0
+        tokens = int(bt.kv_lens[:nseq].sum())
+        return dt, tokens * per_tok + 2 * nseq * bt.num_heads * d * 2, tokens
+
+    n0 = max(1, min(bt.decoding_batches, 4))
+    dt, nbytes, tokens = run(n0)  # also warms the pages
+    rate = tokens / max(dt, 1e-6)
+    want = rate * budget_s
+    cum = np.cumsum(bt.kv_lens[:bt.decoding_batches])
+    nseq = int(min(bt.decoding_batches, max(n0, np.searchsorted(cum, want) + 1)))
+    dt, nbytes, tokens = run(nseq)
+    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": oracle.num_threads(), "kind": "port",
+            "sample": "decode attention of the first %d of %d sequences (%d kv tokens), one pass, %.2f s"
+                      % (nseq, bt.decoding_batches, tokens, dt),
+            "us_per_layer_extrapolated": dt * 1e6 * bt.decode_kv_tokens / max(tokens, 1)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C3m0", "C4", "C5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--ranges", type=int, default=0, help="token ranges for decode (0 = planned)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards by kv head "
+              "with no exchange, see DESIGN.md)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    pkg = entry.load_package()
+    if not os.path.exists(pkg._lib.LIB_PATH):
+        entry.build()
+    wl, harness, ops = pkg.workloads, pkg.harness, pkg.ops
+    torch.cuda.set_device(0)
+
+    bt, rng = wl.make_batch(args.workload)
+    dev = harness.DeviceBatch(bt)
+    # context already in the cache: quantised from seeded fp16 rows by the HIP append kernel
+    dev.fill_history(rng, max_rows=1 << 15)
+    q, k, v = wl.step_inputs(bt, rng)
+    dev.set_step_inputs(q, k, v)
+    op = dev.make_operator(specify_decoding_multi_block=1)
+    if args.ranges:
+        plan = ops.decode_plan(bt.decoding_batches, bt.num_heads, bt.num_kv_heads, bt.head_dim, bt.max_kvlen,
+                               ranges_hint=args.ranges)
+    else:
+        plan = ops.decode_plan(bt.decoding_batches, bt.num_heads, bt.num_kv_heads, bt.head_dim, bt.max_kvlen)
+    stream = torch.cuda.current_stream()
+
+    def step():
+        rc = op.forward(stream)
+        if rc != 0:
+            raise RuntimeError("forward() returned %d" % rc)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    step_s = (time.perf_counter() - t0) / args.steps
+
+    # per-kernel durations: events on the launch stream around each stage
+    def time_stage(fn, n):
+        fn()
+        torch.cuda.synchronize()
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+        for a, b in evs:
+            a.record(stream)
+            fn()
+            b.record(stream)
+        torch.cuda.synchronize()
+        ts = sorted(a.elapsed_time(b) * 1e3 for a, b in evs)
+        return {"avg_us": float(np.mean(ts)), "median_us": float(ts[len(ts) // 2]), "min_us": float(ts[0])}
+
+    n_ev = max(20, args.steps)
+    ws = op.workspace
+    t_ranges = time_stage(lambda: dev.decode_only(num_token_ranges=plan.num_token_ranges, workspace=ws, stage=1), n_ev)
+    t_combine = time_stage(lambda: dev.decode_only(num_token_ranges=plan.num_token_ranges, workspace=ws, stage=2), n_ev)
+    t_append = time_stage(lambda: op.forward_kvstore(stream), n_ev)
+    stages = {"decode_ranges": t_ranges, "decode_combine": t_combine, "append": t_append}
+    if bt.batch > bt.decoding_batches:
+        stages["prefill"] = time_stage(lambda: op.forward_prefill(stream), n_ev)
+
+    dec_bytes = bt.decode_algorithmic_bytes()
+    achieved = dec_bytes / (t_ranges["avg_us"] * 1e-6) / 1e9
+    out = {
+        "metric": "int8-KV decode attention: achieved HBM GB/s over the whole layer call (us/layer in us_per_layer)",
+        "value": dec_bytes / step_s / 1e9,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": step_s * 1e3,
+        "us_per_layer": step_s * 1e6,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 cache, fp16 in/out, fp32 accumulate",
+        "data": "synthetic (numpy default_rng(%d); cache filled through the HIP quantise/append kernel)" % bt.seed,
+        "config": {
+            "workload": "%s: %d decode seqs, %d q / %d kv heads, D=%d, %d kv tokens (max %d), cache_mode %d%s" % (
+                bt.name, bt.decoding_batches, bt.num_heads, bt.num_kv_heads, bt.head_dim, bt.decode_kv_tokens,
+                bt.max_kvlen, bt.cache_mode,
+                ", + %d prefill seqs (%d query rows)" % (bt.batch - bt.decoding_batches,
+                                                         int(bt.q_lens[bt.decoding_batches:].sum()))
+                if bt.batch > bt.decoding_batches else ""),
+            "algorithmic_bytes": dec_bytes,
+            "token_ranges": int(plan.num_token_ranges),
+            "kv_heads_per_group": int(plan.kv_heads_per_group),
+            "q_heads_per_pass": int(plan.q_heads_per_pass),
+            "step": "append + decode (token-range kernel + combine)" + (" + prefill" if "prefill" in stages else ""),
+        },
+        "stages_us": stages,
+        "roofline": {
+            "kernel": "decode_attention_kernel",
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": read_traffic(bt.name),
+        },
+    }
+    if "prefill" in stages:
+        fl = bt.prefill_flops()
+        out["prefill"] = {"flops": fl, "achieved_tflops": fl / (stages["prefill"]["avg_us"] * 1e-6) / 1e12,
+                          "peak_tflops": 2500.0}
+    if not args.no_cpu_baseline:
+        oracle = entry.load_oracle()
+        out["cpu_baseline"] = cpu_baseline(oracle, bt, q, dev.cache.cpu().numpy(), dev.scale.cpu().numpy())
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

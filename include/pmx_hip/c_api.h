@@ -143,6 +143,13 @@ PMXHIP_API int pmxhip_decode_plan_make(int64_t decoding_batches, int64_t num_hea
 
 PMXHIP_API int pmxhip_decode_attention(const pmxhip_decode_params* p, pmxhip_stream_t stream);
 
+/* The same step split at its kernel boundary, for callers that time or overlap
+ * the two kernels: stage 1 = the token-range kernel only (final rows of
+ * sequences that fit one range, float32 pieces of the others), stage 2 = the
+ * combine kernel only, stage 0 = both (== pmxhip_decode_attention).  The
+ * reference fuses the two (kernel.cu:600-678), so it has no counterpart. */
+PMXHIP_API int pmxhip_decode_attention_stage(const pmxhip_decode_params* p, int32_t stage, pmxhip_stream_t stream);
+
 /* ---- split-KV combine on caller-supplied pieces ----------------------------
  * The merge of kernel.cu:617-665 as a stand-alone kernel: for each of `rows`
  * (sequence, head) pairs, merges pieces [piece_begin[r], piece_end[r]) of

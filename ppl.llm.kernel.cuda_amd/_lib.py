@@ -23,7 +23,8 @@ DATATYPE_FLOAT32 = 6
 EXPORTED_SYMBOLS = (
     "pmxhip_version", "pmxhip_last_error",
     "pmxhip_kv_cache_quantize", "pmxhip_key_value_cache",
-    "pmxhip_decode_plan_make", "pmxhip_decode_attention", "pmxhip_splitkv_combine",
+    "pmxhip_decode_plan_make", "pmxhip_decode_attention", "pmxhip_decode_attention_stage",
+    "pmxhip_splitkv_combine",
     "pmxhip_prefill_attention",
     "pmxhip_mhca_create", "pmxhip_mhca_destroy", "pmxhip_mhca_heuristic_prepare",
     "pmxhip_mhca_get_derived", "pmxhip_mhca_set_workspace",
@@ -160,6 +161,8 @@ def lib():
     L.pmxhip_decode_plan_make.argtypes = [c_i64] * 5 + [c_i32, c_i32, ctypes.POINTER(DecodePlan)]
     L.pmxhip_decode_attention.restype = ctypes.c_int
     L.pmxhip_decode_attention.argtypes = [ctypes.POINTER(DecodeParams), c_vp]
+    L.pmxhip_decode_attention_stage.restype = ctypes.c_int
+    L.pmxhip_decode_attention_stage.argtypes = [ctypes.POINTER(DecodeParams), c_i32, c_vp]
     L.pmxhip_splitkv_combine.restype = ctypes.c_int
     L.pmxhip_splitkv_combine.argtypes = [c_vp] * 4 + [c_i64, c_i64, c_vp, c_vp]
     L.pmxhip_prefill_attention.restype = ctypes.c_int

@@ -187,6 +187,12 @@ int pmxhip_decode_plan_make(int64_t decoding_batches, int64_t num_heads, int64_t
 
 int pmxhip_decode_attention(const pmxhip_decode_params* p, pmxhip_stream_t stream)
 {
+    return pmxhip_decode_attention_stage(p, 0, stream);
+}
+
+int pmxhip_decode_attention_stage(const pmxhip_decode_params* p, int32_t stage, pmxhip_stream_t stream)
+{
+    if (stage < 0 || stage > 2) return fail(PMXHIP_INVALID_VALUE, "decode_attention: stage must be 0, 1 or 2");
     if (!p) return fail(PMXHIP_INVALID_VALUE, "decode_attention: null params");
     if (p->decoding_batches < 0) return fail(PMXHIP_INVALID_VALUE, "decode_attention: negative decoding_batches");
     if (p->decoding_batches == 0) return PMXHIP_SUCCESS; // kernel.cu:2084
@@ -250,7 +256,7 @@ int pmxhip_decode_attention(const pmxhip_decode_params* p, pmxhip_stream_t strea
     a.num_passes = plan.num_passes;
     a.wg_tokens = pmxhip::decode_wg_tokens((int)p->head_dim, plan.kv_heads_per_group);
     a.min_tokens_per_range = a.wg_tokens > 128 ? a.wg_tokens : 128;
-    if (pmxhip::launch_decode(a, stream) != 0) return fail(PMXHIP_UNSUPPORTED, "decode_attention: no kernel for this shape");
+    if (pmxhip::launch_decode(a, stage, stream) != 0) return fail(PMXHIP_UNSUPPORTED, "decode_attention: no kernel for this shape");
     return launch_status("decode_attention");
 }
 

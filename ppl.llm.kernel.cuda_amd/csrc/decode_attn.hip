@@ -412,28 +412,31 @@ static void launch_decode_dgt(const DecodeLaunch& a, dim3 grid, hipStream_t stre
 }
 
 template <int D>
-static int launch_decode_d(const DecodeLaunch& a, hipStream_t stream)
+static int launch_decode_d(const DecodeLaunch& a, int stage, hipStream_t stream)
 {
     const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / a.kv_heads_per_group), (unsigned)a.num_passes);
-    switch (a.q_heads_per_pass) {
-        case 1: launch_decode_dgt<D, 1>(a, grid, stream); break;
-        case 2: launch_decode_dgt<D, 2>(a, grid, stream); break;
-        case 4: launch_decode_dgt<D, 4>(a, grid, stream); break;
-        case 8: launch_decode_dgt<D, 8>(a, grid, stream); break;
-        default: return 1;
+    if (stage != 2) {
+        switch (a.q_heads_per_pass) {
+            case 1: launch_decode_dgt<D, 1>(a, grid, stream); break;
+            case 2: launch_decode_dgt<D, 2>(a, grid, stream); break;
+            case 4: launch_decode_dgt<D, 4>(a, grid, stream); break;
+            case 8: launch_decode_dgt<D, 8>(a, grid, stream); break;
+            default: return 1;
+        }
     }
+    if (stage == 1) return 0;
     // always run: it also writes the zero rows of empty sequences
     hipLaunchKernelGGL((decode_combine_kernel<D>), dim3((unsigned)a.num_heads, (unsigned)a.decoding_batches), dim3(64), 0, stream, a);
     return 0;
 }
 
-int launch_decode(const DecodeLaunch& a, hipStream_t stream)
+int launch_decode(const DecodeLaunch& a, int stage, hipStream_t stream)
 {
     switch (a.head_dim) {
-        case 64: return launch_decode_d<64>(a, stream);
-        case 96: return launch_decode_d<96>(a, stream);
-        case 128: return launch_decode_d<128>(a, stream);
-        case 256: return launch_decode_d<256>(a, stream);
+        case 64: return launch_decode_d<64>(a, stage, stream);
+        case 96: return launch_decode_d<96>(a, stage, stream);
+        case 128: return launch_decode_d<128>(a, stage, stream);
+        case 256: return launch_decode_d<256>(a, stage, stream);
         default: return 1;
     }
 }

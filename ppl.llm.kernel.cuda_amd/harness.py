@@ -108,7 +108,7 @@ class DeviceBatch:
         return op
 
     def decode_only(self, num_token_ranges=0, workspace=None, attn_mask=None, mask_stride_s=0, mask_stride_h=0,
-                    output=None):
+                    output=None, stage=0):
         """Decode attention through the flat C entry point (no operator object)."""
         bt = self.bt
         plan = ops.decode_plan(bt.decoding_batches, bt.num_heads, bt.num_kv_heads, bt.head_dim, bt.max_kvlen,
@@ -121,6 +121,6 @@ class DeviceBatch:
                              decoding_batches=bt.decoding_batches, num_heads=bt.num_heads,
                              num_kv_heads=bt.num_kv_heads, head_dim=bt.head_dim,
                              num_token_ranges=plan.num_token_ranges, workspace=workspace,
-                             attn_mask=attn_mask, mask_stride_s=mask_stride_s, mask_stride_h=mask_stride_h,
+                             attn_mask=attn_mask, mask_stride_s=mask_stride_s, mask_stride_h=mask_stride_h, stage=stage,
                              **self.layout_kwargs())
         return plan, workspace

@@ -97,7 +97,7 @@ def decode_attention(query, output, cache, scale, cachestarts, kvstarts, *, attn
                      decoding_batches, num_heads, num_kv_heads, head_dim, cache_mode, page_size,
                      cache_stride_s, cache_stride_l, cache_stride_h, cache_stride_kv, cachestarts_stride_b,
                      num_token_ranges, workspace=None, attn_mask=None, mask_stride_s=0, mask_stride_h=0,
-                     stream=None, check=True):
+                     stage=0, stream=None, check=True):
     """Decode attention of sequences [0, decoding_batches); output fp16 [B_dec, Hq, D]."""
     p = DecodeParams()
     p.query = _ptr(query)
@@ -128,7 +128,7 @@ def decode_attention(query, output, cache, scale, cachestarts, kvstarts, *, attn
     p.num_token_ranges = num_token_ranges
     p.workspace = _ptr(workspace)
     p.workspace_size = 0 if workspace is None else workspace.numel() * workspace.element_size()
-    rc = _lib.lib().pmxhip_decode_attention(ctypes.byref(p), _stream(stream))
+    rc = _lib.lib().pmxhip_decode_attention_stage(ctypes.byref(p), stage, _stream(stream))
     if check and rc != RC_SUCCESS:
         raise PmxError(rc, "decode_attention")
     return rc
