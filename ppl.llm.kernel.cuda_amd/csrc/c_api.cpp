@@ -223,6 +223,13 @@ int pmxhip_decode_attention_stage(const pmxhip_decode_params* p, int32_t stage, 
         if (!aligned16(p->workspace)) return fail(PMXHIP_INVALID_VALUE, "decode_attention: workspace must be 16-byte aligned");
     }
 
+    {   // per-lane cache offsets are 32-bit: (tokens of one wave block) * stride_s + (kv heads of a group) * stride_h
+        const int wg_tok = pmxhip::decode_wg_tokens((int)p->head_dim, plan.kv_heads_per_group);
+        const double span = (double)wg_tok * (double)p->cache_stride_s + (double)plan.kv_heads_per_group * (double)p->cache_stride_h;
+        if (p->cache_stride_s < 0 || p->cache_stride_h < 0 || span >= 2147483648.0)
+            return fail(PMXHIP_UNSUPPORTED, "decode_attention: cache_stride_s/cache_stride_h too large for 32-bit lane offsets");
+    }
+
     pmxhip::DecodeLaunch a{};
     a.query = p->query;
     a.attn_mask = p->attn_mask;

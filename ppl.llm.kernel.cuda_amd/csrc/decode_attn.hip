@@ -34,16 +34,53 @@ namespace {
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kNegBig = -1.0e30f; // finite "no token yet" running max (log2 units)
-constexpr float kPShift = 14.0f;    // p = 2^(s - max + 14): keeps small p out of the fp16 subnormal range
 
 constexpr int kDecodeThreads = 256;
 constexpr int kDecodeWaves = kDecodeThreads / kWave;
-constexpr int kTB = 8; // tokens a slot handles per block
+constexpr int kTB = 4; // tokens a slot handles per block (= lanes of a quad)
+static_assert(kTB == 4, "the quad reduce-scatter and the explicit wait counts assume four tokens per block");
 
-struct RangeInfo {
-    int64_t total;   // T
-    int64_t per;     // tokens per range
-};
+// ---- hand-scheduled cache loads of the pipelined loop ---------------------------------------
+// The loads of the steady-state loop are issued through inline assembly and awaited with explicit
+// wait counts.  Written as plain C++ loads, the compiler's automatic wait-count placement reuses
+// staging registers for temporaries and then waits for loads issued only moments earlier, which
+// serialises the memory latency into every iteration.  Vector memory operations complete in issue
+// order, so "at most N still outstanding" identifies exactly which loads have landed.
+__device__ __forceinline__ void load_b128(u32x4& dst, uint32_t lane_off, const char* wave_base)
+{
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(dst) : "v"(lane_off), "s"(wave_base) : "memory");
+}
+__device__ __forceinline__ void load_b32(uint32_t& dst, uint32_t lane_off, const char* wave_base)
+{
+    asm volatile("global_load_dword %0, %1, %2" : "=&v"(dst) : "v"(lane_off), "s"(wave_base) : "memory");
+}
+// waits until at most N vector memory operations are outstanding; the values pass through the
+// statement so that no use of them can be scheduled before the wait
+template <int N>
+__device__ __forceinline__ void wait_loads(u32x4& a, uint32_t& b)
+{
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+// Waits for every outstanding load.  A register that is the target of an in-flight load must stay
+// allocated until a wait covers it, even when its value is never used (the redundant request of
+// the last block): passing it through this statement keeps it reserved, so that nothing else can
+// be placed in it and then be overwritten when the load lands.
+__device__ __forceinline__ void drain_loads(u32x4 (&q)[4], uint32_t (&sc)[4])
+{
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(q[0]), "+v"(q[1]), "+v"(q[2]), "+v"(q[3]), "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3]));
+}
+
+// value held by quad lane (lane ^ j), j in 0..3; j is a compile-time constant after unrolling
+__device__ __forceinline__ float quad_xor(float v, int j)
+{
+    switch (j) {
+        case 0: return v;
+        case 1: return dpp_f32<kDppXor1>(v);
+        case 2: return dpp_f32<kDppXor2>(v);
+        default: return dpp_f32<0x1B>(v); // quad_perm:[3,2,1,0]
+    }
+}
 
 // Tokens per range: equal shares rounded up to a whole number of workgroup
 // iterations, never below kMinTokensPerRange.  Shared by both kernels.
@@ -55,7 +92,7 @@ __device__ __forceinline__ int64_t tokens_per_range(int64_t total, int ranges, i
 }
 
 // first b in [0, n) with starts[b + 1] - starts[0] > g   (starts is non-decreasing)
-__device__ __forceinline__ int find_sequence(const int64_t* __restrict__ starts, int n, int64_t g)
+__device__ __forceinline__ int find_sequence(const_i64_ptr starts, int n, int64_t g)
 {
     const int64_t base = starts[0];
     int lo = 0, hi = n; // answer in [lo, hi]
@@ -69,14 +106,27 @@ __device__ __forceinline__ int find_sequence(const int64_t* __restrict__ starts,
 
 } // namespace
 
+// One block of kTB tokens for one slot: raw cache bytes as loaded, K and V staged separately.
+struct KBlock {
+    u32x4 q8[kTB];    // 16 int8 key channels per token
+    uint32_t sc[kTB]; // their two fp16 group scales
+    int pos;          // sequence position of the wave block's first token
+    int64_t boff;     // element offset of that token's row in the cache
+};
+struct VBlock {
+    u32x4 q8[kTB];
+    uint32_t sc[kTB];
+};
+
 // D: head dim (64, 96, 128, 256).  GT: query heads per kv head held in registers.
 template <int D, int GT, bool PAGED, bool MASK>
-__global__ __launch_bounds__(kDecodeThreads) void decode_attention_kernel(const DecodeLaunch a)
+__global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_attention_kernel(const DecodeLaunch a)
 {
     constexpr int LPS = (D == 64) ? 4 : (D == 256 ? 16 : 8); // lanes per slot
     constexpr int LPS_ACTIVE = D / 16;                        // 6 of 8 for D = 96
     constexpr int SPW = kWave / LPS;                          // slots per wave
     constexpr int NSLOT = SPW * kDecodeWaves;
+    constexpr bool kHandScheduled = GT <= 4; // inline-assembly loads with explicit wait counts in the steady-state loop
 
     __shared__ float sm_acc[NSLOT * D];
     __shared__ float sm_m[NSLOT];
@@ -87,6 +137,12 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_attention_kernel(const 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ls = lane % LPS;            // lane in slot -> channels [16*ls, 16*ls+16)
     const int slot = lane / LPS;          // slot in wave
+    // Token order inside a block is permuted per lane: register slot j of a lane holds token j ^ tp.
+    // With tp = (lane in quad) ^ (3 on odd quads) the cross-lane sum of the four partial logits needs
+    // no selects: slot k of a lane and slot k ^ 2 of its xor-2 partner are the same token, and so on
+    // down to one complete logit per lane (token tp); the mirror partners used across quads own the
+    // same token.  The probability of slot j's token is then found in quad lane (lane ^ j).
+    const int tp = (lane & 3) ^ ((lane & 4) ? 3 : 0);
     const bool lane_on = ls < LPS_ACTIVE;
     const int ch0 = (lane_on ? ls : 0) * 16;
 
@@ -102,23 +158,39 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_attention_kernel(const 
     const int g_first = blockIdx.z * GT; // first query head (within the kv head's group) of this pass
     const int G = (int)a.num_kv_repeats;
 
-    const int64_t kv_base = a.kvstarts[0];
-    const int64_t total = a.kvstarts[a.decoding_batches] - kv_base;
+    const const_i64_ptr kvstarts = as_constant(a.kvstarts);
+    const const_i64_ptr cachestarts = as_constant(a.cachestarts);
+    const int64_t kv_base = kvstarts[0];
+    const int64_t total = kvstarts[a.decoding_batches] - kv_base;
     const int64_t per = tokens_per_range(total, a.ranges, wg_tokens, a.min_tokens_per_range);
     const int64_t r0 = (int64_t)blockIdx.x * per;
     if (r0 >= total) return;
     const int64_t r1 = (r0 + per < total) ? r0 + per : total;
+#ifdef PMX_WG_TRACE
+    const unsigned long long trace_t0 = wall_clock64();
+#endif
 
-    const int8_t* __restrict__ cache = (const int8_t*)a.cache;
-    const half_t* __restrict__ scale = (const half_t*)a.scale;
-    const int64_t head_off = a.layer_idx * a.cache_stride_l + (int64_t)kvh * a.cache_stride_h + ch0;
+    // Addressing: a wave-uniform 64-bit base per block (scalar registers) plus a 32-bit per-lane
+    // offset that never changes: (token in block) * stride_s + (head in group) * stride_h + channel.
+    const int64_t group_off = a.layer_idx * a.cache_stride_l + (int64_t)(blockIdx.y * kvhb) * a.cache_stride_h;
+    uint32_t voff[kTB];
+#pragma unroll
+    for (int j = 0; j < kTB; ++j)
+        voff[j] = (uint32_t)((int64_t)((j ^ tp) * tpl + tsub) * a.cache_stride_s + (int64_t)head_local * a.cache_stride_h + ch0);
+    uint32_t voff_sc[kTB]; // the same offsets in the scale tensor: one fp16 scale per 8 channels
+#pragma unroll
+    for (int j = 0; j < kTB; ++j) voff_sc[j] = voff[j] >> 2;
+    const char* const cache_k = (const char*)a.cache + group_off;
+    const char* const cache_v = cache_k + a.cache_stride_kv;
+    const char* const scale_k = (const char*)a.scale + (group_off >> 3) * 2;
+    const char* const scale_v = scale_k + (a.cache_stride_kv >> 3) * 2;
     const float logit_scale = a.attn_scale * kLog2e;
 
-    int b = find_sequence(a.kvstarts, (int)a.decoding_batches, r0);
+    int b = find_sequence(kvstarts, (int)a.decoding_batches, r0);
     for (; b < a.decoding_batches; ++b) {
-        const int64_t s_beg = a.kvstarts[b] - kv_base;
+        const int64_t s_beg = kvstarts[b] - kv_base;
         if (s_beg >= r1) break;
-        const int64_t s_end = a.kvstarts[b + 1] - kv_base;
+        const int64_t s_end = kvstarts[b + 1] - kv_base;
         const int64_t len = s_end - s_beg;
         // piece [pa, pe) in sequence coordinates
         const int64_t pa = (r0 > s_beg ? r0 : s_beg) - s_beg;
@@ -126,7 +198,11 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_attention_kernel(const 
         if (pe <= pa) continue;
 
         // ---- query heads of this kv head into registers (packed halves) ----
+        // qb[g][i] = -1152 * (sum of the 8 query channels of group i): the int8 -> half conversion
+        // leaves keys biased by +1152 (see device_common.h); starting the dot product at qb removes
+        // the bias exactly where it is cheapest.
         half2_t q[GT][8];
+        float qb[GT][2];
 #pragma unroll
         for (int g = 0; g < GT; ++g) {
             const int gi = g_first + g;
@@ -135,141 +211,305 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_attention_kernel(const 
             const u32x4* qp = (const u32x4*)((const half_t*)a.query + (int64_t)b * a.query_stride_s + (int64_t)h * D + ch0);
             u32x4 lo = qp[0], hi = qp[1];
             if (!on) { lo = u32x4{0, 0, 0, 0}; hi = lo; }
+            float s0 = 0.f, s1 = 0.f;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 q[g][i] = bitcast<half2_t>(lo[i]);
                 q[g][4 + i] = bitcast<half2_t>(hi[i]);
+                s0 += (float)q[g][i].x + (float)q[g][i].y;
+                s1 += (float)q[g][4 + i].x + (float)q[g][4 + i].y;
             }
+            qb[g][0] = -1152.f * s0;
+            qb[g][1] = -1152.f * s1;
         }
 
         float m_run[GT], l_run[GT], acc[GT][16];
 #pragma unroll
         for (int g = 0; g < GT; ++g) {
             m_run[g] = kNegBig;
-            l_run[g] = 0.f;
+            l_run[g] = 0.f; // partial: this lane's own tokens only
 #pragma unroll
             for (int c = 0; c < 16; ++c) acc[g][c] = 0.f;
         }
 
         const int64_t table_base = PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b;
-        const int64_t seq_row0 = PAGED ? 0 : a.cachestarts[b];
+        const int64_t seq_row0 = PAGED ? 0 : cachestarts[b];
         const half_t* mask_row = nullptr;
-        if (MASK) mask_row = (const half_t*)a.attn_mask + (int64_t)b * a.mask_stride_s + a.kvstarts[b];
+        if (MASK) mask_row = (const half_t*)a.attn_mask + (int64_t)b * a.mask_stride_s + kvstarts[b];
+        // sequence-relative positions fit 32 bits
+        const int pa32 = (int)pa, pe32 = (int)pe;
+        const int last_page = (pe32 - 1) >> 7;
 
-        // iterations are aligned to wg_tokens in sequence coordinates so that a
-        // wave's block never straddles a page
-        for (int64_t it0 = pa / wg_tokens * wg_tokens; it0 < pe; it0 += wg_tokens) {
-            const int64_t wave0 = it0 + (int64_t)wave * wave_tokens;
-            if (wave0 >= pe || wave0 + wave_tokens <= pa) continue; // wave-uniform
-            int64_t row_base;
-            if (PAGED) {
-                row_base = a.cachestarts[table_base + (wave0 >> 7)] + (wave0 & (kPage - 1));
-            } else {
-                row_base = seq_row0 + wave0;
+        // Page table entries are read one page ahead with scalar loads, so that no block waits
+        // for its row base: `page_row` belongs to page `page_idx`, `next_row` to the page after it.
+        int page_idx = -2;
+        int64_t page_row = 0, next_row = 0;
+        auto row_base_of = [&](int pos) -> int64_t {
+            if (!PAGED) return seq_row0 + pos;
+            const int pg = pos >> 7;
+            if (pg != page_idx) {
+                page_row = (pg == page_idx + 1) ? next_row : cachestarts[table_base + pg];
+                page_idx = pg;
+                const int nx = pg + 1 <= last_page ? pg + 1 : last_page;
+                next_row = cachestarts[table_base + nx];
             }
+            return page_row + (pos & (kPage - 1));
+        };
 
-            u32x4 kq[kTB], vq[kTB];
-            uint32_t ks[kTB], vs[kTB];
-            bool valid[kTB];
+        // ---- loads of one wave block (positions pos .. pos + wave_tokens): K with its scales, V with its scales.
+        // FULL blocks lie inside the piece; in a partial block the tokens outside the piece are redirected
+        // to a token inside it (the load is harmless, the logit is masked later) ----
+        auto lane_off = [&](int pos, int j) -> uint32_t {
+            const int t = pos + (j ^ tp) * tpl + tsub;
+            const int tc = t < pa32 ? pa32 : (t >= pe32 ? pe32 - 1 : t);
+            return (uint32_t)((int64_t)(tc - pos) * a.cache_stride_s + (int64_t)head_local * a.cache_stride_h + ch0);
+        };
+        // steady-state versions: full blocks only, inline-assembly loads in a fixed order
+        // (token 0: 16 bytes then scales, token 1: ..., 8 operations per half-block)
+        auto issue_k_fast = [&](KBlock& kb, int pos) {
+            kb.pos = pos;
+            const int64_t boff = row_base_of(pos) * a.cache_stride_s;
+            kb.boff = boff;
+            const char* bk = cache_k + boff;
+            const char* sk = scale_k + (boff >> 3) * 2;
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
-                const int tin = j * tpl + tsub; // token within the wave block
-                const int64_t t = wave0 + tin;
-                valid[j] = (t >= pa) && (t < pe);
-                // clamp invalid tokens onto a valid one of this piece: the load is harmless, the logit is masked
-                int64_t tc = t < pa ? pa : (t >= pe ? pe - 1 : t);
-                const int64_t row = row_base + (tc - wave0);
-                const int64_t off = row * a.cache_stride_s + head_off;
-                kq[j] = *(const u32x4*)(cache + off);
-                vq[j] = *(const u32x4*)(cache + off + a.cache_stride_kv);
-                ks[j] = *(const uint32_t*)(scale + (off >> 3));
-                vs[j] = *(const uint32_t*)(scale + ((off + a.cache_stride_kv) >> 3));
+                load_b128(kb.q8[j], voff[j], bk);
+                load_b32(kb.sc[j], voff_sc[j], sk);
             }
-
-            // ---- logits: s[g][j] in log2 units ----
-            float s[GT][kTB];
+        };
+        auto issue_v_fast = [&](VBlock& vb, int64_t boff) {
+            const char* bv = cache_v + boff;
+            const char* sv = scale_v + (boff >> 3) * 2;
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
+                load_b128(vb.q8[j], voff[j], bv);
+                load_b32(vb.sc[j], voff_sc[j], sv);
+            }
+        };
+        auto issue_k = [&](KBlock& kb, int pos, bool full) {
+            kb.pos = pos;
+            const int64_t boff = row_base_of(pos) * a.cache_stride_s;
+            kb.boff = boff;
+            const char* bk = cache_k + boff;
+            const char* sk = scale_k + (boff >> 3) * 2;
+#pragma unroll
+            for (int j = 0; j < kTB; ++j) {
+                const uint32_t off = full ? voff[j] : lane_off(pos, j);
+                kb.q8[j] = *(const u32x4*)(bk + off);
+                kb.sc[j] = *(const uint32_t*)(sk + (off >> 2));
+            }
+        };
+        auto issue_v = [&](VBlock& vb, int pos, int64_t boff, bool full) {
+            const char* bv = cache_v + boff;
+            const char* sv = scale_v + (boff >> 3) * 2;
+#pragma unroll
+            for (int j = 0; j < kTB; ++j) {
+                const uint32_t off = full ? voff[j] : lane_off(pos, j);
+                vb.q8[j] = *(const u32x4*)(bv + off);
+                vb.sc[j] = *(const uint32_t*)(sv + (off >> 2));
+            }
+        };
+
+        // ---- QK^T and softmax of one block: leaves this lane's probability (token ql) in p[g] ----
+        float p[GT];
+        auto logits_softmax = [&](KBlock& kb, bool full, bool fast) {
+            // logits, still partial over the slot's lanes: part[g][j], log2 units
+            float part[GT][kTB];
+#pragma unroll
+            for (int j = 0; j < kTB; ++j) {
+                if (fast) {
+                    // outstanding and younger than token j of this half-block: the rest of this half-block,
+                    // and the two half-blocks requested after it
+                    if (j == 0) wait_loads<22>(kb.q8[0], kb.sc[0]);
+                    if (j == 1) wait_loads<20>(kb.q8[1], kb.sc[1]);
+                    if (j == 2) wait_loads<18>(kb.q8[2], kb.sc[2]);
+                    if (j == 3) wait_loads<16>(kb.q8[3], kb.sc[3]);
+                }
                 half2_t kh[8];
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
-                    const uint32_t f = kq[j][w] ^ kFlipSigns;
-                    kh[2 * w] = cvt_bytes01(f);
-                    kh[2 * w + 1] = cvt_bytes23(f);
+                    const uint32_t f = kb.q8[j][w] ^ kFlipSigns;
+                    kh[2 * w] = bitcast<half2_t>(__builtin_amdgcn_perm(kExpBytes, f, 0x04010400u));     // 1152 + x
+                    kh[2 * w + 1] = bitcast<half2_t>(__builtin_amdgcn_perm(kExpBytes, f, 0x04030402u));
                 }
-                const half2_t sc = bitcast<half2_t>(ks[j]);
+                const half2_t sc = bitcast<half2_t>(kb.sc[j]);
                 const float s0 = (float)sc.x * logit_scale;
                 const float s1 = (float)sc.y * logit_scale;
 #pragma unroll
                 for (int g = 0; g < GT; ++g) {
-                    float d0 = 0.f, d1 = 0.f;
+                    float d0 = qb[g][0], d1 = qb[g][1];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         d0 = dot2(q[g][i], kh[i], d0);
                         d1 = dot2(q[g][4 + i], kh[4 + i], d1);
                     }
-                    float part = d0 * s0 + d1 * s1;
-                    part = group_sum<LPS>(part);
-                    if (MASK) {
-                        const int h = kvh * G + g_first + g;
-                        if (g_first + g < G && valid[j]) {
-                            const int64_t t = wave0 + j * tpl + tsub;
-                            part += (float)mask_row[(int64_t)h * a.mask_stride_h + t] * kLog2e;
-                        }
-                    }
-                    s[g][j] = valid[j] ? part : -INFINITY;
+                    part[g][j] = __builtin_fmaf(d1, s1, d0 * s0);
                 }
             }
 
-            // ---- online softmax update, probabilities packed as halves ----
-            half2_t p[GT][kTB / 2];
+            // reduce-scatter inside the quad (slot k here and slot k ^ 2 of the xor-2 partner are the
+            // same token), then all-reduce across the quads of the slot: the lane ends with the complete
+            // logit of token tp
+            bool rescale = false;
+            float m_new[GT];
 #pragma unroll
             for (int g = 0; g < GT; ++g) {
-                float mx = s[g][0];
-#pragma unroll
-                for (int j = 1; j < kTB; ++j) mx = fmaxf(mx, s[g][j]);
-                const float m_new = fmaxf(m_run[g], mx);
-                const float alpha = __builtin_amdgcn_exp2f(m_run[g] - m_new);
-                m_run[g] = m_new;
-                const float bias = kPShift - m_new;
-                float lsum = 0.f;
-#pragma unroll
-                for (int j = 0; j < kTB; j += 2) {
-                    const float p0 = __builtin_amdgcn_exp2f(s[g][j] + bias);
-                    const float p1 = __builtin_amdgcn_exp2f(s[g][j + 1] + bias);
-                    const half2_t ph = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(p0, p1));
-                    p[g][j / 2] = ph;
-                    const half2_t ones = {(half_t)1.0f, (half_t)1.0f};
-                    lsum = dot2(ph, ones, lsum); // the sum uses the rounded p, like the PV product
+                const float u0 = part[g][0] + dpp_f32<kDppXor2>(part[g][2]);
+                const float u1 = part[g][1] + dpp_f32<kDppXor2>(part[g][3]);
+                float logit = u0 + dpp_f32<kDppXor1>(u1);
+                if (LPS >= 8) logit += dpp_f32<kDppHalfMirror>(logit);
+                if (LPS >= 16) logit += dpp_f32<kDppMirror>(logit);
+                if (MASK || !full) {
+                    const int tk = kb.pos + tp * tpl + tsub;
+                    const bool ok = tk >= pa32 && tk < pe32;
+                    if (MASK && ok && g_first + g < G) {
+                        const int h = kvh * G + g_first + g;
+                        logit += (float)mask_row[(int64_t)h * a.mask_stride_h + tk] * kLog2e;
+                    }
+                    if (!ok) logit = -INFINITY;
                 }
-                l_run[g] = l_run[g] * alpha + lsum;
-#pragma unroll
-                for (int c = 0; c < 16; ++c) acc[g][c] *= alpha;
+                // block max over the quad (= over the block's tokens)
+                float mx = fmaxf(logit, dpp_f32<kDppXor1>(logit));
+                mx = fmaxf(mx, dpp_f32<kDppXor2>(mx));
+                m_new[g] = fmaxf(m_run[g], mx);
+                rescale = rescale || (m_new[g] > m_run[g]);
+                p[g] = __builtin_amdgcn_exp2f(logit - m_new[g]);
             }
-
-            // ---- PV: token pairs (j, j+1) share one dot2 per channel ----
-#pragma unroll
-            for (int j = 0; j < kTB; j += 2) {
-                const u32x4 va = vq[j], vb = vq[j + 1];
-                // scale pairs: (group0 of token j, group0 of token j+1), same for group1
-                const half2_t sc0 = bitcast<half2_t>(__builtin_amdgcn_perm(vs[j + 1], vs[j], 0x05040100u));
-                const half2_t sc1 = bitcast<half2_t>(__builtin_amdgcn_perm(vs[j + 1], vs[j], 0x07060302u));
-                half2_t vh[16];
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    const half2_t sc = (w < 2) ? sc0 : sc1;
-                    vh[4 * w + 0] = cvt_byte_pair<0>(va[w], vb[w]) * sc;
-                    vh[4 * w + 1] = cvt_byte_pair<1>(va[w], vb[w]) * sc;
-                    vh[4 * w + 2] = cvt_byte_pair<2>(va[w], vb[w]) * sc;
-                    vh[4 * w + 3] = cvt_byte_pair<3>(va[w], vb[w]) * sc;
-                }
+            if (__builtin_amdgcn_ballot_w64(rescale) != 0) { // wave-uniform and rare: a running max moved
 #pragma unroll
                 for (int g = 0; g < GT; ++g) {
+                    const float al = __builtin_amdgcn_exp2f(m_run[g] - m_new[g]);
+                    m_run[g] = m_new[g];
+                    l_run[g] *= al;
 #pragma unroll
-                    for (int c = 0; c < 16; ++c) acc[g][c] = dot2(p[g][j / 2], vh[c], acc[g][c]);
+                    for (int c = 0; c < 16; ++c) acc[g][c] *= al;
                 }
             }
+#pragma unroll
+            for (int g = 0; g < GT; ++g) l_run[g] += p[g];
+        };
+
+        // ---- PV of one block: int8 values converted straight to fp32 (exact), fp32 weights p * scale,
+        // fp32 multiply-accumulate in the two-source form (v_fmac_f32), which issues at twice the rate
+        // of the three-source and packed forms on this chip ----
+        auto accumulate_pv = [&](VBlock& vb, bool fast) {
+#pragma unroll
+            for (int j = 0; j < kTB; ++j) {
+                if (fast) {
+                    if (j == 0) wait_loads<22>(vb.q8[0], vb.sc[0]);
+                    if (j == 1) wait_loads<20>(vb.q8[1], vb.sc[1]);
+                    if (j == 2) wait_loads<18>(vb.q8[2], vb.sc[2]);
+                    if (j == 3) wait_loads<16>(vb.q8[3], vb.sc[3]);
+                }
+                float x[16];
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    x[4 * w + 0] = byte_to_f32<0>(vb.q8[j][w]);
+                    x[4 * w + 1] = byte_to_f32<1>(vb.q8[j][w]);
+                    x[4 * w + 2] = byte_to_f32<2>(vb.q8[j][w]);
+                    x[4 * w + 3] = byte_to_f32<3>(vb.q8[j][w]);
+                }
+                const half2_t sc = bitcast<half2_t>(vb.sc[j]);
+                const float sv0 = (float)sc.x, sv1 = (float)sc.y;
+#pragma unroll
+                for (int g = 0; g < GT; ++g) {
+                    const float pj = quad_xor(p[g], j); // slot j holds token j ^ tp, whose probability is in quad lane (lane ^ j)
+                    const float w0 = pj * sv0, w1 = pj * sv1;
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) {
+                        acc[g][c] = __builtin_fmaf(w0, x[c], acc[g][c]);
+                        acc[g][8 + c] = __builtin_fmaf(w1, x[8 + c], acc[g][8 + c]);
+                    }
+                }
+            }
+        };
+
+        // Wave blocks of this piece are aligned to wg_tokens in sequence coordinates, so that a block
+        // never straddles a page.  At most the first and the last block of a wave are partial; they take
+        // the simple path.  The full blocks in between run software-pipelined: K of block i+1 is
+        // requested before the logits of block i, V of block i+1 before the PV of block i, so that three
+        // half-blocks of cache bytes are in registers or in flight at any time.
+        auto simple_block = [&](int pos) {
+            KBlock kx;
+            VBlock vx;
+            issue_k(kx, pos, false);
+            issue_v(vx, pos, kx.boff, false);
+            logits_softmax(kx, false, false);
+            accumulate_pv(vx, false);
+        };
+        int pos = (int)(pa / wg_tokens * wg_tokens) + wave * wave_tokens;
+        if (pos + wave_tokens <= pa32) pos += wg_tokens;
+        if (pos < pe32 && pos < pa32) {
+            simple_block(pos);
+            pos += wg_tokens;
         }
+        int n_full = (pos + wave_tokens <= pe32) ? (pe32 - wave_tokens - pos) / wg_tokens + 1 : 0;
+        if (kHandScheduled && n_full > 0) {
+            // Every block requests the next one unconditionally (the last re-requests itself): with no
+            // branch around the loads, and no register copies between stages (two named buffer pairs,
+            // loop unrolled by two), the hardware wait counts stay exact.
+            KBlock ka, kb;
+            VBlock va, vb;
+            __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): the explicit wait counts below assume that only the loop's own loads are in flight
+            issue_k_fast(ka, pos);
+            issue_v_fast(va, ka.boff);
+            // the first block has landed before the loop is entered: any register copy the compiler
+            // places on the loop's entry edge then copies data, not a register still being loaded
+            drain_loads(ka.q8, ka.sc);
+            drain_loads(va.q8, va.sc);
+            for (int i = 0;;) {
+                // even block: consume (ka, va), request (kb, vb)
+                int npos = pos + (i + 1 < n_full ? wg_tokens : 0);
+                issue_k_fast(kb, npos);
+                logits_softmax(ka, true, true);
+                issue_v_fast(vb, kb.boff);
+                accumulate_pv(va, true);
+                pos = npos;
+                if (++i == n_full) break;
+                // odd block: consume (kb, vb), request (ka, va)
+                npos = pos + (i + 1 < n_full ? wg_tokens : 0);
+                issue_k_fast(ka, npos);
+                logits_softmax(kb, true, true);
+                issue_v_fast(va, ka.boff);
+                accumulate_pv(vb, true);
+                pos = npos;
+                if (++i == n_full) break;
+            }
+            // drain the last (redundant) requests; all four staging buffers stay reserved until then
+            drain_loads(ka.q8, ka.sc);
+            drain_loads(kb.q8, kb.sc);
+            drain_loads(va.q8, va.sc);
+            drain_loads(vb.q8, vb.sc);
+            pos += wg_tokens;
+        }
+        if (!kHandScheduled && n_full > 0) {
+            // GT = 8 does not fit the register file without moving values to accumulation registers,
+            // which is not compatible with loads that land behind the compiler's back: this variant
+            // leaves load scheduling to the compiler.
+            KBlock ka, kb;
+            VBlock va, vb;
+            issue_k(ka, pos, true);
+            issue_v(va, pos, ka.boff, true);
+            for (int i = 0;;) {
+                int npos = pos + (i + 1 < n_full ? wg_tokens : 0);
+                issue_k(kb, npos, true);
+                logits_softmax(ka, true, false);
+                issue_v(vb, npos, kb.boff, true);
+                accumulate_pv(va, false);
+                pos = npos;
+                if (++i == n_full) break;
+                npos = pos + (i + 1 < n_full ? wg_tokens : 0);
+                issue_k(ka, npos, true);
+                logits_softmax(kb, true, false);
+                issue_v(va, npos, ka.boff, true);
+                accumulate_pv(vb, false);
+                pos = npos;
+                if (++i == n_full) break;
+            }
+            pos += wg_tokens;
+        }
+        if (pos < pe32) simple_block(pos);
 
         // ---- merge the slots of each kv head through LDS, one query head at a time ----
         const bool whole = (pa == 0) && (pe == len);
@@ -278,6 +518,9 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_attention_kernel(const 
         const int dup = NSLOT / kvhb; // slots per kv head
 #pragma unroll
         for (int g = 0; g < GT; ++g) {
+            // exp-sum of the slot = sum over the quad lanes' partial sums
+            float lq = l_run[g] + dpp_f32<kDppXor1>(l_run[g]);
+            lq += dpp_f32<kDppXor2>(lq);
             __syncthreads();
             if (lane_on) {
 #pragma unroll
@@ -286,7 +529,7 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_attention_kernel(const 
                 }
                 if (ls == 0) {
                     sm_m[gslot] = m_run[g];
-                    sm_l[gslot] = l_run[g];
+                    sm_l[gslot] = lq;
                 }
             }
             __syncthreads();
@@ -324,6 +567,19 @@ __global__ __launch_bounds__(kDecodeThreads) void decode_attention_kernel(const 
         }
         __syncthreads();
     }
+#ifdef PMX_WG_TRACE
+    if (tid == 0) {
+        unsigned long long* tr = (unsigned long long*)(a.partial_ml + (int64_t)(a.ranges + a.decoding_batches) * a.num_heads * 2);
+        const int64_t wg = blockIdx.x + (int64_t)gridDim.x * (blockIdx.y + (int64_t)gridDim.y * blockIdx.z);
+        unsigned xcc = 0, hwid = 0;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+        tr[wg * 4 + 0] = trace_t0;
+        tr[wg * 4 + 1] = wall_clock64();
+        tr[wg * 4 + 2] = xcc;
+        tr[wg * 4 + 3] = hwid;
+    }
+#endif
 }
 
 // One workgroup per (sequence, query head): merges the pieces the decode kernel

@@ -85,9 +85,30 @@ __device__ __forceinline__ half2_t cvt_byte_pair(uint32_t a, uint32_t b)
     return pk_sub_1152(placed ^ 0x64806480u);
 }
 
+// signed byte K of a word -> fp32, one SDWA conversion (sign-extending byte select)
+template <int K>
+__device__ __forceinline__ float byte_to_f32(uint32_t w)
+{
+    float r;
+    if (K == 0) asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(r) : "v"(w));
+    if (K == 1) asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1" : "=v"(r) : "v"(w));
+    if (K == 2) asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(r) : "v"(w));
+    if (K == 3) asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3" : "=v"(r) : "v"(w));
+    return r;
+}
+
 __device__ __forceinline__ float dot2(half2_t a, half2_t b, float c)
 {
     return __builtin_amdgcn_fdot2(a, b, c, false);
+}
+
+// Index arrays (kvstarts, cachestarts) are read-only for the whole launch and are read at
+// wave-uniform addresses: viewing them through the constant address space lets the compiler use
+// scalar loads (scalar cache, no vector registers, no vector wait count) for them.
+typedef const int64_t __attribute__((address_space(4)))* const_i64_ptr;
+__device__ __forceinline__ const_i64_ptr as_constant(const int64_t* p)
+{
+    return (const_i64_ptr)(uintptr_t)p;
 }
 
 // ---- token addressing ----------------------------------------------------------

@@ -1,5 +1,322 @@
-// placeholder until the MFMA tile lands
+// Multi-query-token (chunked prefill) attention over the int8 group-8 KV cache
+// for gfx950, on MFMA.
+//
+// Semantics follow the reference's prefill stage
+// (src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/kernel.cu:2127-2179, which
+// calls flash_attn2_paged_fmha): query rows seqstarts[b]..seqstarts[b+1], kv length
+// kvstarts[b+1]-kvstarts[b], K/V from the int8 cache through cachestarts, dequantised
+// as fp16(int8) * fp16(scale) (flash_attn2/src/utils.h:397-436), causal mask aligned
+// bottom-right: row i sees columns < i + 1 + kvlen - qlen (flash_attn2/src/mask.h:186).
+//
+// Decomposition (this file's own):
+//   * one workgroup (4 waves) = one kv head of one sequence x a tile of query
+//     positions x ALL query heads of that kv head.  The (position, head) pairs
+//     are the 128 "columns" of the tile, 32 per wave, so a dequantised K/V tile
+//     is shared by every query head of the group.
+//   * K/V tiles of 64 tokens are dequantised int8 -> fp16 into LDS once per
+//     workgroup; raw bytes of the next tile are prefetched into registers while
+//     the current tile is computed.
+//   * S^T = K Q^T (tokens are MFMA rows, columns stay columns): a lane then owns
+//     one column, so the softmax max/sum are register-local apart from one
+//     exchange between the two half-waves, and the S^T accumulator layout is
+//     already the B-operand layout of O^T = V^T P^T -- no shuffle between the
+//     two MFMA stages.  V is stored transposed in LDS with tokens permuted to
+//     match that layout.
+//   * v_mfma_f32_32x32x16_f16, fp32 accumulate, base-2 online softmax.
+#include "device_common.h"
 #include "launch_params.h"
+
 namespace pmxhip {
-int launch_prefill(const PrefillLaunch&, hipStream_t) { return 1; }
+
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kPrefillThreads = 256;
+constexpr int kBN = 64;        // kv tokens per tile
+constexpr int kCols = 128;     // (position, head) columns per workgroup
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kNegBig = -1.0e30f;
+constexpr float kPShift = 14.0f;
+
+// position of token offset o (0..15) inside its 16-token group of the transposed V tile:
+// token bits (a, h, r1, r0) -> position bits (h, a, r1, r0)
+__device__ __forceinline__ int vt_pos16(int o) { return ((o & 4) << 1) | ((o & 8) >> 1) | (o & 3); }
+
+} // namespace
+
+template <int D, bool PAGED>
+__global__ __launch_bounds__(kPrefillThreads) void prefill_attention_kernel(const PrefillLaunch a)
+{
+    constexpr int KSTEPS = D / 16;          // MFMA k-steps over channels for S
+    constexpr int CB = D / 32;              // 32-channel blocks of O^T
+    constexpr int GPT = D / 8;              // quantisation groups per token row
+    constexpr int K_STRIDE = D + 8;         // halves per K row in LDS (+16 B: conflict-free b128 reads)
+    constexpr int V_STRIDE = kBN + 8;       // halves per V^T row in LDS
+    constexpr int K_UNITS = kBN * GPT / kPrefillThreads;  // (token, group) units per thread
+    constexpr int V_THREADS = (kBN / 4) * GPT;            // threads with a (token quad, group) unit
+
+    // K is kept as an unevaluated sum hi + lo of two halves: hi = fp16(int8 * scale) and
+    // lo = the rounding error of that product (exact, from one fused multiply-add), so that
+    // q.k carries no fp16 rounding of the dequantised key.  With a single rounded copy a
+    // 2^-12 relative error on |q_c k_c| ~ 1e3 (outlier channels) moves logits by ~1e-2.
+    __shared__ __attribute__((aligned(16))) half_t sK[kBN * K_STRIDE];
+    __shared__ __attribute__((aligned(16))) half_t sKlo[kBN * K_STRIDE];
+    __shared__ __attribute__((aligned(16))) half_t sV[D * V_STRIDE];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int hh = lane >> 5;   // half-wave
+    const int l32 = lane & 31;
+
+    const int b = blockIdx.y;
+    const int kvh = blockIdx.z;
+    const int G = (int)(a.num_heads / a.num_kv_heads);
+    const int ppw = kCols / G > 0 ? kCols / G : 1; // query positions per workgroup
+    const int64_t q_row0 = a.seqstarts[b];
+    const int qlen = (int)(a.seqstarts[b + 1] - q_row0);
+    const int kvlen = (int)(a.kvstarts[b + 1] - a.kvstarts[b]);
+    const int p0 = blockIdx.x * ppw;
+    if (p0 >= qlen) return;
+
+    // ---- this lane's column ----
+    const int col = wave * 32 + l32;
+    const int pos = p0 + col / G;
+    const int g = col % G;
+    const bool col_on = (col < ppw * G) && (pos < qlen);
+    const int pos_c = pos < qlen ? pos : qlen - 1;
+    const int h = kvh * G + (col < ppw * G ? g : 0);
+    int lim = kvlen;                                   // this column attends tokens [0, lim)
+    if (a.is_causal) {
+        lim = pos_c + 1 + kvlen - qlen;
+        lim = lim < 0 ? 0 : (lim > kvlen ? kvlen : lim);
+    }
+    if (!col_on) lim = 0;
+    // tokens the workgroup must walk: the largest limit of its columns
+    int last_pos = p0 + ppw - 1;
+    if (last_pos > qlen - 1) last_pos = qlen - 1;
+    int wg_lim = kvlen;
+    if (a.is_causal) {
+        wg_lim = last_pos + 1 + kvlen - qlen;
+        wg_lim = wg_lim < 0 ? 0 : (wg_lim > kvlen ? kvlen : wg_lim);
+    }
+    const int n_tiles = (wg_lim + kBN - 1) / kBN;
+
+    // ---- Q fragments: B operand of S^T = K Q^T; lane holds Q[col][16 s + 8 hh .. +8] ----
+    f16x8 qf[KSTEPS];
+    {
+        const half_t* qp = (const half_t*)a.query + (q_row0 + pos_c) * a.query_stride_s + (int64_t)h * D + 8 * hh;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) qf[s] = *(const f16x8*)(qp + 16 * s);
+    }
+
+    f32x16 o_acc[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o_acc[cb][i] = 0.f;
+    float m_run = kNegBig, l_run = 0.f;
+    const float sm_scale = a.attn_scale * kLog2e;
+
+    // ---- global -> register staging of one tile's raw bytes ----
+    const int8_t* __restrict__ cache = (const int8_t*)a.cache;
+    const half_t* __restrict__ scale = (const half_t*)a.scale;
+    const int64_t head_off = a.layer_idx * a.cache_stride_l + (int64_t)kvh * a.cache_stride_h;
+    const int64_t table_base = PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b;
+
+    const int k_g = tid % GPT;           // channel group of this thread's K units
+    const int k_t0 = tid / GPT;          // first token; further units are kPrefillThreads / GPT tokens apart
+    const int v_g = tid % GPT;
+    const int v_q = tid / GPT;           // token quad (tokens 4 v_q .. 4 v_q + 3)
+    const bool v_on = tid < V_THREADS;
+
+    u32x2 k_raw[K_UNITS];
+    half_t k_sc[K_UNITS];
+    u32x2 v_raw[4];
+    half_t v_sc[4];
+
+    auto token_off = [&](int t) -> int64_t {
+        // row of token t (clamped into the sequence), times the token stride, plus the head offset
+        int tc = t < kvlen ? t : kvlen - 1;
+        if (tc < 0) tc = 0;
+        int64_t row;
+        if (PAGED) row = a.cachestarts[table_base + (tc >> 7)] + (tc & (kPage - 1));
+        else row = a.cachestarts[table_base] + tc;
+        return row * a.cache_stride_s + head_off;
+    };
+    auto load_tile = [&](int tile) {
+        const int t_base = tile * kBN;
+#pragma unroll
+        for (int u = 0; u < K_UNITS; ++u) {
+            const int64_t off = token_off(t_base + k_t0 + u * (kPrefillThreads / GPT)) + 8 * k_g;
+            k_raw[u] = *(const u32x2*)(cache + off);
+            k_sc[u] = scale[off >> 3];
+        }
+        if (v_on) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t off = token_off(t_base + 4 * v_q + r) + a.cache_stride_kv + 8 * v_g;
+                v_raw[r] = *(const u32x2*)(cache + off);
+                v_sc[r] = scale[off >> 3];
+            }
+        }
+    };
+    auto store_tile = [&]() {
+        // K: 8 halves of one (token, group) -> one 128-bit LDS store
+#pragma unroll
+        for (int u = 0; u < K_UNITS; ++u) {
+            const half2_t sc = {k_sc[u], k_sc[u]};
+            const uint32_t f0 = k_raw[u][0] ^ kFlipSigns, f1 = k_raw[u][1] ^ kFlipSigns;
+            const half2_t x0 = cvt_bytes01(f0), x1 = cvt_bytes23(f0), x2 = cvt_bytes01(f1), x3 = cvt_bytes23(f1);
+            const half2_t h0 = x0 * sc, h1 = x1 * sc, h2 = x2 * sc, h3 = x3 * sc;
+            u32x4 w, wl;
+            w[0] = bitcast<uint32_t>(h0);
+            w[1] = bitcast<uint32_t>(h1);
+            w[2] = bitcast<uint32_t>(h2);
+            w[3] = bitcast<uint32_t>(h3);
+            wl[0] = bitcast<uint32_t>(__builtin_elementwise_fma(x0, sc, -h0));
+            wl[1] = bitcast<uint32_t>(__builtin_elementwise_fma(x1, sc, -h1));
+            wl[2] = bitcast<uint32_t>(__builtin_elementwise_fma(x2, sc, -h2));
+            wl[3] = bitcast<uint32_t>(__builtin_elementwise_fma(x3, sc, -h3));
+            const int t = k_t0 + u * (kPrefillThreads / GPT);
+            *(u32x4*)&sK[t * K_STRIDE + 8 * k_g] = w;
+            *(u32x4*)&sKlo[t * K_STRIDE + 8 * k_g] = wl;
+        }
+        // V: four tokens of one channel -> one 64-bit LDS store into the transposed tile
+        if (v_on) {
+            const half2_t s01 = {v_sc[0], v_sc[1]}, s23 = {v_sc[2], v_sc[3]};
+            const int grp = v_q >> 2;
+            const int posv = 16 * grp + vt_pos16(4 * (v_q & 3));
+#pragma unroll
+            for (int e8 = 0; e8 < 8; ++e8) {
+                const int e = (e8 + v_g) & 7; // rotate the channel order per lane: spreads LDS banks
+                // byte e of each of the four tokens; the byte index is a run-time value, so the
+                // v_perm selector is built instead of templated
+                const uint32_t sel = 0x0c000c00u | (uint32_t)(e & 3) | ((uint32_t)(4 + (e & 3)) << 16);
+                const bool upper = e >= 4;
+                const uint32_t w0 = upper ? v_raw[0][1] : v_raw[0][0], w1 = upper ? v_raw[1][1] : v_raw[1][0];
+                const uint32_t w2 = upper ? v_raw[2][1] : v_raw[2][0], w3 = upper ? v_raw[3][1] : v_raw[3][0];
+                const half2_t lo = pk_sub_1152(__builtin_amdgcn_perm(w1, w0, sel) ^ 0x64806480u);
+                const half2_t hi = pk_sub_1152(__builtin_amdgcn_perm(w3, w2, sel) ^ 0x64806480u);
+                u32x2 out;
+                out[0] = bitcast<uint32_t>(lo * s01);
+                out[1] = bitcast<uint32_t>(hi * s23);
+                *(u32x2*)&sV[(8 * v_g + e) * V_STRIDE + posv] = out;
+            }
+        }
+    };
+
+    if (n_tiles > 0) load_tile(0);
+    for (int tile = 0; tile < n_tiles; ++tile) {
+        __syncthreads(); // everyone is done reading the previous tile
+        store_tile();
+        __syncthreads();
+        if (tile + 1 < n_tiles) load_tile(tile + 1);
+
+        // ---- S^T = K Q^T : two 32-token blocks ----
+        f32x16 s_acc[2];
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s_acc[mb][i] = 0.f;
+#pragma unroll
+            for (int s = 0; s < KSTEPS; ++s) {
+                const f16x8 kf = *(const f16x8*)&sK[(32 * mb + l32) * K_STRIDE + 16 * s + 8 * hh];
+                const f16x8 kl = *(const f16x8*)&sKlo[(32 * mb + l32) * K_STRIDE + 16 * s + 8 * hh];
+                s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kl, qf[s], s_acc[mb], 0, 0, 0);
+                s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], s_acc[mb], 0, 0, 0);
+            }
+        }
+
+        // ---- online softmax per column (element i <-> token 32 mb + 8 (i/4) + 4 hh + i%4) ----
+        const int t_base = tile * kBN;
+        const bool need_mask = t_base + kBN > lim;
+        float mx = kNegBig;
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                float v = s_acc[mb][i] * sm_scale;
+                if (need_mask) {
+                    const int t = t_base + 32 * mb + 8 * (i >> 2) + 4 * hh + (i & 3);
+                    if (t >= lim) v = -INFINITY;
+                }
+                s_acc[mb][i] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        m_run = m_new;
+        const float bias = kPShift - m_new;
+        f16x8 pf[2][2];
+        float lsum = 0.f;
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const half_t ph = (half_t)__builtin_amdgcn_exp2f(s_acc[mb][i] + bias);
+                lsum += (float)ph; // the sum uses the rounded probability, like the PV product
+                pf[mb][i >> 3][i & 7] = ph;
+            }
+        l_run = l_run * alpha + lsum;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o_acc[cb][i] *= alpha;
+
+        // ---- O^T += V^T P^T ----
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                    const f16x8 vf = *(const f16x8*)&sV[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
+                    o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[mb][t], o_acc[cb], 0, 0, 0);
+                }
+    }
+
+    // ---- normalise and store: element i of block cb <-> channel 32 cb + 8 (i/4) + 4 hh + i%4 ----
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (col_on) {
+        half_t* op = (half_t*)a.output + (q_row0 + pos) * a.output_stride_s + (int64_t)h * D;
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                f16x4 w;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[e] = (half_t)(o_acc[cb][4 * r + e] * inv);
+                *(f16x4*)(op + 32 * cb + 8 * r + 4 * hh) = w;
+            }
+    }
 }
+
+template <int D>
+static void launch_prefill_d(const PrefillLaunch& a, hipStream_t stream)
+{
+    const int G = (int)(a.num_heads / a.num_kv_heads);
+    const int ppw = kCols / G > 0 ? kCols / G : 1;
+    const dim3 grid((unsigned)((a.max_seqlen + ppw - 1) / ppw), (unsigned)a.prefill_batches, (unsigned)a.num_kv_heads);
+    if (a.cache_mode == 1)
+        hipLaunchKernelGGL((prefill_attention_kernel<D, true>), grid, dim3(kPrefillThreads), 0, stream, a);
+    else
+        hipLaunchKernelGGL((prefill_attention_kernel<D, false>), grid, dim3(kPrefillThreads), 0, stream, a);
+}
+
+int launch_prefill(const PrefillLaunch& a, hipStream_t stream)
+{
+    if (a.num_heads / a.num_kv_heads > kCols) return 1;
+    switch (a.head_dim) {
+        case 64: launch_prefill_d<64>(a, stream); return 0;
+        case 128: launch_prefill_d<128>(a, stream); return 0;
+        default: return 1;
+    }
+}
+
+} // namespace pmxhip

@@ -1,0 +1,87 @@
+"""The operator class end to end on the GPU: heuristic_prepare -> workspace ->
+forward() (append, decode, chunked prefill on one stream), checked against the
+CPU oracle: cache bytes and scales bit-exact, outputs within tolerance."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import (assert_attention_close, host_cache, oracle_append_step, oracle_decode, oracle_fill_history,
+                      oracle_prefill)
+
+pytestmark = pytest.mark.gpu
+
+
+def full_step(pkg, oracle, bt, rng, **op_kw):
+    cache, scale = host_cache(bt, canary=(0x5A, 1.5))
+    dev = pkg.harness.DeviceBatch(bt)
+    dev.fill_canary()
+    for b, pos, k_rows, v_rows in oracle_fill_history(oracle, pkg, bt, rng, cache, scale):
+        dev.append_rows(b, pos, k_rows, v_rows)
+    q, k, v = pkg.workloads.step_inputs(bt, rng)
+    dev.set_step_inputs(q, k, v)
+    dev.output.fill_(float("nan"))
+    op = dev.make_operator(**op_kw)
+    rc = op.forward()
+    torch.cuda.synchronize()
+    assert rc == 0
+    oracle_append_step(oracle, bt, k, v, cache, scale)
+    assert np.array_equal(dev.cache.cpu().numpy(), cache)
+    assert np.array_equal(dev.scale.cpu().numpy().view(np.uint16), scale.view(np.uint16))
+    ref = oracle_prefill(oracle, bt, q, cache, scale) if bt.batch > bt.decoding_batches else np.zeros(
+        (q.shape[0], bt.num_heads, bt.head_dim), np.float32)
+    if bt.decoding_batches:
+        ref[:bt.decoding_batches] = oracle_decode(oracle, bt, q, cache, scale)
+    got = dev.output.float().cpu().numpy()
+    return assert_attention_close(got, ref, bt.name), op
+
+
+def test_c1_through_the_operator(pkg, oracle):
+    bt, rng = pkg.workloads.make_batch("C1")
+    full_step(pkg, oracle, bt, rng)
+
+
+@pytest.mark.parametrize("multi_block", [0, 1, 2])
+def test_mixed_batch_through_the_operator(pkg, oracle, multi_block):
+    bt, rng = pkg.workloads.custom_batch(401, num_heads=32, num_kv_heads=8, head_dim=128, cache_mode=1,
+                                         dec_kv_lens=[600, 33, 1500, 129, 1, 256], prefill_q_lens=[100, 17],
+                                         prefill_prior=[150, 0], outliers=True, num_layer=2, layer_idx=1)
+    _, op = full_step(pkg, oracle, bt, rng, specify_decoding_multi_block=multi_block)
+    if multi_block == 0:
+        assert op.cfg.decoding_multi_block_size == 1 and op.cfg.workspace_size == 0
+
+
+def test_scaled_c5_through_the_operator(pkg, oracle):
+    bt, rng = pkg.workloads.make_batch("C5", scale=0.06)
+    full_step(pkg, oracle, bt, rng)
+
+
+def test_contiguous_mode_and_stagewise_calls(pkg, oracle):
+    bt, rng = pkg.workloads.custom_batch(402, num_heads=8, num_kv_heads=8, head_dim=64, cache_mode=0,
+                                         dec_kv_lens=[200, 31], prefill_q_lens=[40], prefill_prior=[9])
+    cache, scale = host_cache(bt)
+    dev = pkg.harness.DeviceBatch(bt)
+    for b, pos, k_rows, v_rows in oracle_fill_history(oracle, pkg, bt, rng, cache, scale):
+        dev.append_rows(b, pos, k_rows, v_rows)
+    q, k, v = pkg.workloads.step_inputs(bt, rng)
+    dev.set_step_inputs(q, k, v)
+    op = dev.make_operator()
+    assert op.forward_kvstore() == 0 and op.forward_decode() == 0 and op.forward_prefill() == 0
+    torch.cuda.synchronize()
+    oracle_append_step(oracle, bt, k, v, cache, scale)
+    ref = oracle_prefill(oracle, bt, q, cache, scale)
+    ref[:2] = oracle_decode(oracle, bt, q, cache, scale)
+    assert_attention_close(dev.output.float().cpu().numpy(), ref, "stagewise")
+
+
+def test_unsupported_configurations_report_not_crash(pkg):
+    bt, rng = pkg.workloads.custom_batch(403, num_heads=4, num_kv_heads=2, head_dim=128, cache_mode=1,
+                                         dec_kv_lens=[20], prefill_q_lens=[8], prefill_prior=[0])
+    dev = pkg.harness.DeviceBatch(bt)
+    q, k, v = pkg.workloads.step_inputs(bt, rng)
+    dev.set_step_inputs(q, k, v)
+    op = dev.make_operator(enable_cache_prefill=False)  # fp16-only prefill is not built: reported, first failure wins
+    assert op.forward_prefill() == pkg.ops.RC_UNSUPPORTED
+    assert op.forward() == pkg.ops.RC_UNSUPPORTED
+    op = dev.make_operator(datatype=6)                  # fp32 tensors: prefill rejects (flash_attn2/fmha.cu:75)
+    assert op.forward_prefill() == pkg.ops.RC_UNSUPPORTED
+    torch.cuda.synchronize()

@@ -1,0 +1,112 @@
+"""GPU parity of the multi-query-token (chunked prefill) kernel against the CPU
+oracle, through the C ABI.  Tolerance: |got - ref| <= 2e-3 + 1e-2 * |ref|."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import (assert_attention_close, host_cache, oracle_append_step, oracle_decode, oracle_fill_history,
+                      oracle_prefill)
+
+pytestmark = pytest.mark.gpu
+
+
+def make_case(pkg, oracle, seed, **kw):
+    bt, rng = pkg.workloads.custom_batch(seed, **kw)
+    cache, scale = host_cache(bt)
+    oracle_fill_history(oracle, pkg, bt, rng, cache, scale)
+    q, k, v = pkg.workloads.step_inputs(bt, rng)
+    oracle_append_step(oracle, bt, k, v, cache, scale)
+    dev = pkg.harness.DeviceBatch(bt)
+    dev.cache.copy_(torch.from_numpy(cache))
+    dev.scale.copy_(torch.from_numpy(scale))
+    dev.set_step_inputs(q, k, v)
+    return bt, dev, q, cache, scale
+
+
+def run_prefill(pkg, dev, is_causal=None):
+    bt = dev.bt
+    dev.output.fill_(float("nan"))
+    pkg.ops.prefill_attention(dev.query, dev.output, dev.cache, dev.scale, dev.seqstarts, dev.kvstarts,
+                              dev.cachestarts, attn_scale=bt.attn_scale,
+                              is_causal=bt.is_causal if is_causal is None else is_causal, batch=bt.batch,
+                              decoding_batches=bt.decoding_batches, max_seqlen=bt.max_seqlen, max_kvlen=bt.max_kvlen,
+                              layer_idx=bt.layer_idx, num_heads=bt.num_heads, num_kv_heads=bt.num_kv_heads,
+                              head_dim=bt.head_dim, **dev.layout_kwargs())
+    torch.cuda.synchronize()
+    return dev.output.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("cache_mode", [0, 1])
+@pytest.mark.parametrize("shape", [(8, 2, 128), (4, 4, 128), (12, 2, 128), (8, 8, 64), (16, 2, 64), (2, 1, 128), (16, 1, 128)])
+def test_prefill_matches_oracle(pkg, oracle, shape, cache_mode):
+    hq, hkv, d = shape
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 300 + hq + d, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                         cache_mode=cache_mode, dec_kv_lens=[33, 140],
+                                         prefill_q_lens=[70, 7, 1, 129, 200], prefill_prior=[130, 0, 50, 127, 0],
+                                         outliers=True)
+    ref = oracle_prefill(oracle, bt, q, cache, scale)
+    got = run_prefill(pkg, dev)
+    n_dec = bt.decoding_batches
+    assert np.isnan(got[:n_dec]).all()  # the prefill stage leaves decode rows alone
+    assert_attention_close(got[n_dec:], ref[n_dec:], "prefill %s mode %d" % (shape, cache_mode))
+
+
+def test_prefill_non_causal_and_single_row_equals_decode(pkg, oracle):
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 320, num_heads=8, num_kv_heads=2, head_dim=128, cache_mode=1,
+                                         dec_kv_lens=[], prefill_q_lens=[1, 65], prefill_prior=[300, 10],
+                                         is_causal=False)
+    ref = oracle_prefill(oracle, bt, q, cache, scale)
+    got = run_prefill(pkg, dev)
+    assert_attention_close(got, ref, "non-causal")
+    # sequence 0 has one query row: the decode kernel over the same cache gives the same answer
+    bt2, _ = pkg.workloads.custom_batch(320, num_heads=8, num_kv_heads=2, head_dim=128, cache_mode=1, dec_kv_lens=[301])
+    dev2 = pkg.harness.DeviceBatch(bt2)
+    dev2.cache = dev.cache
+    dev2.scale = dev.scale
+    dev2.cachestarts = dev.cachestarts[0:1].contiguous()
+    bt2.cachestarts_stride_b = bt.cachestarts_stride_b
+    bt2.layout = bt.layout
+    dev2.set_step_inputs(q[0:1], q[0:1, :2], q[0:1, :2])
+    dev2.decode_only(num_token_ranges=3)
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(dev2.output.float().cpu().numpy()[0], got[0], rtol=1e-2, atol=2e-3)
+
+
+def test_prefill_kv_shorter_than_query(pkg, oracle):
+    """kvlen < qlen under the bottom-right mask: the first rows see no key and come out zero."""
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 330, num_heads=4, num_kv_heads=2, head_dim=128, cache_mode=0,
+                                         dec_kv_lens=[], prefill_q_lens=[40], prefill_prior=[0])
+    bt.kv_lens[0] = 25
+    bt.kvstarts = np.array([0, 25], dtype=np.int64)
+    dev.kvstarts.copy_(torch.from_numpy(bt.kvstarts))
+    ref = oracle_prefill(oracle, bt, q, cache, scale)
+    got = run_prefill(pkg, dev)
+    assert (ref[:15] == 0).all() and (got[:15] == 0).all()
+    assert_attention_close(got, ref, "kv shorter than q")
+
+
+def test_prefill_full_size_c5(pkg, oracle):
+    """The C5 prefill part at full size: sampled rows against the oracle."""
+    bt, rng = pkg.workloads.make_batch("C5")
+    dev = pkg.harness.DeviceBatch(bt)
+    dev.fill_history_random_bytes(seed=5)
+    q, k, v = pkg.workloads.step_inputs(bt, rng)
+    dev.set_step_inputs(q, k, v)
+    got = run_prefill(pkg, dev)
+    n_dec = bt.decoding_batches
+    assert not np.isnan(got[n_dec:]).any()
+    cache = dev.cache.cpu().numpy()
+    scale = dev.scale.cpu().numpy()
+    from conftest import oracle_layout_kwargs
+    kw = oracle_layout_kwargs(bt)
+    pick = np.random.default_rng(1)
+    for b in pick.choice(np.arange(n_dec, bt.batch), size=4, replace=False):
+        qlen, kvlen = int(bt.q_lens[b]), int(bt.kv_lens[b])
+        for i in (0, qlen // 2, qlen - 1):
+            row = int(bt.seqstarts[b]) + i
+            lim = i + 1 + kvlen - qlen
+            for h in pick.choice(bt.num_heads, size=2, replace=False):
+                o, _, _ = oracle.decode_partial(q[row:], cache, scale, bt.cachestarts[b:], 0, int(h), 0, lim,
+                                                bt.num_heads, bt.num_kv_heads, bt.head_dim, bt.attn_scale, 0,
+                                                bt.page_size, **kw)
+                assert_attention_close(got[row, h], o, "C5 b=%d row=%d h=%d" % (b, i, h))
