@@ -168,6 +168,7 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
     const int64_t r1 = (r0 + per < total) ? r0 + per : total;
 #ifdef PMX_WG_TRACE
     const unsigned long long trace_t0 = wall_clock64();
+    const unsigned long long trace_c0 = clock64();
 #endif
 
     // Addressing: a wave-uniform 64-bit base per block (scalar registers) plus a 32-bit per-lane
@@ -576,8 +577,8 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
         asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
         tr[wg * 4 + 0] = trace_t0;
         tr[wg * 4 + 1] = wall_clock64();
-        tr[wg * 4 + 2] = xcc;
-        tr[wg * 4 + 3] = hwid;
+        tr[wg * 4 + 2] = clock64() - trace_c0;
+        tr[wg * 4 + 3] = ((unsigned long long)xcc << 32) | hwid;
     }
 #endif
 }

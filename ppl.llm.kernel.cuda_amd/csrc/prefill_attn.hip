@@ -62,9 +62,14 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_attention_kernel(cons
     // lo = the rounding error of that product (exact, from one fused multiply-add), so that
     // q.k carries no fp16 rounding of the dequantised key.  With a single rounded copy a
     // 2^-12 relative error on |q_c k_c| ~ 1e3 (outlier channels) moves logits by ~1e-2.
-    __shared__ __attribute__((aligned(16))) half_t sK[kBN * K_STRIDE];
-    __shared__ __attribute__((aligned(16))) half_t sKlo[kBN * K_STRIDE];
-    __shared__ __attribute__((aligned(16))) half_t sV[D * V_STRIDE];
+    // V and the probabilities are split the same way (V^ = hi + lo from the same multiply-add
+    // trick, p = hi + lo), and O accumulates hi*hi + lo*hi + hi*lo: at |v| ~ 40 a single fp16
+    // rounding of either factor already costs ~1e-2 absolute where contributions cancel.
+    extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+    half_t* const sK = (half_t*)smem_raw;
+    half_t* const sKlo = sK + kBN * K_STRIDE;
+    half_t* const sV = sKlo + kBN * K_STRIDE;
+    half_t* const sVlo = sV + D * V_STRIDE;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -201,10 +206,14 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_attention_kernel(cons
                 const uint32_t w2 = upper ? v_raw[2][1] : v_raw[2][0], w3 = upper ? v_raw[3][1] : v_raw[3][0];
                 const half2_t lo = pk_sub_1152(__builtin_amdgcn_perm(w1, w0, sel) ^ 0x64806480u);
                 const half2_t hi = pk_sub_1152(__builtin_amdgcn_perm(w3, w2, sel) ^ 0x64806480u);
-                u32x2 out;
-                out[0] = bitcast<uint32_t>(lo * s01);
-                out[1] = bitcast<uint32_t>(hi * s23);
+                const half2_t h01 = lo * s01, h23 = hi * s23;
+                u32x2 out, outl;
+                out[0] = bitcast<uint32_t>(h01);
+                out[1] = bitcast<uint32_t>(h23);
+                outl[0] = bitcast<uint32_t>(__builtin_elementwise_fma(lo, s01, -h01));
+                outl[1] = bitcast<uint32_t>(__builtin_elementwise_fma(hi, s23, -h23));
                 *(u32x2*)&sV[(8 * v_g + e) * V_STRIDE + posv] = out;
+                *(u32x2*)&sVlo[(8 * v_g + e) * V_STRIDE + posv] = outl;
             }
         }
     };
@@ -252,15 +261,18 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_attention_kernel(cons
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
         m_run = m_new;
         const float bias = kPShift - m_new;
-        f16x8 pf[2][2];
+        f16x8 pf[2][2], pfl[2][2];
         float lsum = 0.f;
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const half_t ph = (half_t)__builtin_amdgcn_exp2f(s_acc[mb][i] + bias);
-                lsum += (float)ph; // the sum uses the rounded probability, like the PV product
+                const float pv = __builtin_amdgcn_exp2f(s_acc[mb][i] + bias);
+                const half_t ph = (half_t)pv;
+                const half_t pl = (half_t)(pv - (float)ph);
+                lsum += (float)ph + (float)pl; // the sum uses exactly what the PV product uses
                 pf[mb][i >> 3][i & 7] = ph;
+                pfl[mb][i >> 3][i & 7] = pl;
             }
         l_run = l_run * alpha + lsum;
 #pragma unroll
@@ -276,6 +288,9 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_attention_kernel(cons
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) {
                     const f16x8 vf = *(const f16x8*)&sV[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
+                    const f16x8 vl = *(const f16x8*)&sVlo[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
+                    o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vl, pf[mb][t], o_acc[cb], 0, 0, 0);
+                    o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pfl[mb][t], o_acc[cb], 0, 0, 0);
                     o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[mb][t], o_acc[cb], 0, 0, 0);
                 }
     }
@@ -303,10 +318,19 @@ static void launch_prefill_d(const PrefillLaunch& a, hipStream_t stream)
     const int G = (int)(a.num_heads / a.num_kv_heads);
     const int ppw = kCols / G > 0 ? kCols / G : 1;
     const dim3 grid((unsigned)((a.max_seqlen + ppw - 1) / ppw), (unsigned)a.prefill_batches, (unsigned)a.num_kv_heads);
-    if (a.cache_mode == 1)
-        hipLaunchKernelGGL((prefill_attention_kernel<D, true>), grid, dim3(kPrefillThreads), 0, stream, a);
-    else
-        hipLaunchKernelGGL((prefill_attention_kernel<D, false>), grid, dim3(kPrefillThreads), 0, stream, a);
+    // K hi/lo tiles + transposed V hi/lo tiles; above the 64 KB static limit for D = 128, hence dynamic
+    constexpr size_t lds_bytes = (2 * kBN * (D + 8) + 2 * D * (kBN + 8)) * sizeof(half_t);
+    if (a.cache_mode == 1) {
+        static const hipError_t once = hipFuncSetAttribute((const void*)prefill_attention_kernel<D, true>,
+                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        (void)once;
+        hipLaunchKernelGGL((prefill_attention_kernel<D, true>), grid, dim3(kPrefillThreads), lds_bytes, stream, a);
+    } else {
+        static const hipError_t once = hipFuncSetAttribute((const void*)prefill_attention_kernel<D, false>,
+                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        (void)once;
+        hipLaunchKernelGGL((prefill_attention_kernel<D, false>), grid, dim3(kPrefillThreads), lds_bytes, stream, a);
+    }
 }
 
 int launch_prefill(const PrefillLaunch& a, hipStream_t stream)

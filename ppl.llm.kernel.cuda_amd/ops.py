@@ -192,8 +192,8 @@ class DynamicBatchingMultiHeadCacheAttention:
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
-        if h:
-            _lib.lib().pmxhip_mhca_destroy(h)
+        if h and _lib is not None and _lib._lib is not None:  # module globals are gone at interpreter exit
+            _lib._lib.pmxhip_mhca_destroy(h)
 
     def heuristic_prepare(self, *, query=None, query_shape, current_key=None, current_key_shape,
                           current_value=None, current_value_shape, attn_mask=None, attn_mask_shape=(),
