@@ -78,6 +78,9 @@ def main():
     ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C3m0", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ranges", type=int, default=0, help="token ranges for decode (0 = planned)")
+    ap.add_argument("--calibration-copy-mib", type=int, default=0,
+                    help="also run one plain device copy of this many MiB (known traffic, for scaling rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards by kv head "
@@ -140,6 +143,12 @@ def main():
     stages = {"decode_ranges": t_ranges, "decode_combine": t_combine, "append": t_append}
     if bt.batch > bt.decoding_batches:
         stages["prefill"] = time_stage(lambda: op.forward_prefill(stream), n_ev)
+
+    if args.calibration_copy_mib:
+        src = torch.ones(args.calibration_copy_mib << 20, dtype=torch.int8, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
 
     dec_bytes = bt.decode_algorithmic_bytes()
     achieved = dec_bytes / (t_ranges["avg_us"] * 1e-6) / 1e9

@@ -7,7 +7,7 @@
  * entry points below are what that class bottoms out in -- one per kernel launch
  * site of src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/kernel.cu -- with
  * plain pointers and sizes only, so that any FFI can bind them.  The C++ class in
- * multi_head_cache_attention.h (this directory) marshals its cfg into these.
+ * cache_attention.h (this directory) marshals its cfg into these.
  *
  * Conventions shared by every entry point:
  *   - all pointers are device pointers unless stated otherwise; the caller owns
