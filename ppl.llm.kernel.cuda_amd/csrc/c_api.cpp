@@ -208,6 +208,8 @@ int pmxhip_decode_attention_stage(const pmxhip_decode_params* p, int32_t stage, 
     if (!aligned16(p->query) || !aligned16(p->cache) || (reinterpret_cast<uintptr_t>(p->scale) & 3u) ||
         p->query_stride_s % 8 != 0)
         return fail(PMXHIP_UNSUPPORTED, "decode_attention: query/cache must be 16-byte aligned, scale 4-byte aligned");
+    if ((reinterpret_cast<uintptr_t>(p->output) & 7u) || p->output_stride_s % 4 != 0) // 8-byte stores of four halves
+        return fail(PMXHIP_UNSUPPORTED, "decode_attention: output must be 8-byte aligned with a row stride that is a multiple of 4");
     if (p->attn_mask && p->mask_stride_s % 8 != 0) // utils.cu:127-130
         return fail(PMXHIP_UNSUPPORTED, "last dimension of attn_mask must be aligned with 8");
 

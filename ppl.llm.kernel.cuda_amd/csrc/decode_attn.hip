@@ -19,6 +19,9 @@
 //     scales.  LPS = D/16 lanes form a "slot" that walks tokens; a wave has
 //     64/LPS slots, distributed over kv heads first and tokens second, so that a
 //     wave's load instruction covers a contiguous run of the token row.
+//   * Inside a sequence the cuts between ranges are moved up to the next multiple
+//     of the workgroup's block of tokens (or to the sequence end), so that every
+//     piece starts on a block boundary and only its last block can be partial.
 //   * Each slot keeps an online-softmax state per query head; slots are merged
 //     through LDS at the end of a piece.  A piece that is a whole sequence is
 //     written as final fp16 output; otherwise a float32 partial (normalised
@@ -91,6 +94,21 @@ __device__ __forceinline__ int64_t tokens_per_range(int64_t total, int ranges, i
     return (per + wg_tokens - 1) / wg_tokens * wg_tokens;
 }
 
+// The piece [pa, pe) of a sequence (stream position s_beg, length len) that the range [r0, r1)
+// owns, in sequence coordinates.  A cut inside the sequence moves up to the next multiple of
+// `align` (a power of two) or to the sequence end; both neighbours compute the same cut, so the
+// pieces of a sequence still partition it.  pe <= pa: the range owns nothing of the sequence.
+__device__ __forceinline__ void piece_bounds(int64_t r0, int64_t r1, int64_t s_beg, int64_t len, int align,
+                                             int64_t& pa, int64_t& pe)
+{
+    const int64_t mask = (int64_t)align - 1;
+    int64_t lo = r0 - s_beg, hi = r1 - s_beg;
+    lo = lo <= 0 ? 0 : ((lo + mask) & ~mask);
+    hi = hi <= 0 ? 0 : ((hi + mask) & ~mask);
+    pa = lo < len ? lo : len;
+    pe = hi < len ? hi : len;
+}
+
 // first b in [0, n) with starts[b + 1] - starts[0] > g   (starts is non-decreasing)
 __device__ __forceinline__ int find_sequence(const_i64_ptr starts, int n, int64_t g)
 {
@@ -118,6 +136,15 @@ struct VBlock {
     uint32_t sc[kTB];
 };
 
+// Bytes of dynamic LDS the decode kernel needs: one slot-partial (D floats) per slot and query
+// head, plus the (max, exp-sum) pair of each.
+constexpr size_t decode_lds_bytes(int head_dim, int gt)
+{
+    const int lps = head_dim == 64 ? 4 : (head_dim == 256 ? 16 : 8);
+    const int nslot = kWave / lps * kDecodeWaves;
+    return (size_t)gt * nslot * (head_dim + 2) * sizeof(float);
+}
+
 // D: head dim (64, 96, 128, 256).  GT: query heads per kv head held in registers.
 template <int D, int GT, bool PAGED, bool MASK>
 __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_attention_kernel(const DecodeLaunch a)
@@ -126,11 +153,15 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
     constexpr int LPS_ACTIVE = D / 16;                        // 6 of 8 for D = 96
     constexpr int SPW = kWave / LPS;                          // slots per wave
     constexpr int NSLOT = SPW * kDecodeWaves;
-    constexpr bool kHandScheduled = GT <= 4; // inline-assembly loads with explicit wait counts in the steady-state loop
+    // Inline-assembly loads with explicit wait counts in the pipelined loop.  Not for GT = 8 (does not fit
+    // the register file without spills) nor with a mask (its loads are the compiler's): a spill or a
+    // compiler-scheduled load inside the loop is not compatible with loads that land behind the compiler's back.
+    constexpr bool kHandScheduled = GT <= 4 && !MASK;
 
-    __shared__ float sm_acc[NSLOT * D];
-    __shared__ float sm_m[NSLOT];
-    __shared__ float sm_l[NSLOT];
+    extern __shared__ float sm_dyn[];
+    float* const sm_acc = sm_dyn;                 // [GT][NSLOT][D]
+    float* const sm_m = sm_dyn + GT * NSLOT * D;  // [GT][NSLOT]
+    float* const sm_l = sm_m + GT * NSLOT;        // [GT][NSLOT]
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -146,13 +177,16 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
     const bool lane_on = ls < LPS_ACTIVE;
     const int ch0 = (lane_on ? ls : 0) * 16;
 
-    // slots over (kv head, token sub-index): kv heads first
-    const int kvhb = a.kv_heads_per_group;        // power of two, <= SPW
-    const int tpl = SPW / kvhb;                   // tokens one wave load covers
+    // slots over (kv head, token sub-index): kv heads first.  kvhb and tpl are powers of two.
+    const int kvhb = a.kv_heads_per_group;        // <= SPW
+    const int kvhb_shift = __builtin_ctz(kvhb);
+    const int tpl = SPW >> kvhb_shift;            // tokens one wave load covers
+    const int tpl_shift = __builtin_ctz(tpl);
     const int head_local = slot & (kvhb - 1);
-    const int tsub = slot / kvhb;
+    const int tsub = slot >> kvhb_shift;
     const int wave_tokens = kTB * tpl;            // tokens a wave handles per iteration
     const int wg_tokens = wave_tokens * kDecodeWaves;
+    const int wg_shift = __builtin_ctz(wg_tokens);
 
     const int kvh = blockIdx.y * kvhb + head_local;
     const int g_first = blockIdx.z * GT; // first query head (within the kv head's group) of this pass
@@ -172,15 +206,10 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
 #endif
 
     // Addressing: a wave-uniform 64-bit base per block (scalar registers) plus a 32-bit per-lane
-    // offset that never changes: (token in block) * stride_s + (head in group) * stride_h + channel.
+    // offset: (token in block) * stride_s + (head in group) * stride_h + channel.
     const int64_t group_off = a.layer_idx * a.cache_stride_l + (int64_t)(blockIdx.y * kvhb) * a.cache_stride_h;
-    uint32_t voff[kTB];
-#pragma unroll
-    for (int j = 0; j < kTB; ++j)
-        voff[j] = (uint32_t)((int64_t)((j ^ tp) * tpl + tsub) * a.cache_stride_s + (int64_t)head_local * a.cache_stride_h + ch0);
-    uint32_t voff_sc[kTB]; // the same offsets in the scale tensor: one fp16 scale per 8 channels
-#pragma unroll
-    for (int j = 0; j < kTB; ++j) voff_sc[j] = voff[j] >> 2;
+    const uint32_t stride_s32 = (uint32_t)a.cache_stride_s; // the host checks that a block's span fits 32 bits
+    const uint32_t lane_base = (uint32_t)((int64_t)head_local * a.cache_stride_h + ch0);
     const char* const cache_k = (const char*)a.cache + group_off;
     const char* const cache_v = cache_k + a.cache_stride_kv;
     const char* const scale_k = (const char*)a.scale + (group_off >> 3) * 2;
@@ -191,12 +220,105 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
     for (; b < a.decoding_batches; ++b) {
         const int64_t s_beg = kvstarts[b] - kv_base;
         if (s_beg >= r1) break;
-        const int64_t s_end = kvstarts[b + 1] - kv_base;
-        const int64_t len = s_end - s_beg;
-        // piece [pa, pe) in sequence coordinates
-        const int64_t pa = (r0 > s_beg ? r0 : s_beg) - s_beg;
-        const int64_t pe = (r1 < s_end ? r1 : s_end) - s_beg;
+        const int64_t len = kvstarts[b + 1] - kv_base - s_beg;
+        int64_t pa, pe; // this workgroup's piece [pa, pe) of the sequence, in sequence coordinates
+        piece_bounds(r0, r1, s_beg, len, wg_tokens, pa, pe);
         if (pe <= pa) continue;
+        // sequence-relative positions fit 32 bits
+        const int pa32 = (int)pa, pe32 = (int)pe;
+
+        // Wave blocks: pa is a multiple of wg_tokens, so every block lies inside one page and only
+        // the last block of a wave can reach beyond the piece.
+        const int pos0 = pa32 + wave * wave_tokens;
+        const int nb = pos0 < pe32 ? (pe32 - pos0 + wg_tokens - 1) >> wg_shift : 0;
+        const bool tail_partial = nb > 0 && pos0 + ((nb - 1) << wg_shift) + wave_tokens > pe32;
+
+        const int64_t table_base = PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b;
+        const int64_t seq_row0 = PAGED ? 0 : cachestarts[b];
+        const half_t* mask_row = nullptr;
+        if (MASK) mask_row = (const half_t*)a.attn_mask + (int64_t)b * a.mask_stride_s + kvstarts[b];
+        const int last_page = (pe32 - 1) >> 7;
+
+        // Page table entries are read one page ahead with scalar loads, so that no block waits
+        // for its row base: `page_row` belongs to page `page_idx`, `next_row` to the page after it.
+        int page_idx = -2;
+        int64_t page_row = 0, next_row = 0;
+        auto row_base_of = [&](int pos) -> int64_t {
+            if (!PAGED) return seq_row0 + pos;
+            const int pg = pos >> 7;
+            if (pg != page_idx) {
+                page_row = (pg == page_idx + 1) ? next_row : cachestarts[table_base + pg];
+                page_idx = pg;
+                const int nx = pg + 1 <= last_page ? pg + 1 : last_page;
+                next_row = cachestarts[table_base + nx];
+            }
+            return page_row + (pos & (kPage - 1));
+        };
+
+        // Per-lane offsets of the block being requested: those of a full block until the wave's last
+        // block is requested; if that one reaches beyond the piece, its out-of-piece tokens are
+        // redirected to the piece's last token (the load is harmless, the logit is masked).
+        uint32_t vo[kTB], vo_sc[kTB];
+#pragma unroll
+        for (int j = 0; j < kTB; ++j) {
+            vo[j] = (uint32_t)((j ^ tp) * tpl + tsub) * stride_s32 + lane_base;
+            vo_sc[j] = vo[j] >> 2; // the same offset in the scale tensor: one fp16 scale per 8 channels
+        }
+        auto clamp_offsets = [&](int pos) {
+#pragma unroll
+            for (int j = 0; j < kTB; ++j) {
+                const int t = pos + (j ^ tp) * tpl + tsub;
+                const int tc = t < pe32 ? t : pe32 - 1;
+                vo[j] = (uint32_t)(tc - pos) * stride_s32 + lane_base;
+                vo_sc[j] = vo[j] >> 2;
+            }
+        };
+
+        // ---- requests of one wave block (positions pos .. pos + wave_tokens): K with its scales, V with
+        // its scales, in a fixed order (token 0: 16 bytes then scales, token 1: ..., 8 operations per
+        // half-block) ----
+        auto request_k = [&](KBlock& kb, int pos) {
+            kb.pos = pos;
+            const int64_t boff = row_base_of(pos) * a.cache_stride_s;
+            kb.boff = boff;
+            const char* bk = cache_k + boff;
+            const char* sk = scale_k + (boff >> 3) * 2;
+#pragma unroll
+            for (int j = 0; j < kTB; ++j) {
+                if (kHandScheduled) {
+                    load_b128(kb.q8[j], vo[j], bk);
+                    load_b32(kb.sc[j], vo_sc[j], sk);
+                } else {
+                    kb.q8[j] = *(const u32x4*)(bk + vo[j]);
+                    kb.sc[j] = *(const uint32_t*)(sk + vo_sc[j]);
+                }
+            }
+        };
+        auto request_v = [&](VBlock& vb, int64_t boff) {
+            const char* bv = cache_v + boff;
+            const char* sv = scale_v + (boff >> 3) * 2;
+#pragma unroll
+            for (int j = 0; j < kTB; ++j) {
+                if (kHandScheduled) {
+                    load_b128(vb.q8[j], vo[j], bv);
+                    load_b32(vb.sc[j], vo_sc[j], sv);
+                } else {
+                    vb.q8[j] = *(const u32x4*)(bv + vo[j]);
+                    vb.sc[j] = *(const uint32_t*)(sv + vo_sc[j]);
+                }
+            }
+        };
+
+        // The first block is requested before anything else of the piece, so that its latency overlaps
+        // the query loads below.
+        KBlock ka, kb;
+        VBlock va, vb;
+        int pos = pos0;
+        if (nb > 0) {
+            if (nb == 1 && tail_partial) clamp_offsets(pos);
+            request_k(ka, pos);
+            request_v(va, ka.boff);
+        }
 
         // ---- query heads of this kv head into registers (packed halves) ----
         // qb[g][i] = -1152 * (sum of the 8 query channels of group i): the int8 -> half conversion
@@ -233,93 +355,14 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
             for (int c = 0; c < 16; ++c) acc[g][c] = 0.f;
         }
 
-        const int64_t table_base = PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b;
-        const int64_t seq_row0 = PAGED ? 0 : cachestarts[b];
-        const half_t* mask_row = nullptr;
-        if (MASK) mask_row = (const half_t*)a.attn_mask + (int64_t)b * a.mask_stride_s + kvstarts[b];
-        // sequence-relative positions fit 32 bits
-        const int pa32 = (int)pa, pe32 = (int)pe;
-        const int last_page = (pe32 - 1) >> 7;
-
-        // Page table entries are read one page ahead with scalar loads, so that no block waits
-        // for its row base: `page_row` belongs to page `page_idx`, `next_row` to the page after it.
-        int page_idx = -2;
-        int64_t page_row = 0, next_row = 0;
-        auto row_base_of = [&](int pos) -> int64_t {
-            if (!PAGED) return seq_row0 + pos;
-            const int pg = pos >> 7;
-            if (pg != page_idx) {
-                page_row = (pg == page_idx + 1) ? next_row : cachestarts[table_base + pg];
-                page_idx = pg;
-                const int nx = pg + 1 <= last_page ? pg + 1 : last_page;
-                next_row = cachestarts[table_base + nx];
-            }
-            return page_row + (pos & (kPage - 1));
-        };
-
-        // ---- loads of one wave block (positions pos .. pos + wave_tokens): K with its scales, V with its scales.
-        // FULL blocks lie inside the piece; in a partial block the tokens outside the piece are redirected
-        // to a token inside it (the load is harmless, the logit is masked later) ----
-        auto lane_off = [&](int pos, int j) -> uint32_t {
-            const int t = pos + (j ^ tp) * tpl + tsub;
-            const int tc = t < pa32 ? pa32 : (t >= pe32 ? pe32 - 1 : t);
-            return (uint32_t)((int64_t)(tc - pos) * a.cache_stride_s + (int64_t)head_local * a.cache_stride_h + ch0);
-        };
-        // steady-state versions: full blocks only, inline-assembly loads in a fixed order
-        // (token 0: 16 bytes then scales, token 1: ..., 8 operations per half-block)
-        auto issue_k_fast = [&](KBlock& kb, int pos) {
-            kb.pos = pos;
-            const int64_t boff = row_base_of(pos) * a.cache_stride_s;
-            kb.boff = boff;
-            const char* bk = cache_k + boff;
-            const char* sk = scale_k + (boff >> 3) * 2;
-#pragma unroll
-            for (int j = 0; j < kTB; ++j) {
-                load_b128(kb.q8[j], voff[j], bk);
-                load_b32(kb.sc[j], voff_sc[j], sk);
-            }
-        };
-        auto issue_v_fast = [&](VBlock& vb, int64_t boff) {
-            const char* bv = cache_v + boff;
-            const char* sv = scale_v + (boff >> 3) * 2;
-#pragma unroll
-            for (int j = 0; j < kTB; ++j) {
-                load_b128(vb.q8[j], voff[j], bv);
-                load_b32(vb.sc[j], voff_sc[j], sv);
-            }
-        };
-        auto issue_k = [&](KBlock& kb, int pos, bool full) {
-            kb.pos = pos;
-            const int64_t boff = row_base_of(pos) * a.cache_stride_s;
-            kb.boff = boff;
-            const char* bk = cache_k + boff;
-            const char* sk = scale_k + (boff >> 3) * 2;
-#pragma unroll
-            for (int j = 0; j < kTB; ++j) {
-                const uint32_t off = full ? voff[j] : lane_off(pos, j);
-                kb.q8[j] = *(const u32x4*)(bk + off);
-                kb.sc[j] = *(const uint32_t*)(sk + (off >> 2));
-            }
-        };
-        auto issue_v = [&](VBlock& vb, int pos, int64_t boff, bool full) {
-            const char* bv = cache_v + boff;
-            const char* sv = scale_v + (boff >> 3) * 2;
-#pragma unroll
-            for (int j = 0; j < kTB; ++j) {
-                const uint32_t off = full ? voff[j] : lane_off(pos, j);
-                vb.q8[j] = *(const u32x4*)(bv + off);
-                vb.sc[j] = *(const uint32_t*)(sv + (off >> 2));
-            }
-        };
-
-        // ---- QK^T and softmax of one block: leaves this lane's probability (token ql) in p[g] ----
+        // ---- QK^T and softmax of one block: leaves this lane's probability (token tp) in p[g] ----
         float p[GT];
-        auto logits_softmax = [&](KBlock& kb, bool full, bool fast) {
+        auto logits_softmax = [&](KBlock& kb) {
             // logits, still partial over the slot's lanes: part[g][j], log2 units
             float part[GT][kTB];
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
-                if (fast) {
+                if (kHandScheduled) {
                     // outstanding and younger than token j of this half-block: the rest of this half-block,
                     // and the two half-blocks requested after it
                     if (j == 0) wait_loads<22>(kb.q8[0], kb.sc[0]);
@@ -339,9 +382,10 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
                 const float s1 = (float)sc.y * logit_scale;
 #pragma unroll
                 for (int g = 0; g < GT; ++g) {
-                    float d0 = qb[g][0], d1 = qb[g][1];
+                    float d0 = dot2_init(q[g][0], kh[0], qb[g][0]);
+                    float d1 = dot2_init(q[g][4], kh[4], qb[g][1]);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
+                    for (int i = 1; i < 4; ++i) {
                         d0 = dot2(q[g][i], kh[i], d0);
                         d1 = dot2(q[g][4 + i], kh[4 + i], d1);
                     }
@@ -352,6 +396,8 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
             // reduce-scatter inside the quad (slot k here and slot k ^ 2 of the xor-2 partner are the
             // same token), then all-reduce across the quads of the slot: the lane ends with the complete
             // logit of token tp
+            const int tk = kb.pos + tp * tpl + tsub;
+            const bool ok = tk < pe32; // false only in a wave's last block, for tokens beyond the piece
             bool rescale = false;
             float m_new[GT];
 #pragma unroll
@@ -361,15 +407,11 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
                 float logit = u0 + dpp_f32<kDppXor1>(u1);
                 if (LPS >= 8) logit += dpp_f32<kDppHalfMirror>(logit);
                 if (LPS >= 16) logit += dpp_f32<kDppMirror>(logit);
-                if (MASK || !full) {
-                    const int tk = kb.pos + tp * tpl + tsub;
-                    const bool ok = tk >= pa32 && tk < pe32;
-                    if (MASK && ok && g_first + g < G) {
-                        const int h = kvh * G + g_first + g;
-                        logit += (float)mask_row[(int64_t)h * a.mask_stride_h + tk] * kLog2e;
-                    }
-                    if (!ok) logit = -INFINITY;
+                if (MASK && ok && g_first + g < G) {
+                    const int h = kvh * G + g_first + g;
+                    logit += (float)mask_row[(int64_t)h * a.mask_stride_h + tk] * kLog2e;
                 }
+                logit = ok ? logit : -INFINITY;
                 // block max over the quad (= over the block's tokens)
                 float mx = fmaxf(logit, dpp_f32<kDppXor1>(logit));
                 mx = fmaxf(mx, dpp_f32<kDppXor2>(mx));
@@ -394,10 +436,10 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
         // ---- PV of one block: int8 values converted straight to fp32 (exact), fp32 weights p * scale,
         // fp32 multiply-accumulate in the two-source form (v_fmac_f32), which issues at twice the rate
         // of the three-source and packed forms on this chip ----
-        auto accumulate_pv = [&](VBlock& vb, bool fast) {
+        auto accumulate_pv = [&](VBlock& vb) {
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
-                if (fast) {
+                if (kHandScheduled) {
                     if (j == 0) wait_loads<22>(vb.q8[0], vb.sc[0]);
                     if (j == 1) wait_loads<20>(vb.q8[1], vb.sc[1]);
                     if (j == 2) wait_loads<18>(vb.q8[2], vb.sc[2]);
@@ -426,147 +468,109 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
             }
         };
 
-        // Wave blocks of this piece are aligned to wg_tokens in sequence coordinates, so that a block
-        // never straddles a page.  At most the first and the last block of a wave are partial; they take
-        // the simple path.  The full blocks in between run software-pipelined: K of block i+1 is
-        // requested before the logits of block i, V of block i+1 before the PV of block i, so that three
-        // half-blocks of cache bytes are in registers or in flight at any time.
-        auto simple_block = [&](int pos) {
-            KBlock kx;
-            VBlock vx;
-            issue_k(kx, pos, false);
-            issue_v(vx, pos, kx.boff, false);
-            logits_softmax(kx, false, false);
-            accumulate_pv(vx, false);
-        };
-        int pos = (int)(pa / wg_tokens * wg_tokens) + wave * wave_tokens;
-        if (pos + wave_tokens <= pa32) pos += wg_tokens;
-        if (pos < pe32 && pos < pa32) {
-            simple_block(pos);
-            pos += wg_tokens;
-        }
-        int n_full = (pos + wave_tokens <= pe32) ? (pe32 - wave_tokens - pos) / wg_tokens + 1 : 0;
-        if (kHandScheduled && n_full > 0) {
-            // Every block requests the next one unconditionally (the last re-requests itself): with no
-            // branch around the loads, and no register copies between stages (two named buffer pairs,
-            // loop unrolled by two), the hardware wait counts stay exact.
-            KBlock ka, kb;
-            VBlock va, vb;
-            __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): the explicit wait counts below assume that only the loop's own loads are in flight
-            issue_k_fast(ka, pos);
-            issue_v_fast(va, ka.boff);
-            // the first block has landed before the loop is entered: any register copy the compiler
-            // places on the loop's entry edge then copies data, not a register still being loaded
-            drain_loads(ka.q8, ka.sc);
-            drain_loads(va.q8, va.sc);
+        // The blocks run software-pipelined: K of block i+1 is requested before the logits of block i,
+        // V of block i+1 before the PV of block i, so that three half-blocks of cache bytes are in
+        // registers or in flight at any time.  Every block requests the next one unconditionally (the
+        // last re-requests itself): with no branch around the loads, and no register copies between
+        // stages (two named buffer pairs, loop unrolled by two), the hardware wait counts stay exact.
+        if (nb > 0) {
+            if (kHandScheduled) {
+                // The first block has landed before the loop is entered, and nothing else is in flight:
+                // the wait counts of the loop count the loop's own requests only, and any register copy
+                // the compiler places on the loop's entry edge copies data, not a register being loaded.
+                drain_loads(ka.q8, ka.sc);
+                drain_loads(va.q8, va.sc);
+            }
             for (int i = 0;;) {
                 // even block: consume (ka, va), request (kb, vb)
-                int npos = pos + (i + 1 < n_full ? wg_tokens : 0);
-                issue_k_fast(kb, npos);
-                logits_softmax(ka, true, true);
-                issue_v_fast(vb, kb.boff);
-                accumulate_pv(va, true);
+                int npos = pos + (i + 1 < nb ? wg_tokens : 0);
+                if (tail_partial && i + 2 == nb) clamp_offsets(npos);
+                request_k(kb, npos);
+                logits_softmax(ka);
+                request_v(vb, kb.boff);
+                accumulate_pv(va);
                 pos = npos;
-                if (++i == n_full) break;
+                if (++i == nb) break;
                 // odd block: consume (kb, vb), request (ka, va)
-                npos = pos + (i + 1 < n_full ? wg_tokens : 0);
-                issue_k_fast(ka, npos);
-                logits_softmax(kb, true, true);
-                issue_v_fast(va, ka.boff);
-                accumulate_pv(vb, true);
+                npos = pos + (i + 1 < nb ? wg_tokens : 0);
+                if (tail_partial && i + 2 == nb) clamp_offsets(npos);
+                request_k(ka, npos);
+                logits_softmax(kb);
+                request_v(va, ka.boff);
+                accumulate_pv(vb);
                 pos = npos;
-                if (++i == n_full) break;
+                if (++i == nb) break;
             }
-            // drain the last (redundant) requests; all four staging buffers stay reserved until then
-            drain_loads(ka.q8, ka.sc);
-            drain_loads(kb.q8, kb.sc);
-            drain_loads(va.q8, va.sc);
-            drain_loads(vb.q8, vb.sc);
-            pos += wg_tokens;
-        }
-        if (!kHandScheduled && n_full > 0) {
-            // GT = 8 does not fit the register file without moving values to accumulation registers,
-            // which is not compatible with loads that land behind the compiler's back: this variant
-            // leaves load scheduling to the compiler.
-            KBlock ka, kb;
-            VBlock va, vb;
-            issue_k(ka, pos, true);
-            issue_v(va, pos, ka.boff, true);
-            for (int i = 0;;) {
-                int npos = pos + (i + 1 < n_full ? wg_tokens : 0);
-                issue_k(kb, npos, true);
-                logits_softmax(ka, true, false);
-                issue_v(vb, npos, kb.boff, true);
-                accumulate_pv(va, false);
-                pos = npos;
-                if (++i == n_full) break;
-                npos = pos + (i + 1 < n_full ? wg_tokens : 0);
-                issue_k(ka, npos, true);
-                logits_softmax(kb, true, false);
-                issue_v(va, npos, ka.boff, true);
-                accumulate_pv(vb, false);
-                pos = npos;
-                if (++i == n_full) break;
+            if (kHandScheduled) {
+                // drain the last (redundant) requests; all four staging buffers stay reserved until then
+                drain_loads(ka.q8, ka.sc);
+                drain_loads(kb.q8, kb.sc);
+                drain_loads(va.q8, va.sc);
+                drain_loads(vb.q8, vb.sc);
             }
-            pos += wg_tokens;
         }
-        if (pos < pe32) simple_block(pos);
 
-        // ---- merge the slots of each kv head through LDS, one query head at a time ----
+        // ---- merge the slots of each kv head through LDS, all query heads in one pass ----
         const bool whole = (pa == 0) && (pe == len);
         const int64_t piece = (int64_t)blockIdx.x + b;
         const int gslot = wave * SPW + slot;
-        const int dup = NSLOT / kvhb; // slots per kv head
+        const int dup = NSLOT >> kvhb_shift; // slots per kv head
 #pragma unroll
         for (int g = 0; g < GT; ++g) {
             // exp-sum of the slot = sum over the quad lanes' partial sums
             float lq = l_run[g] + dpp_f32<kDppXor1>(l_run[g]);
             lq += dpp_f32<kDppXor2>(lq);
-            __syncthreads();
             if (lane_on) {
+                float* dst = sm_acc + (g * NSLOT + gslot) * D + ch0;
 #pragma unroll
-                for (int c = 0; c < 16; c += 4) {
-                    *(f32x4*)&sm_acc[gslot * D + ch0 + c] = f32x4{acc[g][c], acc[g][c + 1], acc[g][c + 2], acc[g][c + 3]};
-                }
+                for (int c = 0; c < 16; c += 4) *(f32x4*)(dst + c) = f32x4{acc[g][c], acc[g][c + 1], acc[g][c + 2], acc[g][c + 3]};
                 if (ls == 0) {
-                    sm_m[gslot] = m_run[g];
-                    sm_l[gslot] = lq;
-                }
-            }
-            __syncthreads();
-            const int gi = g_first + g;
-            if (gi < G) {
-                for (int idx = tid; idx < kvhb * D; idx += kDecodeThreads) {
-                    const int hl = idx / D;
-                    const int c = idx - hl * D;
-                    // slots of kv head hl: every wave, slot index hl + kvhb * k
-                    float M = kNegBig;
-                    for (int k = 0; k < dup; ++k) {
-                        const int sidx = (k / tpl) * SPW + hl + kvhb * (k % tpl);
-                        M = fmaxf(M, sm_m[sidx]);
-                    }
-                    float L = 0.f, O = 0.f;
-                    for (int k = 0; k < dup; ++k) {
-                        const int sidx = (k / tpl) * SPW + hl + kvhb * (k % tpl);
-                        const float w = __builtin_amdgcn_exp2f(sm_m[sidx] - M);
-                        L += sm_l[sidx] * w;
-                        O += sm_acc[sidx * D + c] * w;
-                    }
-                    const float o = L > 0.f ? O / L : 0.f;
-                    const int h = (blockIdx.y * kvhb + hl) * G + gi;
-                    if (whole) {
-                        ((half_t*)a.output)[(int64_t)b * a.output_stride_s + (int64_t)h * D + c] = (half_t)o;
-                    } else {
-                        a.partial_out[(piece * a.num_heads + h) * D + c] = o;
-                        if (c == 0) {
-                            a.partial_ml[(piece * a.num_heads + h) * 2 + 0] = M;
-                            a.partial_ml[(piece * a.num_heads + h) * 2 + 1] = L;
-                        }
-                    }
+                    sm_m[g * NSLOT + gslot] = m_run[g];
+                    sm_l[g * NSLOT + gslot] = lq;
                 }
             }
         }
         __syncthreads();
+        // one output quad (4 channels of one (query head, kv head)) per thread and step
+        constexpr int QPH = D / 4; // quads per head
+        for (int idx = tid; idx < GT * kvhb * QPH; idx += kDecodeThreads) {
+            const int c = (idx % QPH) * 4;
+            const int gh = idx / QPH;
+            const int hl = gh & (kvhb - 1);
+            const int g = gh >> kvhb_shift;
+            const int gi = g_first + g;
+            if (gi >= G) continue;
+            // slots of kv head hl: slot hl + kvhb * (k % tpl) of wave k / tpl
+            float M = kNegBig;
+            for (int k = 0; k < dup; ++k) {
+                const int sidx = (k >> tpl_shift) * SPW + hl + ((k & (tpl - 1)) << kvhb_shift);
+                M = fmaxf(M, sm_m[g * NSLOT + sidx]);
+            }
+            float L = 0.f;
+            f32x4 O = {0.f, 0.f, 0.f, 0.f};
+            for (int k = 0; k < dup; ++k) {
+                const int sidx = (k >> tpl_shift) * SPW + hl + ((k & (tpl - 1)) << kvhb_shift);
+                const float w = __builtin_amdgcn_exp2f(sm_m[g * NSLOT + sidx] - M);
+                L += sm_l[g * NSLOT + sidx] * w;
+                const f32x4 v = *(const f32x4*)(sm_acc + (g * NSLOT + sidx) * D + c);
+                O += v * w;
+            }
+            const float inv = L > 0.f ? 1.f / L : 0.f;
+            O *= inv;
+            const int h = (blockIdx.y * kvhb + hl) * G + gi;
+            if (whole) {
+                half_t* out = (half_t*)a.output + (int64_t)b * a.output_stride_s + (int64_t)h * D + c;
+                typedef half_t half4_t __attribute__((ext_vector_type(4)));
+                *(half4_t*)out = half4_t{(half_t)O[0], (half_t)O[1], (half_t)O[2], (half_t)O[3]};
+            } else {
+                *(f32x4*)(a.partial_out + (piece * a.num_heads + h) * D + c) = O;
+                if (c == 0) {
+                    a.partial_ml[(piece * a.num_heads + h) * 2 + 0] = M;
+                    a.partial_ml[(piece * a.num_heads + h) * 2 + 1] = L;
+                }
+            }
+        }
+        __syncthreads(); // the next piece overwrites the LDS partials
     }
 #ifdef PMX_WG_TRACE
     if (tid == 0) {
@@ -583,8 +587,8 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
 #endif
 }
 
-// One workgroup per (sequence, query head): merges the pieces the decode kernel
-// left in the workspace.  Sequences that fit one range were already written.
+// One wave per (sequence, query head): merges the pieces the decode kernel left in the
+// workspace.  A sequence with a single piece was already written by the decode kernel.
 template <int D>
 __global__ __launch_bounds__(64) void decode_combine_kernel(const DecodeLaunch a)
 {
@@ -602,26 +606,62 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(const DecodeLaunch a
     }
     const int64_t per = tokens_per_range(total, a.ranges, a.wg_tokens, a.min_tokens_per_range);
     const int64_t w0 = s_beg / per, w1 = (s_end - 1) / per;
-    if (w0 == w1) return; // single piece, final output already written
+    if (w0 == w1) return; // one range covers the sequence: final output already written
+
+    // lanes over ranges: (max, exp-sum) of every non-empty piece, then the weights of the merge
     float M = kNegBig;
-    for (int64_t w = w0; w <= w1; ++w) M = fmaxf(M, a.partial_ml[((w + b) * a.num_heads + h) * 2]);
-    float o[(D + 63) / 64];
+    int pieces = 0;
+    for (int64_t wb = w0; wb <= w1; wb += 64) {
+        const int64_t w = wb + lane;
+        float m = kNegBig;
+        bool live = false;
+        if (w <= w1) {
+            int64_t pa, pe;
+            const int64_t r0 = w * per;
+            piece_bounds(r0, (r0 + per < total) ? r0 + per : total, s_beg, s_end - s_beg, a.wg_tokens, pa, pe);
+            live = pe > pa;
+            if (live) m = a.partial_ml[((w + b) * a.num_heads + h) * 2];
+        }
+        pieces += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live));
+        M = fmaxf(M, m);
+    }
+    if (pieces <= 1) return; // the cuts moved onto one boundary: the decode kernel wrote the final output
 #pragma unroll
-    for (int i = 0; i < (D + 63) / 64; ++i) o[i] = 0.f;
+    for (int s = 32; s >= 1; s >>= 1) M = fmaxf(M, __shfl_xor(M, s));
+
+    constexpr int NC = (D + 63) / 64;
+    float o[NC];
+#pragma unroll
+    for (int i = 0; i < NC; ++i) o[i] = 0.f;
     float den = 0.f;
-    for (int64_t w = w0; w <= w1; ++w) {
-        const int64_t pi = (w + b) * a.num_heads + h;
-        const float wt = a.partial_ml[pi * 2 + 1] * __builtin_amdgcn_exp2f(a.partial_ml[pi * 2] - M);
-        den += wt;
+    for (int64_t wb = w0; wb <= w1; wb += 64) {
+        const int64_t w = wb + lane;
+        float wt = 0.f;
+        if (w <= w1) {
+            int64_t pa, pe;
+            const int64_t r0 = w * per;
+            piece_bounds(r0, (r0 + per < total) ? r0 + per : total, s_beg, s_end - s_beg, a.wg_tokens, pa, pe);
+            if (pe > pa) {
+                const int64_t pi = (w + b) * a.num_heads + h;
+                wt = a.partial_ml[pi * 2 + 1] * __builtin_amdgcn_exp2f(a.partial_ml[pi * 2] - M);
+            }
+        }
+        const int n = (int)((w1 - wb < 63 ? w1 - wb : 63) + 1);
+        for (int k = 0; k < n; ++k) {
+            const float wk = __shfl(wt, k);
+            if (wk == 0.f) continue; // empty piece (or one without weight): its workspace row may be stale
+            den += wk;
+            const float* src = a.partial_out + ((wb + k + b) * a.num_heads + h) * D;
 #pragma unroll
-        for (int i = 0; i < (D + 63) / 64; ++i) {
-            const int c = lane + 64 * i;
-            if (c < D) o[i] += wt * a.partial_out[pi * D + c];
+            for (int i = 0; i < NC; ++i) {
+                const int c = lane + 64 * i;
+                if (c < D) o[i] += wk * src[c];
+            }
         }
     }
     const float inv = den > 0.f ? 1.f / den : 0.f;
 #pragma unroll
-    for (int i = 0; i < (D + 63) / 64; ++i) {
+    for (int i = 0; i < NC; ++i) {
         const int c = lane + 64 * i;
         if (c < D) out[c] = (half_t)(o[i] * inv);
     }
@@ -654,17 +694,28 @@ __global__ __launch_bounds__(64) void splitkv_combine_rows_kernel(
 
 // ---- host-side launchers (called from the C ABI) -------------------------------
 
+template <int D, int GT, bool PAGED, bool MASK>
+static void launch_decode_variant(const DecodeLaunch& a, dim3 grid, hipStream_t stream)
+{
+    constexpr size_t lds_bytes = decode_lds_bytes(D, GT);
+    // above the default limit of dynamic LDS per workgroup for the wider variants
+    static const hipError_t once = hipFuncSetAttribute((const void*)decode_attention_kernel<D, GT, PAGED, MASK>,
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    (void)once;
+    hipLaunchKernelGGL((decode_attention_kernel<D, GT, PAGED, MASK>), grid, dim3(kDecodeThreads), lds_bytes, stream, a);
+}
+
 template <int D, int GT>
 static void launch_decode_dgt(const DecodeLaunch& a, dim3 grid, hipStream_t stream)
 {
     const bool paged = a.cache_mode == 1;
     const bool mask = a.attn_mask != nullptr;
     if (paged) {
-        if (mask) hipLaunchKernelGGL((decode_attention_kernel<D, GT, true, true>), grid, dim3(kDecodeThreads), 0, stream, a);
-        else hipLaunchKernelGGL((decode_attention_kernel<D, GT, true, false>), grid, dim3(kDecodeThreads), 0, stream, a);
+        if (mask) launch_decode_variant<D, GT, true, true>(a, grid, stream);
+        else launch_decode_variant<D, GT, true, false>(a, grid, stream);
     } else {
-        if (mask) hipLaunchKernelGGL((decode_attention_kernel<D, GT, false, true>), grid, dim3(kDecodeThreads), 0, stream, a);
-        else hipLaunchKernelGGL((decode_attention_kernel<D, GT, false, false>), grid, dim3(kDecodeThreads), 0, stream, a);
+        if (mask) launch_decode_variant<D, GT, false, true>(a, grid, stream);
+        else launch_decode_variant<D, GT, false, false>(a, grid, stream);
     }
 }
 

@@ -101,6 +101,14 @@ __device__ __forceinline__ float dot2(half2_t a, half2_t b, float c)
 {
     return __builtin_amdgcn_fdot2(a, b, c, false);
 }
+// first link of a dot-product chain whose start value stays live: the three-address form writes a
+// new register, where the accumulating two-address form would first need a copy of c
+__device__ __forceinline__ float dot2_init(half2_t a, half2_t b, float c)
+{
+    float r;
+    asm("v_dot2_f32_f16 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
 
 // Index arrays (kvstarts, cachestarts) are read-only for the whole launch and are read at
 // wave-uniform addresses: viewing them through the constant address space lets the compiler use
