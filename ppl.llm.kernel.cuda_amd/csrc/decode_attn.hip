@@ -28,113 +28,11 @@
 //     output, running max, exp-sum) goes to the workspace and the combine kernel
 //     merges the pieces of each sequence (kernel.cu:617-665 is the reference's
 //     fused form of that merge).
-#include "device_common.h"
-#include "launch_params.h"
+#include <cstdlib>
+
+#include "decode_common.h"
 
 namespace pmxhip {
-
-namespace {
-
-constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kNegBig = -1.0e30f; // finite "no token yet" running max (log2 units)
-
-constexpr int kDecodeThreads = 256;
-constexpr int kDecodeWaves = kDecodeThreads / kWave;
-constexpr int kTB = 4; // tokens a slot handles per block (= lanes of a quad)
-static_assert(kTB == 4, "the quad reduce-scatter and the explicit wait counts assume four tokens per block");
-
-// ---- hand-scheduled cache loads of the pipelined loop ---------------------------------------
-// The loads of the steady-state loop are issued through inline assembly and awaited with explicit
-// wait counts.  Written as plain C++ loads, the compiler's automatic wait-count placement reuses
-// staging registers for temporaries and then waits for loads issued only moments earlier, which
-// serialises the memory latency into every iteration.  Vector memory operations complete in issue
-// order, so "at most N still outstanding" identifies exactly which loads have landed.
-__device__ __forceinline__ void load_b128(u32x4& dst, uint32_t lane_off, const char* wave_base)
-{
-    asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(dst) : "v"(lane_off), "s"(wave_base) : "memory");
-}
-__device__ __forceinline__ void load_b32(uint32_t& dst, uint32_t lane_off, const char* wave_base)
-{
-    asm volatile("global_load_dword %0, %1, %2" : "=&v"(dst) : "v"(lane_off), "s"(wave_base) : "memory");
-}
-// waits until at most N vector memory operations are outstanding; the values pass through the
-// statement so that no use of them can be scheduled before the wait
-template <int N>
-__device__ __forceinline__ void wait_loads(u32x4& a, uint32_t& b)
-{
-    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
-}
-// Waits for every outstanding load.  A register that is the target of an in-flight load must stay
-// allocated until a wait covers it, even when its value is never used (the redundant request of
-// the last block): passing it through this statement keeps it reserved, so that nothing else can
-// be placed in it and then be overwritten when the load lands.
-__device__ __forceinline__ void drain_loads(u32x4 (&q)[4], uint32_t (&sc)[4])
-{
-    asm volatile("s_waitcnt vmcnt(0)"
-                 : "+v"(q[0]), "+v"(q[1]), "+v"(q[2]), "+v"(q[3]), "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3]));
-}
-
-// value held by quad lane (lane ^ j), j in 0..3; j is a compile-time constant after unrolling
-__device__ __forceinline__ float quad_xor(float v, int j)
-{
-    switch (j) {
-        case 0: return v;
-        case 1: return dpp_f32<kDppXor1>(v);
-        case 2: return dpp_f32<kDppXor2>(v);
-        default: return dpp_f32<0x1B>(v); // quad_perm:[3,2,1,0]
-    }
-}
-
-// Tokens per range: equal shares rounded up to a whole number of workgroup
-// iterations, never below kMinTokensPerRange.  Shared by both kernels.
-__device__ __forceinline__ int64_t tokens_per_range(int64_t total, int ranges, int wg_tokens, int min_tokens)
-{
-    int64_t per = (total + ranges - 1) / ranges;
-    if (per < min_tokens) per = min_tokens;
-    return (per + wg_tokens - 1) / wg_tokens * wg_tokens;
-}
-
-// The piece [pa, pe) of a sequence (stream position s_beg, length len) that the range [r0, r1)
-// owns, in sequence coordinates.  A cut inside the sequence moves up to the next multiple of
-// `align` (a power of two) or to the sequence end; both neighbours compute the same cut, so the
-// pieces of a sequence still partition it.  pe <= pa: the range owns nothing of the sequence.
-__device__ __forceinline__ void piece_bounds(int64_t r0, int64_t r1, int64_t s_beg, int64_t len, int align,
-                                             int64_t& pa, int64_t& pe)
-{
-    const int64_t mask = (int64_t)align - 1;
-    int64_t lo = r0 - s_beg, hi = r1 - s_beg;
-    lo = lo <= 0 ? 0 : ((lo + mask) & ~mask);
-    hi = hi <= 0 ? 0 : ((hi + mask) & ~mask);
-    pa = lo < len ? lo : len;
-    pe = hi < len ? hi : len;
-}
-
-// first b in [0, n) with starts[b + 1] - starts[0] > g   (starts is non-decreasing)
-__device__ __forceinline__ int find_sequence(const_i64_ptr starts, int n, int64_t g)
-{
-    const int64_t base = starts[0];
-    int lo = 0, hi = n; // answer in [lo, hi]
-    while (lo < hi) {
-        const int mid = (lo + hi) >> 1;
-        if (starts[mid + 1] - base > g) hi = mid;
-        else lo = mid + 1;
-    }
-    return lo;
-}
-
-} // namespace
-
-// One block of kTB tokens for one slot: raw cache bytes as loaded, K and V staged separately.
-struct KBlock {
-    u32x4 q8[kTB];    // 16 int8 key channels per token
-    uint32_t sc[kTB]; // their two fp16 group scales
-    int pos;          // sequence position of the wave block's first token
-    int64_t boff;     // element offset of that token's row in the cache
-};
-struct VBlock {
-    u32x4 q8[kTB];
-    uint32_t sc[kTB];
-};
 
 // Bytes of dynamic LDS the decode kernel needs: one slot-partial (D floats) per slot and query
 // head, plus the (max, exp-sum) pair of each.
@@ -719,11 +617,23 @@ static void launch_decode_dgt(const DecodeLaunch& a, dim3 grid, hipStream_t stre
     }
 }
 
+// PMX_HIP_DECODE_GENERAL=1 keeps every shape on the general kernel (for comparisons)
+static bool general_kernel_forced()
+{
+    static const bool forced = [] {
+        const char* e = getenv("PMX_HIP_DECODE_GENERAL");
+        return e && e[0] == '1';
+    }();
+    return forced;
+}
+
 template <int D>
 static int launch_decode_d(const DecodeLaunch& a, int stage, hipStream_t stream)
 {
     const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / a.kv_heads_per_group), (unsigned)a.num_passes);
-    if (stage != 2) {
+    if (stage != 2 && D == 128 && decode_quad_applicable(a) && !general_kernel_forced()) {
+        launch_decode_quad(a, stream);
+    } else if (stage != 2) {
         switch (a.q_heads_per_pass) {
             case 1: launch_decode_dgt<D, 1>(a, grid, stream); break;
             case 2: launch_decode_dgt<D, 2>(a, grid, stream); break;

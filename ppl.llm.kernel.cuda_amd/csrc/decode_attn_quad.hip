@@ -1,0 +1,439 @@
+// Decode attention over the int8 group-8 KV cache, variant for head_dim 128, groups of at
+// most four query heads per kv head and kv heads in multiples of eight (the common GQA
+// shapes).  Same semantics, token ranges, pieces and workspace as decode_attn.hip
+// (reference: src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/kernel.cu:229-679,
+// 1115-1891); what differs is the lane layout, chosen so that the matrix pipe computes
+// the q.k products while the vector pipe converts and accumulates:
+//
+//   * A wave owns two kv heads.  The four lanes of a quad hold four different TOKENS of the
+//     same 16 channels; the eight quads of a half-wave hold the eight 16-channel chunks of
+//     those tokens; the two half-waves hold the two kv heads.  A block is 16 tokens: step j
+//     of a lane is token 4 j + (lane in quad).
+//   * v_mfma_f32_4x4x4_16b_f16 multiplies, per quad, a 4 x 4 A (row i from lane i) by a 4 x 4
+//     B (column j from lane j).  Row i = query head i (its 4 channels), column j = token j
+//     (the same 4 channels of K, converted int8 -> 1152 + x halves): one instruction gives
+//     each lane the four heads' partial dot products of its own token.  Two instructions
+//     cover one 8-channel scale group; the accumulator starts at -1152 * sum(q), which
+//     removes the conversion bias.
+//   * The partial logits (4 heads x 4 steps per lane, over 16 channels) are summed over the
+//     eight chunk lanes by a reduce-scatter (DPP adds with bank masks, a row swap), which
+//     leaves two complete logits per lane; exp2 runs on those; an all-gather hands every
+//     lane the 16 probabilities of its own tokens.  Lanes keep the heads in a lane-local
+//     order (slot s = head (own head) ^ s), so the gather needs no selects.
+//   * PV is per lane: int8 -> fp32 exactly, weights p * scale in fp32, v_fmac_f32.  Each lane
+//     accumulates its own token stream; the four streams of a quad are merged at the end of
+//     a piece.  Waves never exchange data: no LDS, no barriers.
+#include "decode_common.h"
+
+namespace pmxhip {
+
+namespace {
+
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kQuadD = 128;
+constexpr int kQuadHeads = 8;   // kv heads per workgroup (two per wave)
+constexpr int kQuadBlock = 16;  // tokens per block
+constexpr int kDppRor8 = 0x128; // row_ror:8 = lane ^ 8 inside a row of 16
+
+// exchanges the odd rows (of 16 lanes) of x with the even rows of y
+__device__ __forceinline__ void swap_rows(float& x, float& y)
+{
+    const u32x2_t r = __builtin_amdgcn_permlane16_swap(bitcast<uint32_t>(x), bitcast<uint32_t>(y), false, false);
+    x = bitcast<float>(r[0]);
+    y = bitcast<float>(r[1]);
+}
+// value of lane ^ 4 (data-share crossbar, no LDS memory involved): and 0x1f, or 0, xor 4
+__device__ __forceinline__ float lane_xor4(float v)
+{
+    return bitcast<float>(__builtin_amdgcn_ds_swizzle(bitcast<int>(v), (4 << 10) | 0x1f));
+}
+// lo + lo(lane ^ 4) on lanes with bit 2 clear, hi + hi(lane ^ 4) on lanes with bit 2 set.  The two
+// instructions write complementary banks of four lanes.  (A DPP operand must not be read within two
+// wait states of its producer; the compiler cannot see into the statement, hence the s_nop.)
+__device__ __forceinline__ float fold_xor4(float lo, float hi)
+{
+    float r;
+    asm("s_nop 1\n\t"
+        "v_add_f32_dpp %0, %1, %1 row_shl:4 row_mask:0xf bank_mask:0x5\n\t"
+        "v_add_f32_dpp %0, %2, %2 row_shr:4 row_mask:0xf bank_mask:0xa"
+        : "=&v"(r)
+        : "v"(lo), "v"(hi));
+    return r;
+}
+// lo + lo(lane ^ 8) on lanes with bit 3 clear, hi + hi(lane ^ 8) on lanes with bit 3 set
+__device__ __forceinline__ float fold_xor8(float lo, float hi)
+{
+    float r;
+    asm("s_nop 1\n\t"
+        "v_add_f32_dpp %0, %1, %1 row_ror:8 row_mask:0xf bank_mask:0x3\n\t"
+        "v_add_f32_dpp %0, %2, %2 row_ror:8 row_mask:0xf bank_mask:0xc"
+        : "=&v"(r)
+        : "v"(lo), "v"(hi));
+    return r;
+}
+// value held by quad lane i (compile-time i)
+template <int I>
+__device__ __forceinline__ float quad_lane(float v)
+{
+    return dpp_f32<I | (I << 2) | (I << 4) | (I << 6)>(v);
+}
+
+} // namespace
+
+template <bool PAGED>
+__global__ __launch_bounds__(kDecodeThreads, 2) void decode_attention_quad_kernel(const DecodeLaunch a)
+{
+    constexpr int D = kQuadD;
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int t4 = lane & 3;           // token within a step
+    const int chunk = (lane >> 2) & 7; // channels [16 chunk, 16 chunk + 16)
+    const int hsel = lane >> 5;        // which of the wave's two kv heads
+    // the head whose complete logits this lane receives from the reduce-scatter
+    const int g_own = (((lane >> 2) & 1) << 1) | ((lane >> 3) & 1);
+    const int row_odd = (lane >> 4) & 1;
+    const int G = (int)a.num_kv_repeats; // <= 4
+    const int kvh = blockIdx.y * kQuadHeads + wave * 2 + hsel;
+
+    const const_i64_ptr kvstarts = as_constant(a.kvstarts);
+    const const_i64_ptr cachestarts = as_constant(a.cachestarts);
+    const int64_t kv_base = kvstarts[0];
+    const int64_t total = kvstarts[a.decoding_batches] - kv_base;
+    const int64_t per = tokens_per_range(total, a.ranges, kQuadBlock, a.min_tokens_per_range);
+    const int64_t r0 = (int64_t)blockIdx.x * per;
+    if (r0 >= total) return;
+    const int64_t r1 = (r0 + per < total) ? r0 + per : total;
+
+    const int64_t group_off = a.layer_idx * a.cache_stride_l + (int64_t)(blockIdx.y * kQuadHeads) * a.cache_stride_h;
+    const uint32_t stride_s32 = (uint32_t)a.cache_stride_s; // the host checks that a block's span fits 32 bits
+    const uint32_t lane_base = (uint32_t)((int64_t)(wave * 2 + hsel) * a.cache_stride_h + chunk * 16);
+    const char* const cache_k = (const char*)a.cache + group_off;
+    const char* const cache_v = cache_k + a.cache_stride_kv;
+    const char* const scale_k = (const char*)a.scale + (group_off >> 3) * 2;
+    const char* const scale_v = scale_k + (a.cache_stride_kv >> 3) * 2;
+    const float logit_scale = a.attn_scale * kLog2e;
+
+    int b = find_sequence(kvstarts, (int)a.decoding_batches, r0);
+    for (; b < a.decoding_batches; ++b) {
+        const int64_t s_beg = kvstarts[b] - kv_base;
+        if (s_beg >= r1) break;
+        const int64_t len = kvstarts[b + 1] - kv_base - s_beg;
+        int64_t pa, pe;
+        piece_bounds(r0, r1, s_beg, len, kQuadBlock, pa, pe);
+        if (pe <= pa) continue;
+        const int pa32 = (int)pa, pe32 = (int)pe;
+        const int nb = (pe32 - pa32 + kQuadBlock - 1) / kQuadBlock; // >= 1
+        const bool tail_partial = ((pe32 - pa32) & (kQuadBlock - 1)) != 0;
+
+        const int64_t table_base = PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b;
+        const int64_t seq_row0 = PAGED ? 0 : cachestarts[b];
+        const int last_page = (pe32 - 1) >> 7;
+        int page_idx = -2;
+        int64_t page_row = 0, next_row = 0;
+        auto row_base_of = [&](int pos) -> int64_t { // page table entries are read one page ahead
+            if (!PAGED) return seq_row0 + pos;
+            const int pg = pos >> 7;
+            if (pg != page_idx) {
+                page_row = (pg == page_idx + 1) ? next_row : cachestarts[table_base + pg];
+                page_idx = pg;
+                const int nx = pg + 1 <= last_page ? pg + 1 : last_page;
+                next_row = cachestarts[table_base + nx];
+            }
+            return page_row + (pos & (kPage - 1));
+        };
+
+        uint32_t vo[kTB], vo_sc[kTB];
+#pragma unroll
+        for (int j = 0; j < kTB; ++j) {
+            vo[j] = (uint32_t)(4 * j + t4) * stride_s32 + lane_base;
+            vo_sc[j] = vo[j] >> 2;
+        }
+        auto clamp_offsets = [&](int pos) { // tokens beyond the piece re-read its last token; their logits are masked
+#pragma unroll
+            for (int j = 0; j < kTB; ++j) {
+                const int t = pos + 4 * j + t4;
+                const int tc = t < pe32 ? t : pe32 - 1;
+                vo[j] = (uint32_t)(tc - pos) * stride_s32 + lane_base;
+                vo_sc[j] = vo[j] >> 2;
+            }
+        };
+        auto request_k = [&](KBlock& kb, int pos) {
+            kb.pos = pos;
+            const int64_t boff = row_base_of(pos) * a.cache_stride_s;
+            kb.boff = boff;
+            const char* bk = cache_k + boff;
+            const char* sk = scale_k + (boff >> 3) * 2;
+#pragma unroll
+            for (int j = 0; j < kTB; ++j) {
+                load_b128(kb.q8[j], vo[j], bk);
+                load_b32(kb.sc[j], vo_sc[j], sk);
+            }
+        };
+        auto request_v = [&](VBlock& vb, int64_t boff) {
+            const char* bv = cache_v + boff;
+            const char* sv = scale_v + (boff >> 3) * 2;
+#pragma unroll
+            for (int j = 0; j < kTB; ++j) {
+                load_b128(vb.q8[j], vo[j], bv);
+                load_b32(vb.sc[j], vo_sc[j], sv);
+            }
+        };
+
+        KBlock ka, kb;
+        VBlock va, vb;
+        int pos = pa32;
+        if (nb == 1 && tail_partial) clamp_offsets(pos);
+        request_k(ka, pos);
+        request_v(va, ka.boff);
+
+        // ---- A operands: this lane supplies row t4 = query head t4, its chunk's 16 channels ----
+        half4_t qa[4];
+        f32x4 qbias0, qbias1; // accumulator start per scale group: row g = -1152 * sum of head g's 8 channels
+        {
+            const bool on = t4 < G;
+            const int h = kvh * G + (on ? t4 : 0);
+            const u32x4* qp = (const u32x4*)((const half_t*)a.query + (int64_t)b * a.query_stride_s + (int64_t)h * D + chunk * 16);
+            u32x4 lo = qp[0], hi = qp[1];
+            if (!on) { lo = u32x4{0, 0, 0, 0}; hi = lo; }
+            qa[0] = bitcast<half4_t>(u32x2_t{lo[0], lo[1]});
+            qa[1] = bitcast<half4_t>(u32x2_t{lo[2], lo[3]});
+            qa[2] = bitcast<half4_t>(u32x2_t{hi[0], hi[1]});
+            qa[3] = bitcast<half4_t>(u32x2_t{hi[2], hi[3]});
+            float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                s0 += (float)qa[0][i] + (float)qa[1][i];
+                s1 += (float)qa[2][i] + (float)qa[3][i];
+            }
+            s0 *= -1152.f;
+            s1 *= -1152.f;
+            qbias0 = f32x4{quad_lane<0>(s0), quad_lane<1>(s0), quad_lane<2>(s0), quad_lane<3>(s0)};
+            qbias1 = f32x4{quad_lane<0>(s1), quad_lane<1>(s1), quad_lane<2>(s1), quad_lane<3>(s1)};
+        }
+
+        // online-softmax state: m_run / l_run for head g_own only (l_run over this lane's own logits);
+        // acc[s] belongs to head g_own ^ s
+        float m_run = kNegBig, l_run = 0.f;
+        float acc[4][16];
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int c = 0; c < 16; ++c) acc[s][c] = 0.f;
+
+        float prob[4][kTB]; // [slot][step]: probabilities of this lane's own tokens
+        auto logits_softmax = [&](KBlock& kx) {
+            float part[4][kTB]; // [head][step], over this lane's 16 channels, log2 units
+#pragma unroll
+            for (int j = 0; j < kTB; ++j) {
+                if (j == 0) wait_loads<22>(kx.q8[0], kx.sc[0]);
+                if (j == 1) wait_loads<20>(kx.q8[1], kx.sc[1]);
+                if (j == 2) wait_loads<18>(kx.q8[2], kx.sc[2]);
+                if (j == 3) wait_loads<16>(kx.q8[3], kx.sc[3]);
+                f32x4 d0 = qbias0, d1 = qbias1;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const uint32_t f = kx.q8[j][w] ^ kFlipSigns;
+                    const half4_t kh = bitcast<half4_t>(u32x2_t{__builtin_amdgcn_perm(kExpBytes, f, 0x04010400u),
+                                                                __builtin_amdgcn_perm(kExpBytes, f, 0x04030402u)}); // 1152 + x
+                    if (w < 2) d0 = __builtin_amdgcn_mfma_f32_4x4x4f16(qa[w], kh, d0, 0, 0, 0);
+                    else d1 = __builtin_amdgcn_mfma_f32_4x4x4f16(qa[w], kh, d1, 0, 0, 0);
+                }
+                const half2_t sc = bitcast<half2_t>(kx.sc[j]);
+                const float s0 = (float)sc.x * logit_scale;
+                const float s1 = (float)sc.y * logit_scale;
+#pragma unroll
+                for (int g = 0; g < 4; ++g) part[g][j] = __builtin_fmaf(d1[g], s1, d0[g] * s0);
+            }
+            // reduce-scatter over the eight chunk lanes: lane bit 2 keeps heads {0,1} or {2,3}, bit 3 keeps
+            // one of the pair, the row pair keeps steps {0,2} or {1,3}
+            float l0, l1; // complete logits of head g_own: steps row_odd and 2 + row_odd
+            {
+                float rb[kTB];
+#pragma unroll
+                for (int j = 0; j < kTB; ++j) {
+                    const float ra0 = fold_xor4(part[0][j], part[2][j]);
+                    const float ra1 = fold_xor4(part[1][j], part[3][j]);
+                    rb[j] = fold_xor8(ra0, ra1);
+                }
+                swap_rows(rb[0], rb[1]);
+                swap_rows(rb[2], rb[3]);
+                l0 = rb[0] + rb[1];
+                l1 = rb[2] + rb[3];
+            }
+            const int tk = kx.pos + 4 * row_odd + t4;
+            l0 = tk < pe32 ? l0 : -INFINITY; // only in the last block: tokens beyond the piece
+            l1 = tk + 8 < pe32 ? l1 : -INFINITY;
+            // block max of the head: both lanes of the row pair
+            float mx = fmaxf(l0, l1), my = mx;
+            swap_rows(mx, my);
+            const float m_new = fmaxf(m_run, fmaxf(mx, my));
+            const bool moved = m_new > m_run;
+            float p0 = __builtin_amdgcn_exp2f(l0 - m_new);
+            float p1 = __builtin_amdgcn_exp2f(l1 - m_new);
+            if (__builtin_amdgcn_ballot_w64(moved) != 0) { // wave-uniform and rare: a running max moved
+                float al[4];
+                al[0] = __builtin_amdgcn_exp2f(m_run - m_new);
+                l_run *= al[0];
+                al[1] = dpp_f32<kDppRor8>(al[0]);
+                al[2] = lane_xor4(al[0]);
+                al[3] = lane_xor4(al[1]);
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+#pragma unroll
+                    for (int c = 0; c < 16; ++c) acc[s][c] *= al[s];
+            }
+            m_run = m_new;
+            l_run += p0 + p1;
+            // all-gather: steps over the row pair, heads over lane bits 3 and 2
+            float q0 = p0, q1 = p1;
+            swap_rows(p0, q0); // p0 = step 0, q0 = step 1
+            swap_rows(p1, q1); // p1 = step 2, q1 = step 3
+            prob[0][0] = p0; prob[0][1] = q0; prob[0][2] = p1; prob[0][3] = q1;
+#pragma unroll
+            for (int j = 0; j < kTB; ++j) prob[1][j] = dpp_f32<kDppRor8>(prob[0][j]);
+#pragma unroll
+            for (int j = 0; j < kTB; ++j) {
+                prob[2][j] = lane_xor4(prob[0][j]);
+                prob[3][j] = lane_xor4(prob[1][j]);
+            }
+        };
+
+        auto accumulate_pv = [&](VBlock& vx) {
+#pragma unroll
+            for (int j = 0; j < kTB; ++j) {
+                if (j == 0) wait_loads<22>(vx.q8[0], vx.sc[0]);
+                if (j == 1) wait_loads<20>(vx.q8[1], vx.sc[1]);
+                if (j == 2) wait_loads<18>(vx.q8[2], vx.sc[2]);
+                if (j == 3) wait_loads<16>(vx.q8[3], vx.sc[3]);
+                float x[16];
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    x[4 * w + 0] = byte_to_f32<0>(vx.q8[j][w]);
+                    x[4 * w + 1] = byte_to_f32<1>(vx.q8[j][w]);
+                    x[4 * w + 2] = byte_to_f32<2>(vx.q8[j][w]);
+                    x[4 * w + 3] = byte_to_f32<3>(vx.q8[j][w]);
+                }
+                const half2_t sc = bitcast<half2_t>(vx.sc[j]);
+                const float sv0 = (float)sc.x, sv1 = (float)sc.y;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const float w0 = prob[s][j] * sv0, w1 = prob[s][j] * sv1;
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) {
+                        acc[s][c] = __builtin_fmaf(w0, x[c], acc[s][c]);
+                        acc[s][8 + c] = __builtin_fmaf(w1, x[8 + c], acc[s][8 + c]);
+                    }
+                }
+            }
+        };
+
+        // software pipeline as in decode_attn.hip: K of block i+1 is requested before the logits of
+        // block i, V of block i+1 before the PV of block i; the last block re-requests itself
+        drain_loads(ka.q8, ka.sc);
+        drain_loads(va.q8, va.sc);
+        for (int i = 0;;) {
+            int npos = pos + (i + 1 < nb ? kQuadBlock : 0);
+            if (tail_partial && i + 2 == nb) clamp_offsets(npos);
+            request_k(kb, npos);
+            logits_softmax(ka);
+            request_v(vb, kb.boff);
+            accumulate_pv(va);
+            pos = npos;
+            if (++i == nb) break;
+            npos = pos + (i + 1 < nb ? kQuadBlock : 0);
+            if (tail_partial && i + 2 == nb) clamp_offsets(npos);
+            request_k(ka, npos);
+            logits_softmax(kb);
+            request_v(va, ka.boff);
+            accumulate_pv(vb);
+            pos = npos;
+            if (++i == nb) break;
+        }
+        drain_loads(ka.q8, ka.sc);
+        drain_loads(kb.q8, kb.sc);
+        drain_loads(va.q8, va.sc);
+        drain_loads(vb.q8, vb.sc);
+
+        // ---- end of the piece: exp-sum of the head over the row pair, (max, sum) of the four slots,
+        // then the four token streams of the quad are merged ----
+        {
+            float lx = l_run, ly = l_run;
+            swap_rows(lx, ly);
+            l_run = lx + ly;
+        }
+        float ms[4], lsum[4];
+        ms[0] = m_run;
+        lsum[0] = l_run;
+        ms[1] = dpp_f32<kDppRor8>(ms[0]);
+        lsum[1] = dpp_f32<kDppRor8>(lsum[0]);
+        ms[2] = lane_xor4(ms[0]);
+        ms[3] = lane_xor4(ms[1]);
+        lsum[2] = lane_xor4(lsum[0]);
+        lsum[3] = lane_xor4(lsum[1]);
+
+        const bool whole = (pa == 0) && (pe == len);
+        const int64_t piece = (int64_t)blockIdx.x + b;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            float M = fmaxf(ms[s], dpp_f32<kDppXor1>(ms[s]));
+            M = fmaxf(M, dpp_f32<kDppXor2>(M));
+            const float w = __builtin_amdgcn_exp2f(ms[s] - M);
+            float L = lsum[s] * w;
+            L += dpp_f32<kDppXor1>(L);
+            L += dpp_f32<kDppXor2>(L);
+            const float inv = L > 0.f ? 1.f / L : 0.f;
+            float o[16];
+#pragma unroll
+            for (int c = 0; c < 16; ++c) {
+                float v = acc[s][c] * w;
+                v += dpp_f32<kDppXor1>(v);
+                v += dpp_f32<kDppXor2>(v);
+                o[c] = v * inv;
+            }
+            const int g = g_own ^ s;
+            if (t4 == 0 && g < G) {
+                const int h = kvh * G + g;
+                if (whole) {
+                    typedef half_t half8_t __attribute__((ext_vector_type(8)));
+                    half_t* out = (half_t*)a.output + (int64_t)b * a.output_stride_s + (int64_t)h * D + chunk * 16;
+                    half8_t v0, v1;
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) {
+                        v0[c] = (half_t)o[c];
+                        v1[c] = (half_t)o[8 + c];
+                    }
+                    *(half8_t*)out = v0;
+                    *(half8_t*)(out + 8) = v1;
+                } else {
+                    float* out = a.partial_out + (piece * a.num_heads + h) * D + chunk * 16;
+#pragma unroll
+                    for (int c = 0; c < 16; c += 4) *(f32x4*)(out + c) = f32x4{o[c], o[c + 1], o[c + 2], o[c + 3]};
+                    if (chunk == 0) {
+                        a.partial_ml[(piece * a.num_heads + h) * 2 + 0] = M;
+                        a.partial_ml[(piece * a.num_heads + h) * 2 + 1] = L;
+                    }
+                }
+            }
+        }
+    }
+}
+
+// true when the variant above serves the launch; the caller falls back to the general kernel otherwise
+bool decode_quad_applicable(const DecodeLaunch& a)
+{
+    return a.head_dim == kQuadD && a.attn_mask == nullptr && a.kv_heads_per_group == kQuadHeads && a.num_kv_repeats <= 4 &&
+           a.num_passes == 1 && a.wg_tokens == kQuadBlock && a.output_stride_s % 8 == 0 &&
+           (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0;
+}
+
+void launch_decode_quad(const DecodeLaunch& a, hipStream_t stream)
+{
+    const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / kQuadHeads), 1);
+    if (a.cache_mode == 1) hipLaunchKernelGGL(decode_attention_quad_kernel<true>, grid, dim3(kDecodeThreads), 0, stream, a);
+    else hipLaunchKernelGGL(decode_attention_quad_kernel<false>, grid, dim3(kDecodeThreads), 0, stream, a);
+}
+
+} // namespace pmxhip

@@ -95,6 +95,8 @@ struct PrefillLaunch {
 int launch_kv_quantize(const QuantLaunch& a, hipStream_t stream);
 int launch_decode(const DecodeLaunch& a, int stage, hipStream_t stream); // stage: 0 both, 1 ranges, 2 combine
 int decode_wg_tokens(int head_dim, int kv_heads_per_group);
+bool decode_quad_applicable(const DecodeLaunch& a); // head_dim 128, <= 4 query heads per kv head, kv heads in eights
+void launch_decode_quad(const DecodeLaunch& a, hipStream_t stream);
 void launch_splitkv_combine_rows(const float* partial_out, const float* partial_ml, const int64_t* piece_begin,
                                  const int64_t* piece_end, int64_t rows, int64_t head_dim, void* output,
                                  hipStream_t stream);
