@@ -7,8 +7,9 @@ LIB_PATH = os.path.join(HERE, "libpmx_hip.so")
 
 
 def build(force=True, jobs=8):
-    """Runs make; with force=True every object is rebuilt."""
-    cmd = ["make", "-C", os.path.join(HERE, "csrc"), "-j%d" % jobs]
+    """Runs make; with force=True every object is rebuilt.  The `lint` target checks the assembly of
+    the kernels with hand-scheduled loads for register hazards and fails the build when it finds one."""
+    cmd = ["make", "-C", os.path.join(HERE, "csrc"), "-j%d" % jobs, "all", "lint"]
     if force:
         cmd.append("-B")
     subprocess.check_call(cmd)

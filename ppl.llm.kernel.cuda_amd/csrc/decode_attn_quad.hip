@@ -1,11 +1,14 @@
 // Decode attention over the int8 group-8 KV cache, variant for head_dim 128, groups of at
-// most four query heads per kv head and kv heads in multiples of eight (the common GQA
+// most eight query heads per kv head and kv heads in multiples of eight (the common GQA
 // shapes).  Same semantics, token ranges, pieces and workspace as decode_attn.hip
 // (reference: src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/kernel.cu:229-679,
 // 1115-1891); what differs is the lane layout, chosen so that the matrix pipe computes
 // the q.k products while the vector pipe converts and accumulates:
 //
-//   * A wave owns two kv heads.  The four lanes of a quad hold four different TOKENS of the
+//   * A wave owns two kv heads and up to four of their query heads; with more than four query
+//     heads per kv head a second set of four waves takes heads 4..7 of the same kv heads (it
+//     requests the same cache lines at about the same time, so they come from the cache levels
+//     and HBM is still read once).  The four lanes of a quad hold four different TOKENS of the
 //     same 16 channels; the eight quads of a half-wave hold the eight 16-channel chunks of
 //     those tokens; the two half-waves hold the two kv heads.  A block is 16 tokens: step j
 //     of a lane is token 4 j + (lane in quad).
@@ -82,20 +85,23 @@ __device__ __forceinline__ float quad_lane(float v)
 
 } // namespace
 
-template <bool PAGED>
-__global__ __launch_bounds__(kDecodeThreads, 2) void decode_attention_quad_kernel(const DecodeLaunch a)
+// GP: sets of four query heads per kv head (1 or 2); the workgroup has 4 * GP waves.
+template <bool PAGED, int GP>
+__global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_kernel(const DecodeLaunch a)
 {
     constexpr int D = kQuadD;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = wave_id & 3;      // which pair of kv heads
+    const int g_first = (wave_id >> 2) * 4; // first query head (within the kv head's group) of this wave
     const int t4 = lane & 3;           // token within a step
     const int chunk = (lane >> 2) & 7; // channels [16 chunk, 16 chunk + 16)
     const int hsel = lane >> 5;        // which of the wave's two kv heads
     // the head whose complete logits this lane receives from the reduce-scatter
     const int g_own = (((lane >> 2) & 1) << 1) | ((lane >> 3) & 1);
     const int row_odd = (lane >> 4) & 1;
-    const int G = (int)a.num_kv_repeats; // <= 4
+    const int G = (int)a.num_kv_repeats; // <= 4 * GP
     const int kvh = blockIdx.y * kQuadHeads + wave * 2 + hsel;
 
     const const_i64_ptr kvstarts = as_constant(a.kvstarts);
@@ -193,8 +199,8 @@ __global__ __launch_bounds__(kDecodeThreads, 2) void decode_attention_quad_kerne
         half4_t qa[4];
         f32x4 qbias0, qbias1; // accumulator start per scale group: row g = -1152 * sum of head g's 8 channels
         {
-            const bool on = t4 < G;
-            const int h = kvh * G + (on ? t4 : 0);
+            const bool on = g_first + t4 < G;
+            const int h = kvh * G + (on ? g_first + t4 : 0);
             const u32x4* qp = (const u32x4*)((const half_t*)a.query + (int64_t)b * a.query_stride_s + (int64_t)h * D + chunk * 16);
             u32x4 lo = qp[0], hi = qp[1];
             if (!on) { lo = u32x4{0, 0, 0, 0}; hi = lo; }
@@ -215,7 +221,7 @@ __global__ __launch_bounds__(kDecodeThreads, 2) void decode_attention_quad_kerne
         }
 
         // online-softmax state: m_run / l_run for head g_own only (l_run over this lane's own logits);
-        // acc[s] belongs to head g_own ^ s
+        // acc[s] belongs to head g_first + (g_own ^ s)
         float m_run = kNegBig, l_run = 0.f;
         float acc[4][16];
 #pragma unroll
@@ -393,7 +399,7 @@ __global__ __launch_bounds__(kDecodeThreads, 2) void decode_attention_quad_kerne
                 v += dpp_f32<kDppXor2>(v);
                 o[c] = v * inv;
             }
-            const int g = g_own ^ s;
+            const int g = g_first + (g_own ^ s);
             if (t4 == 0 && g < G) {
                 const int h = kvh * G + g;
                 if (whole) {
@@ -424,7 +430,7 @@ __global__ __launch_bounds__(kDecodeThreads, 2) void decode_attention_quad_kerne
 // true when the variant above serves the launch; the caller falls back to the general kernel otherwise
 bool decode_quad_applicable(const DecodeLaunch& a)
 {
-    return a.head_dim == kQuadD && a.attn_mask == nullptr && a.kv_heads_per_group == kQuadHeads && a.num_kv_repeats <= 4 &&
+    return a.head_dim == kQuadD && a.attn_mask == nullptr && a.kv_heads_per_group == kQuadHeads && a.num_kv_repeats <= 8 &&
            a.num_passes == 1 && a.wg_tokens == kQuadBlock && a.output_stride_s % 8 == 0 &&
            (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0;
 }
@@ -432,8 +438,14 @@ bool decode_quad_applicable(const DecodeLaunch& a)
 void launch_decode_quad(const DecodeLaunch& a, hipStream_t stream)
 {
     const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / kQuadHeads), 1);
-    if (a.cache_mode == 1) hipLaunchKernelGGL(decode_attention_quad_kernel<true>, grid, dim3(kDecodeThreads), 0, stream, a);
-    else hipLaunchKernelGGL(decode_attention_quad_kernel<false>, grid, dim3(kDecodeThreads), 0, stream, a);
+    const bool paged = a.cache_mode == 1;
+    if (a.num_kv_repeats <= 4) {
+        if (paged) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1>), grid, dim3(kDecodeThreads), 0, stream, a);
+        else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1>), grid, dim3(kDecodeThreads), 0, stream, a);
+    } else {
+        if (paged) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 2>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
+        else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 2>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
+    }
 }
 
 } // namespace pmxhip
