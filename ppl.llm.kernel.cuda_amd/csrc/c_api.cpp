@@ -299,6 +299,9 @@ int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t str
         return fail(PMXHIP_INVALID_VALUE, "prefill_attention: null device pointer");
     if (!aligned16(p->query) || p->query_stride_s % 8 != 0 || (reinterpret_cast<uintptr_t>(p->cache) & 7u))
         return fail(PMXHIP_UNSUPPORTED, "prefill_attention: query must be 16-byte aligned, cache 8-byte aligned");
+    // per-lane cache offsets inside a 64-token tile are 32-bit
+    if (p->cache_stride_s < 0 || 64.0 * (double)p->cache_stride_s + (double)p->head_dim >= 2147483648.0)
+        return fail(PMXHIP_UNSUPPORTED, "prefill_attention: cache_stride_s too large for 32-bit lane offsets");
 
     pmxhip::PrefillLaunch a{};
     a.query = p->query;

@@ -48,7 +48,7 @@ __device__ __forceinline__ int vt_pos16(int o) { return ((o & 4) << 1) | ((o & 8
 } // namespace
 
 template <int D, bool PAGED>
-__global__ __launch_bounds__(kPrefillThreads) void prefill_attention_kernel(const PrefillLaunch a)
+__global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(const PrefillLaunch a)
 {
     constexpr int KSTEPS = D / 16;          // MFMA k-steps over channels for S
     constexpr int CB = D / 32;              // 32-channel blocks of O^T
@@ -84,7 +84,8 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_attention_kernel(cons
     const int64_t q_row0 = a.seqstarts[b];
     const int qlen = (int)(a.seqstarts[b + 1] - q_row0);
     const int kvlen = (int)(a.kvstarts[b + 1] - a.kvstarts[b]);
-    const int p0 = blockIdx.x * ppw;
+    // query tiles in descending order: the workgroups that walk the most kv tokens are dispatched first
+    const int p0 = (int)(gridDim.x - 1 - blockIdx.x) * ppw;
     if (p0 >= qlen) return;
 
     // ---- this lane's column ----
@@ -143,29 +144,64 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_attention_kernel(cons
     u32x2 v_raw[4];
     half_t v_sc[4];
 
-    auto token_off = [&](int t) -> int64_t {
-        // row of token t (clamped into the sequence), times the token stride, plus the head offset
-        int tc = t < kvlen ? t : kvlen - 1;
-        if (tc < 0) tc = 0;
-        int64_t row;
-        if (PAGED) row = a.cachestarts[table_base + (tc >> 7)] + (tc & (kPage - 1));
-        else row = a.cachestarts[table_base] + tc;
-        return row * a.cache_stride_s + head_off;
+    // Addressing: a tile of 64 tokens starts at a multiple of 64, so it lies inside one page.  Its row
+    // base is wave-uniform (scalar loads of the page table, read one tile ahead); the per-lane part
+    // (token in tile, channel group) never changes and is computed once.
+    const const_i64_ptr cachestarts = as_constant(a.cachestarts);
+    auto tile_row = [&](int tile) -> int64_t {
+        int t_base = tile * kBN;
+        if (t_base > kvlen - 1) t_base = kvlen > 0 ? kvlen - 1 : 0;
+        if (PAGED) return cachestarts[table_base + (t_base >> 7)] + (t_base & (kPage - 1));
+        return cachestarts[table_base] + t_base;
     };
-    auto load_tile = [&](int tile) {
-        const int t_base = tile * kBN;
+    const uint32_t stride_s32 = (uint32_t)a.cache_stride_s; // the host checks that a tile's span fits 32 bits
+    constexpr int K_TSTEP = kPrefillThreads / GPT;           // tokens between a thread's K units
+    uint32_t k_off[K_UNITS], v_off[4];
 #pragma unroll
-        for (int u = 0; u < K_UNITS; ++u) {
-            const int64_t off = token_off(t_base + k_t0 + u * (kPrefillThreads / GPT)) + 8 * k_g;
-            k_raw[u] = *(const u32x2*)(cache + off);
-            k_sc[u] = scale[off >> 3];
-        }
-        if (v_on) {
+    for (int u = 0; u < K_UNITS; ++u) k_off[u] = (uint32_t)(k_t0 + u * K_TSTEP) * stride_s32 + 8 * k_g;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int64_t off = token_off(t_base + 4 * v_q + r) + a.cache_stride_kv + 8 * v_g;
-                v_raw[r] = *(const u32x2*)(cache + off);
-                v_sc[r] = scale[off >> 3];
+    for (int r = 0; r < 4; ++r) v_off[r] = (uint32_t)(4 * v_q + r) * stride_s32 + 8 * v_g;
+    const int8_t* const cache_k = cache + head_off;
+    const int8_t* const cache_v = cache_k + a.cache_stride_kv;
+    const half_t* const scale_k = scale + (head_off >> 3);
+    const half_t* const scale_v = scale_k + (a.cache_stride_kv >> 3);
+
+    auto load_tile = [&](int tile, int64_t row) {
+        const int64_t boff = row * a.cache_stride_s;
+        const int8_t* bk = cache_k + boff;
+        const int8_t* bv = cache_v + boff;
+        const half_t* sk = scale_k + (boff >> 3);
+        const half_t* sv = scale_v + (boff >> 3);
+        const int left = kvlen - 1 - tile * kBN; // offset of the sequence's last token inside this tile
+        if (left >= kBN - 1) {
+#pragma unroll
+            for (int u = 0; u < K_UNITS; ++u) {
+                k_raw[u] = *(const u32x2*)(bk + k_off[u]);
+                k_sc[u] = sk[k_off[u] >> 3];
+            }
+            if (v_on) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    v_raw[r] = *(const u32x2*)(bv + v_off[r]);
+                    v_sc[r] = sv[v_off[r] >> 3];
+                }
+            }
+        } else { // last tile of the sequence: tokens beyond it re-read its last token (masked later)
+#pragma unroll
+            for (int u = 0; u < K_UNITS; ++u) {
+                const int t = k_t0 + u * K_TSTEP;
+                const uint32_t off = (uint32_t)(t < left ? t : (left > 0 ? left : 0)) * stride_s32 + 8 * k_g;
+                k_raw[u] = *(const u32x2*)(bk + off);
+                k_sc[u] = sk[off >> 3];
+            }
+            if (v_on) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int t = 4 * v_q + r;
+                    const uint32_t off = (uint32_t)(t < left ? t : (left > 0 ? left : 0)) * stride_s32 + 8 * v_g;
+                    v_raw[r] = *(const u32x2*)(bv + off);
+                    v_sc[r] = sv[off >> 3];
+                }
             }
         }
     };
@@ -218,12 +254,19 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_attention_kernel(cons
         }
     };
 
-    if (n_tiles > 0) load_tile(0);
+    int64_t row_next = 0;
+    if (n_tiles > 0) {
+        load_tile(0, tile_row(0));
+        row_next = tile_row(1);
+    }
     for (int tile = 0; tile < n_tiles; ++tile) {
         __syncthreads(); // everyone is done reading the previous tile
         store_tile();
         __syncthreads();
-        if (tile + 1 < n_tiles) load_tile(tile + 1);
+        if (tile + 1 < n_tiles) {
+            load_tile(tile + 1, row_next);
+            row_next = tile_row(tile + 2);
+        }
 
         // ---- S^T = K Q^T : two 32-token blocks ----
         f32x16 s_acc[2];
@@ -243,42 +286,49 @@ __global__ __launch_bounds__(kPrefillThreads) void prefill_attention_kernel(cons
         // ---- online softmax per column (element i <-> token 32 mb + 8 (i/4) + 4 hh + i%4) ----
         const int t_base = tile * kBN;
         const bool need_mask = t_base + kBN > lim;
-        float mx = kNegBig;
+        float mx = kNegBig; // of the raw dot products; the (positive) logit scale is applied to the maximum
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                float v = s_acc[mb][i] * sm_scale;
                 if (need_mask) {
                     const int t = t_base + 32 * mb + 8 * (i >> 2) + 4 * hh + (i & 3);
-                    if (t >= lim) v = -INFINITY;
+                    if (t >= lim) s_acc[mb][i] = -INFINITY;
                 }
-                s_acc[mb][i] = v;
-                mx = fmaxf(mx, v);
+                mx = fmaxf(mx, s_acc[mb][i]);
             }
+        mx *= sm_scale;
         mx = fmaxf(mx, __shfl_xor(mx, 32));
         const float m_new = fmaxf(m_run, mx);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new;
-        const float bias = kPShift - m_new;
+        // the running max moves rarely once a few tiles have been seen: rescale only then (wave-uniform)
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            l_run *= alpha;
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o_acc[cb][i] *= alpha;
+            m_run = m_new;
+        }
+        const float bias = kPShift - m_run;
+        // p = hi + lo in halves: hi = p rounded toward zero (two at a time), lo = the exact remainder
         f16x8 pf[2][2], pfl[2][2];
         float lsum = 0.f;
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const float pv = __builtin_amdgcn_exp2f(s_acc[mb][i] + bias);
-                const half_t ph = (half_t)pv;
-                const half_t pl = (half_t)(pv - (float)ph);
-                lsum += (float)ph + (float)pl; // the sum uses exactly what the PV product uses
-                pf[mb][i >> 3][i & 7] = ph;
-                pfl[mb][i >> 3][i & 7] = pl;
+            for (int i = 0; i < 16; i += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[mb][i], sm_scale, bias));
+                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[mb][i + 1], sm_scale, bias));
+                lsum += p0 + p1;
+                const half2_t ph = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(p0, p1));
+                const half2_t pl = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(p0 - (float)ph.x, p1 - (float)ph.y));
+                pf[mb][i >> 3][i & 7] = ph.x;
+                pf[mb][i >> 3][(i & 7) + 1] = ph.y;
+                pfl[mb][i >> 3][i & 7] = pl.x;
+                pfl[mb][i >> 3][(i & 7) + 1] = pl.y;
             }
-        l_run = l_run * alpha + lsum;
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) o_acc[cb][i] *= alpha;
+        l_run += lsum;
 
         // ---- O^T += V^T P^T ----
 #pragma unroll
