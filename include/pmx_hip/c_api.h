@@ -163,7 +163,8 @@ PMXHIP_API int pmxhip_splitkv_combine(const float* partial_out, const float* par
 
 /* ---- multi-query-token (chunked prefill) attention over the int8 cache -----
  * Replaces the flash_attn2_paged_fmha call of forward_prefill
- * (kernel.cu:2127-2179; include/ppl/kernel/llm/cuda/flash_attn2/fmha.h:73).
+ * (kernel.cu:2127-2179; include/ppl/kernel/llm/cuda/flash_attn2/fmha.h:73) and, with
+ * current_key set, its flash_attn2_fmha call (kernel.cu:2181-2212).
  * Sequences [decoding_batches, batch) are prefill; query/output rows are
  * addressed through seqstarts, kv length through kvstarts, cache rows through
  * cachestarts; causal masking is bottom-right aligned (mask.h:186). */
@@ -194,6 +195,23 @@ typedef struct pmxhip_prefill_params {
     int64_t cache_stride_h;
     int64_t cache_stride_kv;
     int64_t cachestarts_stride_b;
+    /* Optional inputs of the two flash_attn2 calls (kernel.cu:2153-2158, 2188-2193); zero = absent.
+     * attn_mask: additive half bias; element (head h, absolute query row r, absolute kv column c)
+     * at h*mask_stride_h + r*mask_stride_s + c, c = kvstarts[b] + t (seqstarts[b] + t when
+     * current_key is given); added to the scaled logit (flash_api.cu:171).
+     * alibi_slopes: float32 (Hq); causal: + slope*t, otherwise - slope*|row + kvlen - qlen - t|
+     * (flash_attn2/src/mask.h:191-197). */
+    const void* attn_mask;
+    int64_t mask_stride_s;
+    int64_t mask_stride_h;
+    const float* alibi_slopes;
+    /* enable_cache_prefill = false (kernel.cu:2181-2212): with current_key != NULL the stage
+     * attends over the step's own half K/V rows (S, KVH, D) only -- kv length = query length,
+     * no cache read; cache/scale/cachestarts/kvstarts are then ignored. */
+    const void* current_key;
+    const void* current_value;
+    int64_t key_stride_s;
+    int64_t value_stride_s;
 } pmxhip_prefill_params;
 
 PMXHIP_API int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t stream);

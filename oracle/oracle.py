@@ -52,6 +52,10 @@ def lib():
         _lib.pmx_oracle_prefill_attention.restype = ctypes.c_int
         _lib.pmx_oracle_prefill_attention.argtypes = (
             [_vp] * 6 + [_i64, _i64, _i32] + [_i64] * 3 + [_f32, _i64, _i32] + [_i64] * 7 + [_vp])
+        _lib.pmx_oracle_prefill_attention_ex.restype = ctypes.c_int
+        _lib.pmx_oracle_prefill_attention_ex.argtypes = (
+            [_vp] * 5 + [_i64, _i64] + [_vp, _i64, _i64] + [_vp] + [_vp] * 3 + [_i64, _i64, _i32] + [_i64] * 3 +
+            [_f32, _i64, _i32] + [_i64] * 7 + [_vp])
         _lib.pmx_oracle_decode_partial.restype = ctypes.c_int
         _lib.pmx_oracle_decode_partial.argtypes = (
             [_vp] * 4 + [_i64] * 7 + [_f32, _i64, _i32] + [_i64] * 6 + [_vp] * 3)
@@ -174,6 +178,39 @@ def prefill_attention(query, cache, scale, seqstarts, kvstarts, cachestarts, bat
     stride = num_heads * head_dim
     rc = lib().pmx_oracle_prefill_attention(
         _p(query), _p(cache), _p(scale), _p(seqstarts), _p(kvstarts), _p(cachestarts),
+        batch, decoding_batches, 1 if is_causal else 0, num_heads, num_kv_heads, head_dim,
+        attn_scale, layer_idx, page_size, stride, stride,
+        cache_stride_s, cache_stride_l, cache_stride_h, cache_stride_kv, cachestarts_stride_b,
+        _p(out))
+    if rc != 0:
+        raise ValueError("oracle prefill rejected the arguments (rc=%d)" % rc)
+    return out
+
+
+def prefill_attention_ex(query, cache, scale, seqstarts, kvstarts, cachestarts, batch,
+                         decoding_batches, is_causal, num_heads, num_kv_heads, head_dim,
+                         attn_scale, layer_idx, page_size,
+                         cache_stride_s, cache_stride_l, cache_stride_h, cache_stride_kv,
+                         cachestarts_stride_b, current_key=None, current_value=None,
+                         attn_mask=None, mask_stride_s=0, mask_stride_h=0, alibi_slopes=None):
+    """Prefill with the optional inputs: fp16 current_key/current_value [rows, KVH, D] instead of
+    the cache, additive fp16 attn_mask, float32 alibi_slopes [Hq].  Returns float32
+    [total_query_rows, num_heads, head_dim]; decode rows stay 0."""
+    query = _c(query, np.float16)
+    seqstarts = _c(seqstarts, np.int64)
+    kvstarts = _c(kvstarts, np.int64)
+    cachestarts = _c(cachestarts, np.int64)
+    ck = None if current_key is None else _c(current_key, np.float16)
+    cv = None if current_value is None else _c(current_value, np.float16)
+    am = None if attn_mask is None else _c(attn_mask, np.float16)
+    al = None if alibi_slopes is None else _c(alibi_slopes, np.float32)
+    out = np.zeros((query.shape[0], num_heads, head_dim), dtype=np.float32)
+    stride = num_heads * head_dim
+    kstride = num_kv_heads * head_dim
+    rc = lib().pmx_oracle_prefill_attention_ex(
+        _p(query), _p(cache), _p(scale), _p(ck), _p(cv), kstride, kstride,
+        _p(am), mask_stride_s, mask_stride_h, _p(al),
+        _p(seqstarts), _p(kvstarts), _p(cachestarts),
         batch, decoding_batches, 1 if is_causal else 0, num_heads, num_kv_heads, head_dim,
         attn_scale, layer_idx, page_size, stride, stride,
         cache_stride_s, cache_stride_l, cache_stride_h, cache_stride_kv, cachestarts_stride_b,

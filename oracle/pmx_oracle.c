@@ -19,6 +19,10 @@
  *                                  cache, naive python loops on tiny inputs.
  *   pmx_oracle_prefill_attention   pinned: torch SDPA with explicit bottom-right
  *                                  causal mask, qlen=1 rows equal decode.
+ *   pmx_oracle_prefill_attention_ex pinned: equals pmx_oracle_prefill_attention without the
+ *                                  optional inputs; torch SDPA with an additive float mask
+ *                                  (bias + alibi + causal) on the dequantised cache and on
+ *                                  fp16 K/V.
  *   pmx_oracle_splitkv_combine     pinned: any split of the kv range equals the
  *                                  single pass (log-sum-exp associativity).
  *   The reference itself cannot be compiled here (CUDA, inline PTX, CUTLASS, and
@@ -342,6 +346,117 @@ int pmx_oracle_prefill_attention(
                                cache_stride_s, cache_stride_kv, head_dim, attn_scale, logits,
                                output + row * output_stride_s + h * head_dim, NULL, NULL);
             }
+            free(logits);
+        }
+    }
+    return 0;
+}
+
+/* Prefill with every optional input of the two flash_attn2 calls of forward_prefill
+ * (KC:2134-2212):
+ *   - K/V either from the int8 cache (enable_cache_prefill, KC:2134-2179) or, with
+ *     current_key != NULL, from the step's own fp16 current_key/current_value rows with
+ *     kv length = query length (seqstart_k = seqstart_q, KC:2181-2212);
+ *   - attn_mask: additive fp16 bias, block-diagonal over the batch: element (head h, absolute
+ *     query row r, absolute kv column c) at h*mask_stride_h + r*mask_stride_s + c, added to the
+ *     scaled logit (flash_attn2/src/flash_api.cu:171 scales it by 1/attn_scale before the
+ *     softmax scale is applied; block_info.h:48-58 gives the offsets);
+ *   - alibi_slopes: float32 per head; causal: + slope * col, otherwise
+ *     - slope * |row + kvlen - qlen - col| (flash_attn2/src/mask.h:191-197, slope divided by
+ *     the softmax scale at flash_fwd_kernel.h:764, i.e. applied to the scaled logit).
+ * kv columns are absolute positions in the kv stream: kvstarts[b] + t for the cache path,
+ * seqstarts[b] + t for the current_key path. */
+int pmx_oracle_prefill_attention_ex(
+    const uint16_t* query,
+    const int8_t* cache, const uint16_t* scale,
+    const uint16_t* current_key, const uint16_t* current_value, int64_t key_stride_s, int64_t value_stride_s,
+    const uint16_t* attn_mask, int64_t mask_stride_s, int64_t mask_stride_h,
+    const float* alibi_slopes,
+    const int64_t* seqstarts, const int64_t* kvstarts, const int64_t* cachestarts,
+    int64_t batch, int64_t decoding_batches, int32_t is_causal,
+    int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+    float attn_scale, int64_t layer_idx, int32_t page_size,
+    int64_t query_stride_s, int64_t output_stride_s,
+    int64_t cache_stride_s, int64_t cache_stride_l, int64_t cache_stride_h, int64_t cache_stride_kv,
+    int64_t cachestarts_stride_b,
+    float* output)
+{
+    if (num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || head_dim % 8 != 0 || head_dim > 256)
+        return 2;
+    const int64_t repeats = num_heads / num_kv_heads;
+    const int from_current = current_key != NULL;
+    for (int64_t b = decoding_batches; b < batch; ++b) {
+        const int64_t qlen = seqstarts[b + 1] - seqstarts[b];
+        const int64_t kvlen = from_current ? qlen : kvstarts[b + 1] - kvstarts[b];
+        const int64_t col0 = from_current ? seqstarts[b] : kvstarts[b];
+        const int64_t work = qlen * num_heads;
+#pragma omp parallel
+        {
+            double* logits = (double*)malloc(sizeof(double) * (size_t)(kvlen > 0 ? kvlen : 1));
+            float* kv = (float*)malloc(sizeof(float) * (size_t)head_dim);
+#pragma omp for schedule(dynamic, 8)
+            for (int64_t w = 0; w < work; ++w) {
+                const int64_t i = w / num_heads, h = w % num_heads;
+                const int64_t kvh = h / repeats;
+                int64_t limit = kvlen;
+                if (is_causal) {
+                    limit = i + 1 + kvlen - qlen;
+                    if (limit > kvlen) limit = kvlen;
+                    if (limit < 0) limit = 0;
+                }
+                const int64_t row = seqstarts[b] + i;
+                const uint16_t* q_row = query + row * query_stride_s + h * head_dim;
+                double mx = -INFINITY;
+                for (int64_t t = 0; t < limit; ++t) {
+                    double acc = 0.0;
+                    if (from_current) {
+                        const uint16_t* k = current_key + (seqstarts[b] + t) * key_stride_s + kvh * head_dim;
+                        for (int64_t d = 0; d < head_dim; ++d)
+                            acc += (double)pmx_oracle_half_to_float(q_row[d]) * (double)pmx_oracle_half_to_float(k[d]);
+                    } else {
+                        const int64_t tok = cache_token_index(cachestarts, cachestarts_stride_b, b, t, page_size);
+                        const int64_t k_off = tok * cache_stride_s + layer_idx * cache_stride_l + kvh * cache_stride_h;
+                        for (int64_t d0 = 0; d0 < head_dim; d0 += 8) {
+                            const float sc = pmx_oracle_half_to_float(scale[(k_off + d0) >> 3]);
+                            for (int64_t d = d0; d < d0 + 8; ++d)
+                                acc += (double)pmx_oracle_half_to_float(q_row[d]) * (double)((float)cache[k_off + d] * sc);
+                        }
+                    }
+                    double l = (double)attn_scale * acc;
+                    if (attn_mask)
+                        l += (double)pmx_oracle_half_to_float(attn_mask[h * mask_stride_h + row * mask_stride_s + col0 + t]);
+                    if (alibi_slopes) {
+                        if (is_causal)
+                            l += (double)alibi_slopes[h] * (double)t;
+                        else
+                            l -= (double)alibi_slopes[h] * fabs((double)(i + kvlen - qlen - t));
+                    }
+                    logits[t] = l;
+                    if (l > mx) mx = l;
+                }
+                double o[256];
+                for (int64_t d = 0; d < head_dim; ++d) o[d] = 0.0;
+                double sum = 0.0;
+                for (int64_t t = 0; t < limit; ++t) {
+                    const double p = (mx == -INFINITY) ? 0.0 : exp(logits[t] - mx);
+                    sum += p;
+                    if (from_current) {
+                        const uint16_t* v = current_value + (seqstarts[b] + t) * value_stride_s + kvh * head_dim;
+                        for (int64_t d = 0; d < head_dim; ++d) o[d] += p * (double)pmx_oracle_half_to_float(v[d]);
+                    } else {
+                        const int64_t tok = cache_token_index(cachestarts, cachestarts_stride_b, b, t, page_size);
+                        const int64_t v_off = tok * cache_stride_s + layer_idx * cache_stride_l + kvh * cache_stride_h + cache_stride_kv;
+                        for (int64_t d0 = 0; d0 < head_dim; d0 += 8) {
+                            const float sc = pmx_oracle_half_to_float(scale[(v_off + d0) >> 3]);
+                            for (int64_t d = d0; d < d0 + 8; ++d) o[d] += p * (double)((float)cache[v_off + d] * sc);
+                        }
+                    }
+                }
+                const double inv = sum > 0.0 ? 1.0 / sum : 0.0;
+                float* out = output + row * output_stride_s + h * head_dim;
+                for (int64_t d = 0; d < head_dim; ++d) out[d] = (float)(o[d] * inv);
+            }
+            free(kv);
             free(logits);
         }
     }

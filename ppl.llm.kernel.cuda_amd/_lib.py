@@ -82,6 +82,8 @@ class PrefillParams(ctypes.Structure):
         ("query_stride_s", c_i64), ("output_stride_s", c_i64),
         ("cache_stride_s", c_i64), ("cache_stride_l", c_i64), ("cache_stride_h", c_i64),
         ("cache_stride_kv", c_i64), ("cachestarts_stride_b", c_i64),
+        ("attn_mask", c_vp), ("mask_stride_s", c_i64), ("mask_stride_h", c_i64), ("alibi_slopes", c_vp),
+        ("current_key", c_vp), ("current_value", c_vp), ("key_stride_s", c_i64), ("value_stride_s", c_i64),
     ]
 
 

@@ -292,16 +292,30 @@ int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t str
         return fail(PMXHIP_UNSUPPORTED, "prefill_attention: head dim %lld not supported (64, 128)", (long long)p->head_dim);
     if (p->num_kv_heads <= 0 || p->num_heads % p->num_kv_heads != 0)
         return fail(PMXHIP_UNSUPPORTED, "only support num_heads %% num_kv_heads == 0.");
-    if (int rc = check_cache_layout("prefill_attention", p->cache_mode, p->page_size, p->cache_stride_s, p->cache_stride_l,
-                                    p->cache_stride_h, p->cache_stride_kv, 8))
-        return rc;
-    if (!p->query || !p->output || !p->cache || !p->scale || !p->seqstarts || !p->kvstarts || !p->cachestarts)
-        return fail(PMXHIP_INVALID_VALUE, "prefill_attention: null device pointer");
-    if (!aligned16(p->query) || p->query_stride_s % 8 != 0 || (reinterpret_cast<uintptr_t>(p->cache) & 7u))
-        return fail(PMXHIP_UNSUPPORTED, "prefill_attention: query must be 16-byte aligned, cache 8-byte aligned");
-    // per-lane cache offsets inside a 64-token tile are 32-bit
-    if (p->cache_stride_s < 0 || 64.0 * (double)p->cache_stride_s + (double)p->head_dim >= 2147483648.0)
-        return fail(PMXHIP_UNSUPPORTED, "prefill_attention: cache_stride_s too large for 32-bit lane offsets");
+    const bool from_current = p->current_key != nullptr;
+    if (from_current) {
+        if (!p->current_value || !p->query || !p->output || !p->seqstarts)
+            return fail(PMXHIP_INVALID_VALUE, "prefill_attention: null device pointer");
+        if (!aligned16(p->current_key) || !aligned16(p->current_value) || p->key_stride_s % 8 != 0 || p->value_stride_s % 8 != 0 ||
+            p->key_stride_s <= 0 || p->value_stride_s <= 0 || 64.0 * (double)p->key_stride_s >= 2147483648.0 ||
+            64.0 * (double)p->value_stride_s >= 2147483648.0)
+            return fail(PMXHIP_UNSUPPORTED, "prefill_attention: current_key/value must be 16-byte aligned with row strides that are multiples of 8");
+    } else {
+        if (int rc = check_cache_layout("prefill_attention", p->cache_mode, p->page_size, p->cache_stride_s, p->cache_stride_l,
+                                        p->cache_stride_h, p->cache_stride_kv, 8))
+            return rc;
+        if (!p->query || !p->output || !p->cache || !p->scale || !p->seqstarts || !p->kvstarts || !p->cachestarts)
+            return fail(PMXHIP_INVALID_VALUE, "prefill_attention: null device pointer");
+        if (reinterpret_cast<uintptr_t>(p->cache) & 7u)
+            return fail(PMXHIP_UNSUPPORTED, "prefill_attention: cache must be 8-byte aligned");
+        // per-lane cache offsets inside a 64-token tile are 32-bit
+        if (p->cache_stride_s < 0 || 64.0 * (double)p->cache_stride_s + (double)p->head_dim >= 2147483648.0)
+            return fail(PMXHIP_UNSUPPORTED, "prefill_attention: cache_stride_s too large for 32-bit lane offsets");
+    }
+    if (!aligned16(p->query) || p->query_stride_s % 8 != 0)
+        return fail(PMXHIP_UNSUPPORTED, "prefill_attention: query must be 16-byte aligned with a row stride that is a multiple of 8");
+    if ((reinterpret_cast<uintptr_t>(p->output) & 7u) || p->output_stride_s % 4 != 0)
+        return fail(PMXHIP_UNSUPPORTED, "prefill_attention: output must be 8-byte aligned with a row stride that is a multiple of 4");
 
     pmxhip::PrefillLaunch a{};
     a.query = p->query;
@@ -309,8 +323,21 @@ int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t str
     a.cache = p->cache;
     a.scale = p->scale;
     a.seqstarts = p->seqstarts + p->decoding_batches;                          // kernel.cu:2131
-    a.kvstarts = p->kvstarts + p->decoding_batches;                            // kernel.cu:2132
-    a.cachestarts = p->cachestarts + p->decoding_batches * p->cachestarts_stride_b; // kernel.cu:2142
+    if (from_current) {
+        a.kvstarts = a.seqstarts;                                              // kernel.cu:2196: seqstart_k = seqstart_q
+        a.cachestarts = nullptr;
+        a.current_key = p->current_key;
+        a.current_value = p->current_value;
+        a.key_stride_s = p->key_stride_s;
+        a.value_stride_s = p->value_stride_s;
+    } else {
+        a.kvstarts = p->kvstarts + p->decoding_batches;                        // kernel.cu:2132
+        a.cachestarts = p->cachestarts + p->decoding_batches * p->cachestarts_stride_b; // kernel.cu:2142
+    }
+    a.attn_mask = p->attn_mask;
+    a.mask_stride_s = p->mask_stride_s;
+    a.mask_stride_h = p->mask_stride_h;
+    a.alibi_slopes = p->alibi_slopes;
     a.attn_scale = p->attn_scale;
     a.is_causal = p->is_causal;
     a.cache_mode = p->cache_mode;

@@ -288,16 +288,6 @@ ppl::common::RetCode dynamic_batching_multi_head_cache_attention::forward_prefil
         PMX_LOG_ERROR("prefill attention only supports fp16");
         return ppl::common::RC_UNSUPPORTED;
     }
-    if (!cfg.enable_cache_prefill) {
-        // kernel.cu:2181-2212: attention over the fp16 current_key/value only, no cache read
-        PMX_LOG_ERROR("prefill over fp16 current_key/value (enable_cache_prefill = false) is not built; "
-                      "use enable_cache_prefill = true");
-        return ppl::common::RC_UNSUPPORTED;
-    }
-    if (cfg.attn_mask || cfg.alibi_slopes) {
-        PMX_LOG_ERROR("prefill attention: attn_mask / alibi_slopes are not built on this path");
-        return ppl::common::RC_UNSUPPORTED;
-    }
     pmxhip_prefill_params p;
     memset(&p, 0, sizeof(p));
     p.query = cfg.query;
@@ -326,6 +316,16 @@ ppl::common::RetCode dynamic_batching_multi_head_cache_attention::forward_prefil
     p.cache_stride_h = cfg.cache_stride_h;
     p.cache_stride_kv = cfg.cache_stride_kv;
     p.cachestarts_stride_b = cfg.cachestarts_stride_b;
+    p.attn_mask = cfg.attn_mask;
+    p.mask_stride_s = cfg.mask_stride_s;
+    p.mask_stride_h = cfg.mask_stride_h;
+    p.alibi_slopes = static_cast<const float*>(cfg.alibi_slopes);
+    if (!cfg.enable_cache_prefill) { // kernel.cu:2181-2212: the step's own fp16 K/V only, no cache read
+        p.current_key = cfg.current_key;
+        p.current_value = cfg.current_value;
+        p.key_stride_s = cfg.k_stride_s;
+        p.value_stride_s = cfg.v_stride_s;
+    }
     return to_retcode(pmxhip_prefill_attention(&p, stream));
 }
 

@@ -90,6 +90,16 @@ struct PrefillLaunch {
     int64_t cache_stride_h;
     int64_t cache_stride_kv;
     int64_t cachestarts_stride_b;
+    // optional inputs
+    const void* attn_mask;      // half, additive; NULL = none
+    int64_t mask_stride_s;
+    int64_t mask_stride_h;
+    const float* alibi_slopes;  // float32 per query head; NULL = none
+    // K/V from the step's own fp16 rows instead of the cache (kv length = query length; kvstarts = seqstarts)
+    const void* current_key;    // NULL = attend over the cache
+    const void* current_value;
+    int64_t key_stride_s;
+    int64_t value_stride_s;
 };
 
 int launch_kv_quantize(const QuantLaunch& a, hipStream_t stream);

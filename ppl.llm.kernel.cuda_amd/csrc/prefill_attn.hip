@@ -47,9 +47,13 @@ __device__ __forceinline__ int vt_pos16(int o) { return ((o & 4) << 1) | ((o & 8
 
 } // namespace
 
-template <int D, bool PAGED>
+// SRC: where K/V come from: 0 = int8 cache in 128-token pages, 1 = int8 cache in contiguous runs,
+// 2 = the step's fp16 current_key/current_value rows.  EXTRA: additive attn_mask and/or alibi slopes.
+template <int D, int SRC, bool EXTRA>
 __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(const PrefillLaunch a)
 {
+    constexpr bool PAGED = SRC == 0;
+    constexpr bool KV16 = SRC == 2;
     constexpr int KSTEPS = D / 16;          // MFMA k-steps over channels for S
     constexpr int CB = D / 32;              // 32-channel blocks of O^T
     constexpr int GPT = D / 8;              // quantisation groups per token row
@@ -67,8 +71,9 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     // rounding of either factor already costs ~1e-2 absolute where contributions cancel.
     extern __shared__ __attribute__((aligned(16))) char smem_raw[];
     half_t* const sK = (half_t*)smem_raw;
+    // (fp16 K/V need no low parts: the tiles are the values themselves)
     half_t* const sKlo = sK + kBN * K_STRIDE;
-    half_t* const sV = sKlo + kBN * K_STRIDE;
+    half_t* const sV = KV16 ? sKlo : sKlo + kBN * K_STRIDE;
     half_t* const sVlo = sV + D * V_STRIDE;
 
     const int tid = threadIdx.x;
@@ -126,6 +131,14 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         for (int i = 0; i < 16; ++i) o_acc[cb][i] = 0.f;
     float m_run = kNegBig, l_run = 0.f;
     const float sm_scale = a.attn_scale * kLog2e;
+    // element (head, absolute query row, absolute kv column) of the additive mask; kvstarts holds absolute columns
+    const half_t* mask_row = nullptr;
+    float slope = 0.f;
+    if (EXTRA) {
+        if (a.attn_mask)
+            mask_row = (const half_t*)a.attn_mask + (int64_t)h * a.mask_stride_h + (q_row0 + pos_c) * a.mask_stride_s + a.kvstarts[b];
+        if (a.alibi_slopes) slope = a.alibi_slopes[h];
+    }
 
     // ---- global -> register staging of one tile's raw bytes ----
     const int8_t* __restrict__ cache = (const int8_t*)a.cache;
@@ -143,6 +156,7 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     half_t k_sc[K_UNITS];
     u32x2 v_raw[4];
     half_t v_sc[4];
+    u32x4 k16[K_UNITS], v16[4]; // fp16 source: 8 halves per unit
 
     // Addressing: a tile of 64 tokens starts at a multiple of 64, so it lies inside one page.  Its row
     // base is wave-uniform (scalar loads of the page table, read one tile ahead); the per-lane part
@@ -151,6 +165,7 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     auto tile_row = [&](int tile) -> int64_t {
         int t_base = tile * kBN;
         if (t_base > kvlen - 1) t_base = kvlen > 0 ? kvlen - 1 : 0;
+        if (KV16) return q_row0 + t_base; // current_key row of kv token t = query row of the same position
         if (PAGED) return cachestarts[table_base + (t_base >> 7)] + (t_base & (kPage - 1));
         return cachestarts[table_base] + t_base;
     };
@@ -166,7 +181,28 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     const half_t* const scale_k = scale + (head_off >> 3);
     const half_t* const scale_v = scale_k + (a.cache_stride_kv >> 3);
 
+    const uint32_t kstride16 = (uint32_t)a.key_stride_s, vstride16 = (uint32_t)a.value_stride_s;
     auto load_tile = [&](int tile, int64_t row) {
+        if (KV16) {
+            const half_t* bk = (const half_t*)a.current_key + row * a.key_stride_s + (int64_t)kvh * D;
+            const half_t* bv = (const half_t*)a.current_value + row * a.value_stride_s + (int64_t)kvh * D;
+            const int left = kvlen - 1 - tile * kBN;
+#pragma unroll
+            for (int u = 0; u < K_UNITS; ++u) {
+                int t = k_t0 + u * K_TSTEP;
+                t = t < left ? t : (left > 0 ? left : 0);
+                k16[u] = *(const u32x4*)(bk + (uint32_t)t * kstride16 + 8 * k_g);
+            }
+            if (v_on) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    int t = 4 * v_q + r;
+                    t = t < left ? t : (left > 0 ? left : 0);
+                    v16[r] = *(const u32x4*)(bv + (uint32_t)t * vstride16 + 8 * v_g);
+                }
+            }
+            return;
+        }
         const int64_t boff = row * a.cache_stride_s;
         const int8_t* bk = cache_k + boff;
         const int8_t* bv = cache_v + boff;
@@ -206,6 +242,29 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         }
     };
     auto store_tile = [&]() {
+        if (KV16) {
+#pragma unroll
+            for (int u = 0; u < K_UNITS; ++u) *(u32x4*)&sK[(k_t0 + u * K_TSTEP) * K_STRIDE + 8 * k_g] = k16[u];
+            if (v_on) {
+                const int grp = v_q >> 2;
+                const int posv = 16 * grp + vt_pos16(4 * (v_q & 3));
+#pragma unroll
+                for (int e8 = 0; e8 < 8; ++e8) {
+                    const int e = (e8 + v_g) & 7; // rotated channel order, as below
+                    const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u; // half (e & 1) of two words
+                    const int w = e >> 1;
+                    const uint32_t w0 = w == 0 ? v16[0][0] : (w == 1 ? v16[0][1] : (w == 2 ? v16[0][2] : v16[0][3]));
+                    const uint32_t w1 = w == 0 ? v16[1][0] : (w == 1 ? v16[1][1] : (w == 2 ? v16[1][2] : v16[1][3]));
+                    const uint32_t w2 = w == 0 ? v16[2][0] : (w == 1 ? v16[2][1] : (w == 2 ? v16[2][2] : v16[2][3]));
+                    const uint32_t w3 = w == 0 ? v16[3][0] : (w == 1 ? v16[3][1] : (w == 2 ? v16[3][2] : v16[3][3]));
+                    u32x2 out;
+                    out[0] = __builtin_amdgcn_perm(w1, w0, sel);
+                    out[1] = __builtin_amdgcn_perm(w3, w2, sel);
+                    *(u32x2*)&sV[(8 * v_g + e) * V_STRIDE + posv] = out;
+                }
+            }
+            return;
+        }
         // K: 8 halves of one (token, group) -> one 128-bit LDS store
 #pragma unroll
         for (int u = 0; u < K_UNITS; ++u) {
@@ -277,8 +336,10 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
 #pragma unroll
             for (int s = 0; s < KSTEPS; ++s) {
                 const f16x8 kf = *(const f16x8*)&sK[(32 * mb + l32) * K_STRIDE + 16 * s + 8 * hh];
-                const f16x8 kl = *(const f16x8*)&sKlo[(32 * mb + l32) * K_STRIDE + 16 * s + 8 * hh];
-                s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kl, qf[s], s_acc[mb], 0, 0, 0);
+                if (!KV16) {
+                    const f16x8 kl = *(const f16x8*)&sKlo[(32 * mb + l32) * K_STRIDE + 16 * s + 8 * hh];
+                    s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kl, qf[s], s_acc[mb], 0, 0, 0);
+                }
                 s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], s_acc[mb], 0, 0, 0);
             }
         }
@@ -286,18 +347,38 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         // ---- online softmax per column (element i <-> token 32 mb + 8 (i/4) + 4 hh + i%4) ----
         const int t_base = tile * kBN;
         const bool need_mask = t_base + kBN > lim;
-        float mx = kNegBig; // of the raw dot products; the (positive) logit scale is applied to the maximum
+        float mx = kNegBig;
+        if (EXTRA) {
+            // additive terms per element (log2 units): mask value and alibi distance of (query row, token)
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
+            for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                if (need_mask) {
+                for (int i = 0; i < 16; ++i) {
                     const int t = t_base + 32 * mb + 8 * (i >> 2) + 4 * hh + (i & 3);
-                    if (t >= lim) s_acc[mb][i] = -INFINITY;
+                    float v = -INFINITY;
+                    if (t < lim) {
+                        float add = 0.f;
+                        if (mask_row) add = (float)mask_row[t];
+                        if (a.alibi_slopes) add += a.is_causal ? slope * (float)t : -slope * fabsf((float)(pos_c + kvlen - qlen - t));
+                        v = __builtin_fmaf(s_acc[mb][i], sm_scale, add * kLog2e);
+                    }
+                    s_acc[mb][i] = v;
+                    mx = fmaxf(mx, v);
                 }
-                mx = fmaxf(mx, s_acc[mb][i]);
-            }
-        mx *= sm_scale;
+        } else {
+            // maximum of the raw dot products; the (positive) logit scale is applied to it afterwards
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    if (need_mask) {
+                        const int t = t_base + 32 * mb + 8 * (i >> 2) + 4 * hh + (i & 3);
+                        if (t >= lim) s_acc[mb][i] = -INFINITY;
+                    }
+                    mx = fmaxf(mx, s_acc[mb][i]);
+                }
+            mx *= sm_scale;
+        }
         mx = fmaxf(mx, __shfl_xor(mx, 32));
         const float m_new = fmaxf(m_run, mx);
         // the running max moves rarely once a few tiles have been seen: rescale only then (wave-uniform)
@@ -318,8 +399,8 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
             for (int i = 0; i < 16; i += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[mb][i], sm_scale, bias));
-                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s_acc[mb][i + 1], sm_scale, bias));
+                const float p0 = __builtin_amdgcn_exp2f(EXTRA ? s_acc[mb][i] + bias : __builtin_fmaf(s_acc[mb][i], sm_scale, bias));
+                const float p1 = __builtin_amdgcn_exp2f(EXTRA ? s_acc[mb][i + 1] + bias : __builtin_fmaf(s_acc[mb][i + 1], sm_scale, bias));
                 lsum += p0 + p1;
                 const half2_t ph = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(p0, p1));
                 const half2_t pl = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(p0 - (float)ph.x, p1 - (float)ph.y));
@@ -338,8 +419,10 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) {
                     const f16x8 vf = *(const f16x8*)&sV[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
-                    const f16x8 vl = *(const f16x8*)&sVlo[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
-                    o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vl, pf[mb][t], o_acc[cb], 0, 0, 0);
+                    if (!KV16) {
+                        const f16x8 vl = *(const f16x8*)&sVlo[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
+                        o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vl, pf[mb][t], o_acc[cb], 0, 0, 0);
+                    }
                     o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pfl[mb][t], o_acc[cb], 0, 0, 0);
                     o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[mb][t], o_acc[cb], 0, 0, 0);
                 }
@@ -362,24 +445,34 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     }
 }
 
+template <int D, int SRC, bool EXTRA>
+static void launch_prefill_variant(const PrefillLaunch& a, dim3 grid, hipStream_t stream)
+{
+    // int8 source: K hi/lo tiles + transposed V hi/lo tiles (above the 64 KB static limit for D = 128, hence
+    // dynamic); fp16 source: one K tile and one transposed V tile
+    constexpr size_t lds_bytes = (SRC == 2 ? 1 : 2) * (kBN * (D + 8) + D * (kBN + 8)) * sizeof(half_t);
+    static const hipError_t once = hipFuncSetAttribute((const void*)prefill_attention_kernel<D, SRC, EXTRA>,
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    (void)once;
+    hipLaunchKernelGGL((prefill_attention_kernel<D, SRC, EXTRA>), grid, dim3(kPrefillThreads), lds_bytes, stream, a);
+}
+
 template <int D>
 static void launch_prefill_d(const PrefillLaunch& a, hipStream_t stream)
 {
     const int G = (int)(a.num_heads / a.num_kv_heads);
     const int ppw = kCols / G > 0 ? kCols / G : 1;
     const dim3 grid((unsigned)((a.max_seqlen + ppw - 1) / ppw), (unsigned)a.prefill_batches, (unsigned)a.num_kv_heads);
-    // K hi/lo tiles + transposed V hi/lo tiles; above the 64 KB static limit for D = 128, hence dynamic
-    constexpr size_t lds_bytes = (2 * kBN * (D + 8) + 2 * D * (kBN + 8)) * sizeof(half_t);
-    if (a.cache_mode == 1) {
-        static const hipError_t once = hipFuncSetAttribute((const void*)prefill_attention_kernel<D, true>,
-                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        (void)once;
-        hipLaunchKernelGGL((prefill_attention_kernel<D, true>), grid, dim3(kPrefillThreads), lds_bytes, stream, a);
+    const bool extra = a.attn_mask != nullptr || a.alibi_slopes != nullptr;
+    const int src = a.current_key ? 2 : (a.cache_mode == 1 ? 0 : 1);
+    if (extra) {
+        if (src == 0) launch_prefill_variant<D, 0, true>(a, grid, stream);
+        else if (src == 1) launch_prefill_variant<D, 1, true>(a, grid, stream);
+        else launch_prefill_variant<D, 2, true>(a, grid, stream);
     } else {
-        static const hipError_t once = hipFuncSetAttribute((const void*)prefill_attention_kernel<D, false>,
-                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        (void)once;
-        hipLaunchKernelGGL((prefill_attention_kernel<D, false>), grid, dim3(kPrefillThreads), lds_bytes, stream, a);
+        if (src == 0) launch_prefill_variant<D, 0, false>(a, grid, stream);
+        else if (src == 1) launch_prefill_variant<D, 1, false>(a, grid, stream);
+        else launch_prefill_variant<D, 2, false>(a, grid, stream);
     }
 }
 

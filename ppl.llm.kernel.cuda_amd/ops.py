@@ -146,7 +146,11 @@ def splitkv_combine(partial_out, partial_ml, piece_begin, piece_end, output, *, 
 def prefill_attention(query, output, cache, scale, seqstarts, kvstarts, cachestarts, *, attn_scale, is_causal,
                       batch, decoding_batches, max_seqlen, max_kvlen, layer_idx, num_heads, num_kv_heads,
                       head_dim, cache_mode, page_size, cache_stride_s, cache_stride_l, cache_stride_h,
-                      cache_stride_kv, cachestarts_stride_b, stream=None, check=True):
+                      cache_stride_kv, cachestarts_stride_b, attn_mask=None, mask_stride_s=0, mask_stride_h=0,
+                      alibi_slopes=None, current_key=None, current_value=None, stream=None, check=True):
+    """Multi-query-token attention of the prefill sequences.  Optional: additive half `attn_mask` with its
+    strides, float32 `alibi_slopes` [Hq], and `current_key`/`current_value` [rows, KVH, D] to attend over
+    the step's own fp16 rows instead of the cache."""
     p = PrefillParams()
     p.query = _ptr(query)
     p.output = _ptr(output)
@@ -174,6 +178,15 @@ def prefill_attention(query, output, cache, scale, seqstarts, kvstarts, cachesta
     p.cache_stride_h = cache_stride_h
     p.cache_stride_kv = cache_stride_kv
     p.cachestarts_stride_b = cachestarts_stride_b
+    p.attn_mask = _ptr(attn_mask) if attn_mask is not None else None
+    p.mask_stride_s = mask_stride_s
+    p.mask_stride_h = mask_stride_h
+    p.alibi_slopes = _ptr(alibi_slopes) if alibi_slopes is not None else None
+    if current_key is not None:
+        p.current_key = _ptr(current_key)
+        p.current_value = _ptr(current_value)
+        p.key_stride_s = num_kv_heads * head_dim
+        p.value_stride_s = num_kv_heads * head_dim
     rc = _lib.lib().pmxhip_prefill_attention(ctypes.byref(p), _stream(stream))
     if check and rc != RC_SUCCESS:
         raise PmxError(rc, "prefill_attention")

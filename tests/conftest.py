@@ -76,6 +76,23 @@ def oracle_prefill(oracle, bt, q, cache, scale):
                                     bt.attn_scale, bt.layer_idx, bt.page_size, **oracle_layout_kwargs(bt))
 
 
+def oracle_prefill_ex(oracle, bt, q, cache, scale, **extra):
+    return oracle.prefill_attention_ex(q, cache, scale, bt.seqstarts, bt.kvstarts, bt.cachestarts, bt.batch,
+                                       bt.decoding_batches, bt.is_causal, bt.num_heads, bt.num_kv_heads, bt.head_dim,
+                                       bt.attn_scale, bt.layer_idx, bt.page_size, **oracle_layout_kwargs(bt), **extra)
+
+
+def make_prefill_mask(bt, rng, per_head):
+    """Additive fp16 attn_mask in the reference's dynamic-batch layout: (rows, aligned(kv columns, 8)) or
+    (heads, rows, aligned(kv columns, 8)); columns are absolute kv-stream positions (kvstarts)."""
+    rows = int(bt.seqstarts[-1])
+    cols = (int(bt.kvstarts[-1]) + 7) // 8 * 8
+    shape = (bt.num_heads, rows, cols) if per_head else (rows, cols)
+    m = (rng.standard_normal(shape) * 2.0).astype(np.float16)
+    m[rng.random(shape) < 0.1] = np.float16(-60000.0)  # some hard-masked entries
+    return m, cols, (rows * cols if per_head else 0)
+
+
 ATOL = 2e-3  # attention output tolerance against the fp32 dequantised reference:
 RTOL = 1e-2  # |got - ref| <= ATOL + RTOL * |ref|
 

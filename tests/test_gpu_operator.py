@@ -79,9 +79,7 @@ def test_unsupported_configurations_report_not_crash(pkg):
     dev = pkg.harness.DeviceBatch(bt)
     q, k, v = pkg.workloads.step_inputs(bt, rng)
     dev.set_step_inputs(q, k, v)
-    op = dev.make_operator(enable_cache_prefill=False)  # fp16-only prefill is not built: reported, first failure wins
-    assert op.forward_prefill() == pkg.ops.RC_UNSUPPORTED
-    assert op.forward() == pkg.ops.RC_UNSUPPORTED
     op = dev.make_operator(datatype=6)                  # fp32 tensors: prefill rejects (flash_attn2/fmha.cu:75)
     assert op.forward_prefill() == pkg.ops.RC_UNSUPPORTED
+    assert op.forward() == pkg.ops.RC_UNSUPPORTED       # first failure wins
     torch.cuda.synchronize()

@@ -4,8 +4,8 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import (assert_attention_close, host_cache, oracle_append_step, oracle_decode, oracle_fill_history,
-                      oracle_prefill)
+from conftest import (assert_attention_close, host_cache, make_prefill_mask, oracle_append_step, oracle_decode,
+                      oracle_fill_history, oracle_prefill, oracle_prefill_ex)
 
 pytestmark = pytest.mark.gpu
 
@@ -23,7 +23,7 @@ def make_case(pkg, oracle, seed, **kw):
     return bt, dev, q, cache, scale
 
 
-def run_prefill(pkg, dev, is_causal=None):
+def run_prefill(pkg, dev, is_causal=None, **extra):
     bt = dev.bt
     dev.output.fill_(float("nan"))
     pkg.ops.prefill_attention(dev.query, dev.output, dev.cache, dev.scale, dev.seqstarts, dev.kvstarts,
@@ -31,7 +31,7 @@ def run_prefill(pkg, dev, is_causal=None):
                               is_causal=bt.is_causal if is_causal is None else is_causal, batch=bt.batch,
                               decoding_batches=bt.decoding_batches, max_seqlen=bt.max_seqlen, max_kvlen=bt.max_kvlen,
                               layer_idx=bt.layer_idx, num_heads=bt.num_heads, num_kv_heads=bt.num_kv_heads,
-                              head_dim=bt.head_dim, **dev.layout_kwargs())
+                              head_dim=bt.head_dim, **dev.layout_kwargs(), **extra)
     torch.cuda.synchronize()
     return dev.output.float().cpu().numpy()
 
@@ -110,3 +110,53 @@ def test_prefill_full_size_c5(pkg, oracle):
                                                 bt.num_heads, bt.num_kv_heads, bt.head_dim, bt.attn_scale, 0,
                                                 bt.page_size, **kw)
                 assert_attention_close(got[row, h], o, "C5 b=%d row=%d h=%d" % (b, i, h))
+
+
+@pytest.mark.parametrize("is_causal", [True, False])
+@pytest.mark.parametrize("shape,cache_mode,per_head", [((8, 2, 128), 1, True), ((4, 4, 64), 0, False), ((8, 8, 128), 1, False)])
+def test_prefill_mask_and_alibi_match_oracle(pkg, oracle, shape, cache_mode, per_head, is_causal):
+    """The optional inputs of the prefill stage: additive attn_mask (2-d and per-head 3-d) and alibi slopes."""
+    hq, hkv, d = shape
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 700 + hq + d, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                         cache_mode=cache_mode, dec_kv_lens=[33], prefill_q_lens=[70, 7, 1, 129],
+                                         prefill_prior=[130, 0, 50, 127], is_causal=is_causal)
+    rng = np.random.default_rng(11)
+    mask, ms, mh = make_prefill_mask(bt, rng, per_head)
+    slopes = (2.0 ** -np.arange(1, hq + 1)).astype(np.float32)
+    d_mask = torch.from_numpy(mask).cuda()
+    d_slopes = torch.from_numpy(slopes).cuda()
+    n_dec = bt.decoding_batches
+    for use_mask, use_alibi in ((True, False), (False, True), (True, True)):
+        kw_o = dict(attn_mask=mask, mask_stride_s=ms, mask_stride_h=mh) if use_mask else {}
+        kw_d = dict(attn_mask=d_mask, mask_stride_s=ms, mask_stride_h=mh) if use_mask else {}
+        if use_alibi:
+            kw_o["alibi_slopes"] = slopes
+            kw_d["alibi_slopes"] = d_slopes
+        ref = oracle_prefill_ex(oracle, bt, q, cache, scale, **kw_o)
+        got = run_prefill(pkg, dev, **kw_d)
+        assert_attention_close(got[n_dec:], ref[n_dec:], "prefill mask=%s alibi=%s %s" % (use_mask, use_alibi, shape))
+
+
+@pytest.mark.parametrize("shape", [(8, 2, 128), (4, 4, 64), (32, 8, 128)])
+def test_prefill_from_current_key_value(pkg, oracle, shape):
+    """enable_cache_prefill = false: attention over the step's own fp16 K/V rows, no cache read."""
+    hq, hkv, d = shape
+    bt, rng = pkg.workloads.custom_batch(800 + hq, num_heads=hq, num_kv_heads=hkv, head_dim=d, cache_mode=0,
+                                         dec_kv_lens=[5, 9], prefill_q_lens=[70, 7, 1, 129, 300], prefill_prior=[0] * 5,
+                                         outliers=True)
+    dev = pkg.harness.DeviceBatch(bt)
+    q, k, v = pkg.workloads.step_inputs(bt, rng)
+    dev.set_step_inputs(q, k, v)
+    dev.cache.fill_(77)  # must not be read
+    cache, scale = host_cache(bt)
+    ref = oracle_prefill_ex(oracle, bt, q, cache, scale, current_key=k, current_value=v)
+    got = run_prefill(pkg, dev, current_key=dev.new_key, current_value=dev.new_value)
+    n_dec = bt.decoding_batches
+    assert np.isnan(got[:n_dec]).all()
+    assert_attention_close(got[n_dec:], ref[n_dec:], "prefill from current K/V %s" % (shape,))
+    # the operator class with enable_cache_prefill = false takes the same path
+    op = dev.make_operator(enable_cache_prefill=False)
+    dev.output.fill_(float("nan"))
+    assert op.forward_prefill() == 0
+    torch.cuda.synchronize()
+    assert_attention_close(dev.output.float().cpu().numpy()[n_dec:], ref[n_dec:], "operator, enable_cache_prefill=false")

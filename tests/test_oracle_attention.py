@@ -5,8 +5,8 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import (host_cache, oracle_append_step, oracle_decode, oracle_fill_history, oracle_layout_kwargs,
-                      oracle_prefill)
+from conftest import (host_cache, make_prefill_mask, oracle_append_step, oracle_decode, oracle_fill_history,
+                      oracle_layout_kwargs, oracle_prefill, oracle_prefill_ex)
 
 
 def dequantised_sequence(bt, cache, scale, b, plane):
@@ -157,6 +157,67 @@ def test_prefill_matches_torch_sdpa_bottom_right_causal(oracle, pkg, cache_mode)
                                          bt.layer_idx, bt.page_size, **oracle_layout_kwargs(bt))
     np.testing.assert_allclose(got[int(bt.seqstarts[b]), 1], single, rtol=1e-6, atol=1e-7)
     assert dec.shape[0] == bt.decoding_batches
+
+
+def sdpa_reference(bt, b, q, kd, vd, bias):
+    """float64 softmax(attn_scale q k^T + bias) v for prefill sequence b; bias [Hq, qlen, kvlen] with -inf where masked."""
+    rep = bt.num_heads // bt.num_kv_heads
+    rows = slice(int(bt.seqstarts[b]), int(bt.seqstarts[b + 1]))
+    qq = torch.from_numpy(q[rows].astype(np.float64)).permute(1, 0, 2)
+    kk = torch.from_numpy(kd).double().repeat_interleave(rep, 1).permute(1, 0, 2)
+    vv = torch.from_numpy(vd).double().repeat_interleave(rep, 1).permute(1, 0, 2)
+    ref = torch.nn.functional.scaled_dot_product_attention(qq, kk, vv, attn_mask=bias, scale=bt.attn_scale)
+    return rows, ref.permute(1, 0, 2).numpy()
+
+
+@pytest.mark.parametrize("is_causal", [True, False])
+@pytest.mark.parametrize("per_head", [False, True])
+def test_prefill_ex_mask_and_alibi_match_torch_sdpa(oracle, pkg, is_causal, per_head):
+    bt, q, k, v, cache, scale = build_case(oracle, pkg, 37, num_heads=4, num_kv_heads=2, head_dim=64, cache_mode=1,
+                                           dec_kv_lens=[33], prefill_q_lens=[20, 7, 1], prefill_prior=[130, 0, 50],
+                                           is_causal=is_causal)
+    rng = np.random.default_rng(5)
+    mask, ms, mh = make_prefill_mask(bt, rng, per_head)
+    slopes = np.array([0.5, 0.25, 0.125, 0.0625], dtype=np.float32)
+    # without the optional inputs the extended function is the plain one
+    np.testing.assert_array_equal(oracle_prefill_ex(oracle, bt, q, cache, scale), oracle_prefill(oracle, bt, q, cache, scale))
+    got = oracle_prefill_ex(oracle, bt, q, cache, scale, attn_mask=mask, mask_stride_s=ms, mask_stride_h=mh,
+                            alibi_slopes=slopes)
+    for b in range(bt.decoding_batches, bt.batch):
+        qlen, kvlen = int(bt.q_lens[b]), int(bt.kv_lens[b])
+        i = torch.arange(qlen)[:, None]
+        j = torch.arange(kvlen)[None, :]
+        r0, c0 = int(bt.seqstarts[b]), int(bt.kvstarts[b])
+        m = mask[:, r0:r0 + qlen, c0:c0 + kvlen] if per_head else np.broadcast_to(mask[r0:r0 + qlen, c0:c0 + kvlen], (4, qlen, kvlen))
+        bias = torch.from_numpy(m.astype(np.float64)).clone()
+        sl = torch.from_numpy(slopes.astype(np.float64))[:, None, None]
+        if is_causal:
+            bias += sl * j  # mask.h:191-193
+            bias = bias.masked_fill(~(j <= i + (kvlen - qlen)), float("-inf"))
+        else:
+            bias -= sl * (i + kvlen - qlen - j).abs()  # mask.h:194-196
+        rows, ref = sdpa_reference(bt, b, q, dequantised_sequence(bt, cache, scale, b, 0),
+                                   dequantised_sequence(bt, cache, scale, b, 1), bias)
+        np.testing.assert_allclose(got[rows], ref, rtol=1e-5, atol=1e-6)
+
+
+def test_prefill_ex_from_current_key_value_matches_torch_sdpa(oracle, pkg):
+    """enable_cache_prefill = false: the step's fp16 K/V rows only, kv length = query length."""
+    bt, q, k, v, cache, scale = build_case(oracle, pkg, 41, num_heads=4, num_kv_heads=2, head_dim=64, cache_mode=0,
+                                           dec_kv_lens=[9, 12], prefill_q_lens=[20, 7, 1], prefill_prior=[0, 0, 0])
+    got = oracle_prefill_ex(oracle, bt, q, cache, scale, current_key=k, current_value=v)
+    for b in range(bt.decoding_batches, bt.batch):
+        qlen = int(bt.q_lens[b])
+        rows = slice(int(bt.seqstarts[b]), int(bt.seqstarts[b + 1]))
+        i = torch.arange(qlen)[:, None]
+        j = torch.arange(qlen)[None, :]
+        bias = torch.zeros(4, qlen, qlen, dtype=torch.float64).masked_fill(~(j <= i), float("-inf"))
+        _, ref = sdpa_reference(bt, b, q, k[rows].astype(np.float32), v[rows].astype(np.float32), bias)
+        np.testing.assert_allclose(got[rows], ref, rtol=1e-5, atol=1e-6)
+    # with no prior context the cache holds exactly these rows, quantised: the two paths agree to quantisation error
+    via_cache = oracle_prefill(oracle, bt, q, cache, scale)
+    rows = slice(int(bt.seqstarts[bt.decoding_batches]), int(bt.seqstarts[-1]))
+    assert np.abs(via_cache[rows] - got[rows]).max() < 0.1
 
 
 def test_combine_is_split_invariant(oracle, pkg):
