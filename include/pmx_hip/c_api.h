@@ -315,6 +315,37 @@ PMXHIP_API int pmxhip_key_value_cache(
     int64_t cachestarts_stride_b,
     void* cache, void* scale);
 
+/* ---- kv_cache_reorder / kv_cache_invert_reorder ------------------------------
+ * Replace ppl::kernel::llm::cuda::pmx::kv_cache_reorder and kv_cache_invert_reorder
+ * (include/ppl/kernel/llm/cuda/pmx/kv_cache_reorder.h:42-74,
+ * src/ppl/kernel/llm/cuda/pmx/kv_cache_reorder.cu:24-199): whole pages of the int8 cache
+ * and of its scales are gathered into (scattered from) a contiguous outer buffer, for
+ * swapping or migrating pages.  Both tensors are addressed as BYTES.  For slot j of
+ * page_ids, layer l, plane kv in {0,1}, head h, token t < tokens and byte d:
+ *   cache side:  page_ids[j]*head_dim*row + l*l_stride + kv*kv_stride + h*h_stride + t*t_stride + d*d_stride
+ *                (row = head_dim for the cache, head_dim/group_size*2 for the scales; the
+ *                 reference takes head_dim as the tokens of a page, kernel line 44)
+ *   outer side:  (p_stride_cache + p_stride_scale)*tp_size*j + tp_rank*p_stride_cache + the five strides,
+ *                scales a further (tp_size - tp_rank)*p_stride_cache + tp_rank*p_stride_scale on
+ *   with p_stride_* taken from src_stride in both directions, as the reference does.
+ * Field order of the stride struct is the reference's `Stride` (kv_cache_reorder.h:25-40). */
+typedef struct pmxhip_reorder_stride {
+    int32_t p_stride_cache, l_stride_cache, kv_stride_cache, h_stride_cache, t_stride_cache, d_stride_cache;
+    int32_t p_stride_scale, l_stride_scale, kv_stride_scale, h_stride_scale, t_stride_scale, d_stride_scale;
+} pmxhip_reorder_stride;
+
+PMXHIP_API int pmxhip_kv_cache_reorder(
+    pmxhip_stream_t stream, const void* kv_cache, const void* kv_scale, const int64_t* page_ids,
+    const pmxhip_reorder_stride* src_stride, const pmxhip_reorder_stride* dst_stride,
+    int64_t page_nums, int64_t layers, int64_t kv_heads, int64_t tokens, int64_t head_dim, int64_t group_size,
+    int64_t tp_rank, int64_t tp_size, void* outer_mem);
+
+PMXHIP_API int pmxhip_kv_cache_invert_reorder(
+    pmxhip_stream_t stream, const void* outer_mem, const int64_t* page_ids,
+    const pmxhip_reorder_stride* src_stride, const pmxhip_reorder_stride* dst_stride,
+    int64_t page_nums, int64_t layers, int64_t kv_heads, int64_t tokens, int64_t head_dim, int64_t group_size,
+    int64_t tp_rank, int64_t tp_size, void* kv_cache, void* kv_scale);
+
 /* Library identity / build check (host only). */
 PMXHIP_API const char* pmxhip_version(void);
 PMXHIP_API const char* pmxhip_last_error(void); /* thread-local text of the last failure */

@@ -62,6 +62,8 @@ def lib():
         _lib.pmx_oracle_splitkv_combine.restype = ctypes.c_int
         _lib.pmx_oracle_splitkv_combine.argtypes = [_vp] * 3 + [_i64, _i64, _vp]
         _lib.pmx_oracle_num_threads.restype = ctypes.c_int
+        _lib.pmx_oracle_kv_cache_reorder.restype = ctypes.c_int
+        _lib.pmx_oracle_kv_cache_reorder.argtypes = [_i32] + [_vp] * 6 + [_i64] * 8
     return _lib
 
 
@@ -252,3 +254,16 @@ def splitkv_combine(partial_out, partial_max, partial_sum):
 
 def num_threads():
     return int(lib().pmx_oracle_num_threads())
+
+
+def kv_cache_reorder(invert, kv_cache, kv_scale, outer_mem, page_ids, src_stride, dst_stride, layers, kv_heads, tokens,
+                     head_dim, group_size, tp_rank, tp_size):
+    """In place on the uint8 numpy arrays: gathers pages into outer_mem (invert=False) or scatters them back
+    into kv_cache / kv_scale (invert=True).  Strides: 12 ints, {p, l, kv, h, t, d} for cache then scale."""
+    assert kv_cache.dtype == np.uint8 and kv_scale.dtype == np.uint8 and outer_mem.dtype == np.uint8
+    page_ids = _c(page_ids, np.int64)
+    ss = _c(src_stride, np.int32)
+    ds = _c(dst_stride, np.int32)
+    lib().pmx_oracle_kv_cache_reorder(1 if invert else 0, _p(kv_cache), _p(kv_scale), _p(outer_mem), _p(page_ids),
+                                      _p(ss), _p(ds), len(page_ids), layers, kv_heads, tokens, head_dim, group_size,
+                                      tp_rank, tp_size)

@@ -23,6 +23,9 @@
  *                                  optional inputs; torch SDPA with an additive float mask
  *                                  (bias + alibi + causal) on the dequantised cache and on
  *                                  fp16 K/V.
+ *   pmx_oracle_kv_cache_reorder    pinned: numpy gather + transpose of the same pages for a
+ *                                  concrete pair of layouts; reorder followed by its inverse
+ *                                  restores the pages and touches nothing else.
  *   pmx_oracle_splitkv_combine     pinned: any split of the kv range equals the
  *                                  single pass (log-sum-exp associativity).
  *   The reference itself cannot be compiled here (CUDA, inline PTX, CUTLASS, and
@@ -527,4 +530,45 @@ int pmx_oracle_num_threads(void)
 #else
     return 1;
 #endif
+}
+
+/* ------------------------------------------------------------------------- */
+/* kv_cache_reorder / kv_cache_invert_reorder (pmx/kv_cache_reorder.cu:24-65,   */
+/* 103-144): one byte per (slot, layer, plane, head, token, d), index formulas */
+/* as in the reference, including head_dim as the tokens of a page (line 44).  */
+/* stride arrays: {p, l, kv, h, t, d} for the cache, then the same for scales. */
+/* ------------------------------------------------------------------------- */
+int pmx_oracle_kv_cache_reorder(
+    int32_t invert,
+    uint8_t* kv_cache, uint8_t* kv_scale, uint8_t* outer_mem, const int64_t* page_ids,
+    const int32_t* src_stride, const int32_t* dst_stride,
+    int64_t page_nums, int64_t layers, int64_t kv_heads, int64_t tokens, int64_t head_dim, int64_t group_size,
+    int64_t tp_rank, int64_t tp_size)
+{
+    const int64_t pcb = src_stride[0], psb = src_stride[6];
+    const int64_t scale_row = head_dim / group_size * 2;
+    const int32_t* cs = invert ? dst_stride : src_stride; /* cache-side strides */
+    const int32_t* os = invert ? src_stride : dst_stride; /* outer-side strides */
+    for (int64_t j = 0; j < page_nums; ++j) {
+        const int64_t page = page_ids[j];
+        uint8_t* outer_cache = outer_mem + (pcb + psb) * tp_size * j + tp_rank * pcb;
+        uint8_t* outer_scale = outer_cache + (tp_size - tp_rank) * pcb + tp_rank * psb;
+        for (int64_t l = 0; l < layers; ++l)
+            for (int64_t kv = 0; kv < 2; ++kv)
+                for (int64_t h = 0; h < kv_heads; ++h)
+                    for (int64_t t = 0; t < tokens; ++t)
+                        for (int64_t d = 0; d < head_dim; ++d) {
+                            const int64_t ci = page * head_dim * head_dim + l * cs[1] + kv * cs[2] + h * cs[3] + t * cs[4] + d * cs[5];
+                            const int64_t oi = l * os[1] + kv * os[2] + h * os[3] + t * os[4] + d * os[5];
+                            if (invert) kv_cache[ci] = outer_cache[oi];
+                            else outer_cache[oi] = kv_cache[ci];
+                            if (d < scale_row) {
+                                const int64_t si = page * head_dim * scale_row + l * cs[7] + kv * cs[8] + h * cs[9] + t * cs[10] + d * cs[11];
+                                const int64_t so = l * os[7] + kv * os[8] + h * os[9] + t * os[10] + d * os[11];
+                                if (invert) kv_scale[si] = outer_scale[so];
+                                else outer_scale[so] = kv_scale[si];
+                            }
+                        }
+    }
+    return 0;
 }

@@ -30,6 +30,7 @@ EXPORTED_SYMBOLS = (
     "pmxhip_mhca_get_derived", "pmxhip_mhca_set_workspace",
     "pmxhip_mhca_forward_kvstore", "pmxhip_mhca_forward_decode", "pmxhip_mhca_forward_prefill",
     "pmxhip_mhca_forward",
+    "pmxhip_kv_cache_reorder", "pmxhip_kv_cache_invert_reorder",
 )
 
 
@@ -85,6 +86,19 @@ class PrefillParams(ctypes.Structure):
         ("attn_mask", c_vp), ("mask_stride_s", c_i64), ("mask_stride_h", c_i64), ("alibi_slopes", c_vp),
         ("current_key", c_vp), ("current_value", c_vp), ("key_stride_s", c_i64), ("value_stride_s", c_i64),
     ]
+
+
+class ReorderStride(ctypes.Structure):
+    """pmxhip_reorder_stride: byte strides {page, layer, plane, head, token, byte} of the cache, then of the scales."""
+    _fields_ = [(n + k, c_i32) for k in ("_cache", "_scale")
+                for n in ("p_stride", "l_stride", "kv_stride", "h_stride", "t_stride", "d_stride")]
+
+    @staticmethod
+    def of(values):
+        s = ReorderStride()
+        for (name, _), v in zip(ReorderStride._fields_, values):
+            setattr(s, name, int(v))
+        return s
 
 
 class TensorShape(ctypes.Structure):
@@ -157,6 +171,10 @@ def lib():
     L.pmxhip_last_error.restype = ctypes.c_char_p
     L.pmxhip_kv_cache_quantize.restype = ctypes.c_int
     L.pmxhip_kv_cache_quantize.argtypes = [ctypes.POINTER(KvstoreParams), c_vp]
+    L.pmxhip_kv_cache_reorder.restype = ctypes.c_int
+    L.pmxhip_kv_cache_reorder.argtypes = [c_vp] * 4 + [ctypes.POINTER(ReorderStride)] * 2 + [c_i64] * 8 + [c_vp]
+    L.pmxhip_kv_cache_invert_reorder.restype = ctypes.c_int
+    L.pmxhip_kv_cache_invert_reorder.argtypes = [c_vp] * 3 + [ctypes.POINTER(ReorderStride)] * 2 + [c_i64] * 8 + [c_vp] * 2
     L.pmxhip_key_value_cache.restype = ctypes.c_int
     L.pmxhip_key_value_cache.argtypes = [c_vp] * 6 + [c_i64] * 6 + [c_i32] + [c_i64] * 6 + [c_vp] * 2
     L.pmxhip_decode_plan_make.restype = ctypes.c_int

@@ -358,4 +358,73 @@ int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t str
     return launch_status("prefill_attention");
 }
 
+static int reorder_common(const char* what, bool invert, pmxhip_stream_t stream, const void* cache, const void* scale,
+                          const void* outer, const int64_t* page_ids, const pmxhip_reorder_stride* src,
+                          const pmxhip_reorder_stride* dst, int64_t page_nums, int64_t layers, int64_t kv_heads,
+                          int64_t tokens, int64_t head_dim, int64_t group_size, int64_t tp_rank, int64_t tp_size)
+{
+    if (!src || !dst) return fail(PMXHIP_INVALID_VALUE, "%s: null stride", what);
+    if (page_nums < 0 || layers < 0 || kv_heads < 0 || tokens < 0)
+        return fail(PMXHIP_INVALID_VALUE, "%s: negative extent", what);
+    if (page_nums == 0 || layers == 0 || kv_heads == 0 || tokens == 0) return PMXHIP_SUCCESS;
+    if (!cache || !scale || !outer || !page_ids) return fail(PMXHIP_INVALID_VALUE, "%s: null device pointer", what);
+    if (head_dim <= 0 || group_size <= 0 || head_dim % group_size != 0)
+        return fail(PMXHIP_INVALID_VALUE, "%s: head_dim must be a positive multiple of group_size", what);
+    if (tp_size <= 0 || tp_rank < 0 || tp_rank >= tp_size) return fail(PMXHIP_INVALID_VALUE, "%s: tp_rank outside [0, tp_size)", what);
+    const int64_t pcb = src->p_stride_cache, psb = src->p_stride_scale; // both directions read them from src_stride
+    const int64_t slot = (pcb + psb) * tp_size;
+    const int64_t scale_row = head_dim / group_size * 2;
+    // cache side / outer side strides of each direction
+    const pmxhip_reorder_stride* cs = invert ? dst : src; // cache-side strides
+    const pmxhip_reorder_stride* os = invert ? src : dst; // outer-side strides
+    for (int part = 0; part < 2; ++part) {
+        pmxhip::PageCopyLaunch a{};
+        a.page_ids = page_ids;
+        a.pages = page_nums;
+        a.layers = layers;
+        a.kv_heads = kv_heads;
+        a.tokens = tokens;
+        a.row_bytes = part == 0 ? head_dim : scale_row;
+        const int64_t c_stride[5] = {part == 0 ? cs->l_stride_cache : cs->l_stride_scale, part == 0 ? cs->kv_stride_cache : cs->kv_stride_scale,
+                                     part == 0 ? cs->h_stride_cache : cs->h_stride_scale, part == 0 ? cs->t_stride_cache : cs->t_stride_scale,
+                                     part == 0 ? cs->d_stride_cache : cs->d_stride_scale};
+        const int64_t o_stride[5] = {part == 0 ? os->l_stride_cache : os->l_stride_scale, part == 0 ? os->kv_stride_cache : os->kv_stride_scale,
+                                     part == 0 ? os->h_stride_cache : os->h_stride_scale, part == 0 ? os->t_stride_cache : os->t_stride_scale,
+                                     part == 0 ? os->d_stride_cache : os->d_stride_scale};
+        const char* c_base = static_cast<const char*>(part == 0 ? cache : scale);
+        const char* o_base = static_cast<const char*>(outer) + tp_rank * pcb + (part == 0 ? 0 : (tp_size - tp_rank) * pcb + tp_rank * psb);
+        const int64_t c_page = head_dim * a.row_bytes; // kv_cache_reorder.cu:44, 57
+        for (int i = 0; i < 5; ++i) {
+            a.src_stride[i] = invert ? o_stride[i] : c_stride[i];
+            a.dst_stride[i] = invert ? c_stride[i] : o_stride[i];
+        }
+        a.src = invert ? o_base : c_base;
+        a.dst = const_cast<char*>(invert ? c_base : o_base);
+        a.src_slot_stride = invert ? slot : 0;
+        a.dst_slot_stride = invert ? 0 : slot;
+        a.src_page_stride = invert ? 0 : c_page;
+        a.dst_page_stride = invert ? c_page : 0;
+        pmxhip::launch_page_copy(a, stream);
+    }
+    return launch_status(what);
+}
+
+int pmxhip_kv_cache_reorder(pmxhip_stream_t stream, const void* kv_cache, const void* kv_scale, const int64_t* page_ids,
+                            const pmxhip_reorder_stride* src_stride, const pmxhip_reorder_stride* dst_stride, int64_t page_nums,
+                            int64_t layers, int64_t kv_heads, int64_t tokens, int64_t head_dim, int64_t group_size,
+                            int64_t tp_rank, int64_t tp_size, void* outer_mem)
+{
+    return reorder_common("kv_cache_reorder", false, stream, kv_cache, kv_scale, outer_mem, page_ids, src_stride, dst_stride,
+                          page_nums, layers, kv_heads, tokens, head_dim, group_size, tp_rank, tp_size);
+}
+
+int pmxhip_kv_cache_invert_reorder(pmxhip_stream_t stream, const void* outer_mem, const int64_t* page_ids,
+                                   const pmxhip_reorder_stride* src_stride, const pmxhip_reorder_stride* dst_stride,
+                                   int64_t page_nums, int64_t layers, int64_t kv_heads, int64_t tokens, int64_t head_dim,
+                                   int64_t group_size, int64_t tp_rank, int64_t tp_size, void* kv_cache, void* kv_scale)
+{
+    return reorder_common("kv_cache_invert_reorder", true, stream, kv_cache, kv_scale, outer_mem, page_ids, src_stride, dst_stride,
+                          page_nums, layers, kv_heads, tokens, head_dim, group_size, tp_rank, tp_size);
+}
+
 } // extern "C"

@@ -14,6 +14,7 @@
 
 #include "pmx_hip/c_api.h"
 #include "pmx_hip/key_value_cache.h"
+#include "pmx_hip/kv_cache_reorder.h"
 
 namespace ppl { namespace kernel { namespace llm { namespace cuda { namespace pmx {
 
@@ -370,6 +371,39 @@ ppl::common::RetCode dynamic_batching_key_value_cache(
         static_cast<const int64_t*>(cachestarts), static_cast<const int64_t*>(start_pos), batch, max_seqlen, num_layer,
         layer_idx, num_kv_heads, head_dim, cache_mode, page_size, cache_stride_s, cache_stride_l, cache_stride_h,
         cache_stride_kv, cachestarts_stride_b, cache, scale));
+}
+
+static pmxhip_reorder_stride to_c_stride(const Stride& s)
+{
+    pmxhip_reorder_stride r;
+    r.p_stride_cache = s.p_stride_cache; r.l_stride_cache = s.l_stride_cache; r.kv_stride_cache = s.kv_stride_cache;
+    r.h_stride_cache = s.h_stride_cache; r.t_stride_cache = s.t_stride_cache; r.d_stride_cache = s.d_stride_cache;
+    r.p_stride_scale = s.p_stride_scale; r.l_stride_scale = s.l_stride_scale; r.kv_stride_scale = s.kv_stride_scale;
+    r.h_stride_scale = s.h_stride_scale; r.t_stride_scale = s.t_stride_scale; r.d_stride_scale = s.d_stride_scale;
+    return r;
+}
+
+ppl::common::RetCode kv_cache_reorder(
+    hipStream_t stream, const void* kv_cache, const void* kv_scale, const void* page_ids,
+    const Stride& src_stride, const Stride& dst_stride,
+    int64_t page_nums, int64_t layers, int64_t kv_heads, int64_t tokens, int64_t head_dim, int64_t group_size,
+    int64_t tp_rank, int64_t tp_size, void* outer_mem)
+{
+    const pmxhip_reorder_stride s = to_c_stride(src_stride), d = to_c_stride(dst_stride);
+    return to_retcode(pmxhip_kv_cache_reorder(stream, kv_cache, kv_scale, static_cast<const int64_t*>(page_ids), &s, &d, page_nums,
+                                              layers, kv_heads, tokens, head_dim, group_size, tp_rank, tp_size, outer_mem));
+}
+
+ppl::common::RetCode kv_cache_invert_reorder(
+    hipStream_t stream, const void* outer_mem, const void* page_ids,
+    const Stride& src_stride, const Stride& dst_stride,
+    int64_t page_nums, int64_t layers, int64_t kv_heads, int64_t tokens, int64_t head_dim, int64_t group_size,
+    int64_t tp_rank, int64_t tp_size, void* kv_cache, void* kv_scale)
+{
+    const pmxhip_reorder_stride s = to_c_stride(src_stride), d = to_c_stride(dst_stride);
+    return to_retcode(pmxhip_kv_cache_invert_reorder(stream, outer_mem, static_cast<const int64_t*>(page_ids), &s, &d, page_nums,
+                                                     layers, kv_heads, tokens, head_dim, group_size, tp_rank, tp_size, kv_cache,
+                                                     kv_scale));
 }
 
 }}}}} // namespace ppl::kernel::llm::cuda::pmx

@@ -102,7 +102,19 @@ struct PrefillLaunch {
     int64_t value_stride_s;
 };
 
+// One strided copy of whole pages (cache bytes or scale bytes) between the cache and the outer buffer.
+struct PageCopyLaunch {
+    const char* src;
+    char* dst;
+    const int64_t* page_ids;
+    int64_t pages, layers, kv_heads, tokens, row_bytes;
+    int64_t src_slot_stride, dst_slot_stride; // per slot (index into page_ids)
+    int64_t src_page_stride, dst_page_stride; // per page id
+    int64_t src_stride[5], dst_stride[5];     // layer, K/V plane, kv head, token, byte
+};
+
 int launch_kv_quantize(const QuantLaunch& a, hipStream_t stream);
+void launch_page_copy(const PageCopyLaunch& a, hipStream_t stream);
 int launch_decode(const DecodeLaunch& a, int stage, hipStream_t stream); // stage: 0 both, 1 ranges, 2 combine
 int decode_wg_tokens(int head_dim, int kv_heads_per_group);
 bool decode_quad_applicable(const DecodeLaunch& a); // head_dim 128, <= 4 query heads per kv head, kv heads in eights

@@ -193,6 +193,31 @@ def prefill_attention(query, output, cache, scale, seqstarts, kvstarts, cachesta
     return rc
 
 
+def kv_cache_reorder(kv_cache, kv_scale, page_ids, src_stride, dst_stride, *, layers, kv_heads, tokens, head_dim,
+                     group_size, tp_rank, tp_size, outer_mem, stream=None, check=True):
+    """Gathers the pages `page_ids` of the int8 cache and of its scales into `outer_mem`.
+    Strides: 12 byte strides, {page, layer, plane, head, token, byte} of the cache then of the scales."""
+    s, d = _lib.ReorderStride.of(src_stride), _lib.ReorderStride.of(dst_stride)
+    rc = _lib.lib().pmxhip_kv_cache_reorder(_stream(stream), _ptr(kv_cache), _ptr(kv_scale), _ptr(page_ids),
+                                            ctypes.byref(s), ctypes.byref(d), int(page_ids.numel()), layers, kv_heads,
+                                            tokens, head_dim, group_size, tp_rank, tp_size, _ptr(outer_mem))
+    if check and rc != RC_SUCCESS:
+        raise PmxError(rc, "kv_cache_reorder")
+    return rc
+
+
+def kv_cache_invert_reorder(outer_mem, page_ids, src_stride, dst_stride, *, layers, kv_heads, tokens, head_dim,
+                            group_size, tp_rank, tp_size, kv_cache, kv_scale, stream=None, check=True):
+    """Scatters pages from `outer_mem` back into the cache and its scales (the inverse of kv_cache_reorder)."""
+    s, d = _lib.ReorderStride.of(src_stride), _lib.ReorderStride.of(dst_stride)
+    rc = _lib.lib().pmxhip_kv_cache_invert_reorder(_stream(stream), _ptr(outer_mem), _ptr(page_ids), ctypes.byref(s),
+                                                   ctypes.byref(d), int(page_ids.numel()), layers, kv_heads, tokens,
+                                                   head_dim, group_size, tp_rank, tp_size, _ptr(kv_cache), _ptr(kv_scale))
+    if check and rc != RC_SUCCESS:
+        raise PmxError(rc, "kv_cache_invert_reorder")
+    return rc
+
+
 class DynamicBatchingMultiHeadCacheAttention:
     """The operator class (C++ `dynamic_batching_multi_head_cache_attention`) behind its C handle."""
 
