@@ -346,6 +346,49 @@ PMXHIP_API int pmxhip_kv_cache_invert_reorder(
     int64_t page_nums, int64_t layers, int64_t kv_heads, int64_t tokens, int64_t head_dim, int64_t group_size,
     int64_t tp_rank, int64_t tp_size, void* kv_cache, void* kv_scale);
 
+/* ---- rotary position embedding, alone and fused with the append --------------
+ * pmxhip_rotary_position_embedding replaces dynamic_batching_rotary_position_embedding
+ * (include/ppl/kernel/llm/cuda/pmx/rotary_position_embedding.h:54-76,
+ * src/ppl/kernel/llm/cuda/pmx/rotary_position_embedding.cu:268-446): channel pairs (2i, 2i+1),
+ * i < rotary_dim/2, of every query head and of the first num_key_heads key heads are rotated by
+ * angle = pos / theta^(i / (rotary_dim/2)), pos = start_pos[b] + position in the sequence;
+ * other channels are copied.  scaling_type: 0 none, 1 linear (pos / scaling_factor), 2 dynamic
+ * (theta rescaled when start_pos + seqlen > max_position_embeddings, kernel lines 68-91); the
+ * reference's header gives all three names the value 0, so only "none" is reachable there.
+ * Strides are in halves per row.  rotated_query may alias query, rotated_key may alias key.
+ *
+ * pmxhip_rope_kv_cache_quantize is the same rotation followed, in the same kernel, by the
+ * quantise/append of the rotated key and of the value rows (pmxhip_kv_cache_quantize): the
+ * rotated key never makes a round trip through memory and one launch is saved.  Of `store`,
+ * current_key is ignored (the key comes from `rope`); rope->rotated_key may be NULL. */
+typedef struct pmxhip_rope_params {
+    const void* query;         /* half (S, Hq, D) */
+    const void* key;           /* half (S, KVH, D) */
+    const int64_t* start_pos;  /* (B) */
+    const int64_t* seqstarts;  /* (B + 1) */
+    float theta;
+    int32_t bypass_key;        /* 1: key rows are copied, not rotated */
+    int64_t rotary_dim;
+    int64_t batch;
+    int64_t num_heads;
+    int64_t num_key_heads;
+    int64_t head_dim;
+    int64_t max_seqlen;
+    int64_t max_position_embeddings;
+    int32_t scaling_type;
+    float scaling_factor;
+    int64_t query_stride_s;
+    int64_t key_stride_s;
+    int64_t rotated_query_stride_s;
+    int64_t rotated_key_stride_s;
+    void* rotated_query;
+    void* rotated_key;
+} pmxhip_rope_params;
+
+PMXHIP_API int pmxhip_rotary_position_embedding(const pmxhip_rope_params* p, pmxhip_stream_t stream);
+PMXHIP_API int pmxhip_rope_kv_cache_quantize(const pmxhip_rope_params* rope, const pmxhip_kvstore_params* store,
+                                             pmxhip_stream_t stream);
+
 /* Library identity / build check (host only). */
 PMXHIP_API const char* pmxhip_version(void);
 PMXHIP_API const char* pmxhip_last_error(void); /* thread-local text of the last failure */

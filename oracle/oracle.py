@@ -62,6 +62,9 @@ def lib():
         _lib.pmx_oracle_splitkv_combine.restype = ctypes.c_int
         _lib.pmx_oracle_splitkv_combine.argtypes = [_vp] * 3 + [_i64, _i64, _vp]
         _lib.pmx_oracle_num_threads.restype = ctypes.c_int
+        _lib.pmx_oracle_rotary_position_embedding.restype = ctypes.c_int
+        _lib.pmx_oracle_rotary_position_embedding.argtypes = (
+            [_vp] * 4 + [_f32, _i32] + [_i64] * 6 + [_i32, _f32] + [_i64] * 4 + [_vp] * 2)
         _lib.pmx_oracle_kv_cache_reorder.restype = ctypes.c_int
         _lib.pmx_oracle_kv_cache_reorder.argtypes = [_i32] + [_vp] * 6 + [_i64] * 8
     return _lib
@@ -267,3 +270,23 @@ def kv_cache_reorder(invert, kv_cache, kv_scale, outer_mem, page_ids, src_stride
     lib().pmx_oracle_kv_cache_reorder(1 if invert else 0, _p(kv_cache), _p(kv_scale), _p(outer_mem), _p(page_ids),
                                       _p(ss), _p(ds), len(page_ids), layers, kv_heads, tokens, head_dim, group_size,
                                       tp_rank, tp_size)
+
+
+def rotary_position_embedding(query, key, start_pos, seqstarts, theta, rotary_dim, bypass_key=False,
+                              max_position_embeddings=2048, scaling_type=0, scaling_factor=1.0):
+    """query [S, Hq, D], key [S, KVH, D] float16 -> (rotated_query, rotated_key) float16."""
+    query = _c(query, np.float16)
+    key = _c(key, np.float16)
+    start_pos = _c(start_pos, np.int64)
+    seqstarts = _c(seqstarts, np.int64)
+    rq = np.zeros_like(query)
+    rk = np.zeros_like(key)
+    hq, d = query.shape[1], query.shape[2]
+    hk = key.shape[1]
+    rc = lib().pmx_oracle_rotary_position_embedding(
+        _p(query), _p(key), _p(start_pos), _p(seqstarts), theta, 1 if bypass_key else 0, rotary_dim,
+        len(start_pos), hq, hk, d, max_position_embeddings, scaling_type, scaling_factor,
+        hq * d, hk * d, hq * d, hk * d, _p(rq), _p(rk))
+    if rc != 0:
+        raise ValueError("oracle rope rejected the arguments (rc=%d)" % rc)
+    return rq, rk

@@ -26,6 +26,11 @@
  *   pmx_oracle_kv_cache_reorder    pinned: numpy gather + transpose of the same pages for a
  *                                  concrete pair of layouts; reorder followed by its inverse
  *                                  restores the pages and touches nothing else.
+ *   pmx_oracle_rotary_position_embedding pinned: numpy complex multiplication by exp(i angle) in
+ *                                  binary64 (half-ulp bound), position 0 = identity, pair norms
+ *                                  preserved, linear scaling = rotation at pos / factor.  The
+ *                                  reference's own bits (approximate __powf / __sincosf) are
+ *                                  parity unpinned.
  *   pmx_oracle_splitkv_combine     pinned: any split of the kv range equals the
  *                                  single pass (log-sum-exp associativity).
  *   The reference itself cannot be compiled here (CUDA, inline PTX, CUTLASS, and
@@ -569,6 +574,72 @@ int pmx_oracle_kv_cache_reorder(
                                 else outer_scale[so] = kv_scale[si];
                             }
                         }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Rotary position embedding for dynamic batches                              */
+/* (pmx/rotary_position_embedding.cu:35-91 coefficients, 268-343 kernel).      */
+/* Pairs (2i, 2i+1), i < rotary_dim/2: (x, y) -> (x c - y s, y c + x s) in      */
+/* binary32, rounded to half; other channels copied.  The angle follows the    */
+/* reference formula 1.0f / powf(theta, i / (rotary_dim/2)) * pos with pow, cos */
+/* and sin evaluated in binary64 and rounded once (the reference uses the      */
+/* approximate __powf / __sincosf, whose bits are unpinned).                    */
+/* scaling_type: 0 none, 1 linear, 2 dynamic.                                   */
+/* ------------------------------------------------------------------------- */
+int pmx_oracle_rotary_position_embedding(
+    const uint16_t* query, const uint16_t* key,
+    const int64_t* start_pos, const int64_t* seqstarts,
+    float theta, int32_t bypass_key, int64_t rotary_dim, int64_t batch,
+    int64_t num_heads, int64_t num_key_heads, int64_t head_dim,
+    int64_t max_position_embeddings, int32_t scaling_type, float scaling_factor,
+    int64_t query_stride_s, int64_t key_stride_s, int64_t rotated_query_stride_s, int64_t rotated_key_stride_s,
+    uint16_t* rotated_query, uint16_t* rotated_key)
+{
+    if (head_dim % 2 != 0 || rotary_dim % 2 != 0 || rotary_dim > head_dim || scaling_type < 0 || scaling_type > 2)
+        return 4;
+    const int64_t rd2 = rotary_dim / 2;
+    for (int64_t b = 0; b < batch; ++b) {
+        const int64_t seqlen = seqstarts[b + 1] - seqstarts[b];
+        float th = theta;
+        if (scaling_type == 2) {
+            const int64_t pos_end = start_pos[b] + seqlen;
+            if (pos_end > max_position_embeddings) {
+                const float base = ((scaling_factor * (float)pos_end) / (float)max_position_embeddings) - (scaling_factor - 1.f);
+                const float expn = (float)rd2 / (float)(rd2 - 1);
+                th = theta * (float)pow((double)base, (double)expn);
+            }
+        }
+        for (int64_t sidx = 0; sidx < seqlen; ++sidx) {
+            const int64_t tok = seqstarts[b] + sidx;
+            const int64_t pos = start_pos[b] + sidx;
+            for (int64_t h = 0; h < num_heads; ++h)
+                for (int64_t i = 0; i < head_dim / 2; ++i) {
+                    float c = 1.f, sn = 0.f;
+                    if (i < rd2) {
+                        const float inv = 1.0f / (float)pow((double)th, (double)((float)i / (float)rd2));
+                        const float p = scaling_type == 1 ? (float)pos / scaling_factor : (float)pos;
+                        const float angle = inv * p;
+                        c = (float)cos((double)angle);
+                        sn = (float)sin((double)angle);
+                    }
+                    for (int which = 0; which < 2; ++which) {
+                        if (which == 1 && h >= num_key_heads) continue;
+                        const uint16_t* src = which == 0 ? query + tok * query_stride_s : key + tok * key_stride_s;
+                        uint16_t* dst = which == 0 ? rotated_query + tok * rotated_query_stride_s : rotated_key + tok * rotated_key_stride_s;
+                        const int64_t e = h * head_dim + 2 * i;
+                        if (i >= rd2 || (which == 1 && bypass_key)) {
+                            dst[e] = src[e];
+                            dst[e + 1] = src[e + 1];
+                        } else {
+                            const float x = pmx_oracle_half_to_float(src[e]), y = pmx_oracle_half_to_float(src[e + 1]);
+                            dst[e] = pmx_oracle_float_to_half(x * c - y * sn);
+                            dst[e + 1] = pmx_oracle_float_to_half(y * c + x * sn);
+                        }
+                    }
+                }
+        }
     }
     return 0;
 }

@@ -31,6 +31,7 @@ EXPORTED_SYMBOLS = (
     "pmxhip_mhca_forward_kvstore", "pmxhip_mhca_forward_decode", "pmxhip_mhca_forward_prefill",
     "pmxhip_mhca_forward",
     "pmxhip_kv_cache_reorder", "pmxhip_kv_cache_invert_reorder",
+    "pmxhip_rotary_position_embedding", "pmxhip_rope_kv_cache_quantize",
 )
 
 
@@ -85,6 +86,17 @@ class PrefillParams(ctypes.Structure):
         ("cache_stride_kv", c_i64), ("cachestarts_stride_b", c_i64),
         ("attn_mask", c_vp), ("mask_stride_s", c_i64), ("mask_stride_h", c_i64), ("alibi_slopes", c_vp),
         ("current_key", c_vp), ("current_value", c_vp), ("key_stride_s", c_i64), ("value_stride_s", c_i64),
+    ]
+
+
+class RopeParams(ctypes.Structure):
+    _fields_ = [
+        ("query", c_vp), ("key", c_vp), ("start_pos", c_vp), ("seqstarts", c_vp),
+        ("theta", c_f32), ("bypass_key", c_i32), ("rotary_dim", c_i64), ("batch", c_i64),
+        ("num_heads", c_i64), ("num_key_heads", c_i64), ("head_dim", c_i64), ("max_seqlen", c_i64),
+        ("max_position_embeddings", c_i64), ("scaling_type", c_i32), ("scaling_factor", c_f32),
+        ("query_stride_s", c_i64), ("key_stride_s", c_i64), ("rotated_query_stride_s", c_i64),
+        ("rotated_key_stride_s", c_i64), ("rotated_query", c_vp), ("rotated_key", c_vp),
     ]
 
 
@@ -171,6 +183,10 @@ def lib():
     L.pmxhip_last_error.restype = ctypes.c_char_p
     L.pmxhip_kv_cache_quantize.restype = ctypes.c_int
     L.pmxhip_kv_cache_quantize.argtypes = [ctypes.POINTER(KvstoreParams), c_vp]
+    L.pmxhip_rotary_position_embedding.restype = ctypes.c_int
+    L.pmxhip_rotary_position_embedding.argtypes = [ctypes.POINTER(RopeParams), c_vp]
+    L.pmxhip_rope_kv_cache_quantize.restype = ctypes.c_int
+    L.pmxhip_rope_kv_cache_quantize.argtypes = [ctypes.POINTER(RopeParams), ctypes.POINTER(KvstoreParams), c_vp]
     L.pmxhip_kv_cache_reorder.restype = ctypes.c_int
     L.pmxhip_kv_cache_reorder.argtypes = [c_vp] * 4 + [ctypes.POINTER(ReorderStride)] * 2 + [c_i64] * 8 + [c_vp]
     L.pmxhip_kv_cache_invert_reorder.restype = ctypes.c_int

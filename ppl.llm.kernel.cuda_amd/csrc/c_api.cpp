@@ -427,4 +427,83 @@ int pmxhip_kv_cache_invert_reorder(pmxhip_stream_t stream, const void* outer_mem
                           page_nums, layers, kv_heads, tokens, head_dim, group_size, tp_rank, tp_size);
 }
 
+static int rope_common(const char* what, const pmxhip_rope_params* p, const pmxhip_kvstore_params* st, pmxhip_stream_t stream)
+{
+    if (!p) return fail(PMXHIP_INVALID_VALUE, "%s: null params", what);
+    if (p->head_dim <= 0 || p->head_dim % 8 != 0 || p->head_dim > 256)
+        return fail(PMXHIP_UNSUPPORTED, "%s: head_dim must be a multiple of 8, at most 256", what);
+    if (p->rotary_dim < 0 || p->rotary_dim % 2 != 0 || p->rotary_dim > p->head_dim) // rotary_position_embedding.cu:395-398
+        return fail(PMXHIP_INVALID_VALUE, "%s: rotary_dim should be an even number not above head_dim", what);
+    if (p->scaling_type < 0 || p->scaling_type > 2) return fail(PMXHIP_INVALID_VALUE, "%s: invalid scaling type: %d", what, p->scaling_type);
+    if (p->scaling_type != 0 && !(p->scaling_factor > 0.f)) return fail(PMXHIP_INVALID_VALUE, "%s: scaling_factor must be positive", what);
+    if (p->batch < 0 || p->max_seqlen < 0 || p->num_heads <= 0 || p->num_key_heads < 0 || p->num_key_heads > p->num_heads)
+        return fail(PMXHIP_INVALID_VALUE, "%s: bad batch/max_seqlen/heads", what);
+    if (p->batch == 0 || p->max_seqlen == 0) return PMXHIP_SUCCESS;
+    if (!p->query || !p->key || !p->start_pos || !p->seqstarts || !p->rotated_query || (!st && !p->rotated_key))
+        return fail(PMXHIP_INVALID_VALUE, "%s: null device pointer", what);
+    if (!aligned16(p->query) || !aligned16(p->key) || !aligned16(p->rotated_query) || (p->rotated_key && !aligned16(p->rotated_key)) ||
+        p->query_stride_s % 8 || p->key_stride_s % 8 || p->rotated_query_stride_s % 8 || p->rotated_key_stride_s % 8)
+        return fail(PMXHIP_UNSUPPORTED, "%s: rows must be 16-byte aligned", what);
+
+    pmxhip::RopeLaunch a{};
+    a.query = p->query;
+    a.key = p->key;
+    a.rotated_query = p->rotated_query;
+    a.rotated_key = p->rotated_key;
+    a.seqstarts = p->seqstarts;
+    a.start_pos = p->start_pos;
+    a.batch = p->batch;
+    a.max_tokens = p->batch * p->max_seqlen;
+    a.num_heads = p->num_heads;
+    a.num_key_heads = p->num_key_heads;
+    a.head_dim = (int32_t)p->head_dim;
+    a.rotary_dim = (int32_t)p->rotary_dim;
+    a.query_stride_s = p->query_stride_s;
+    a.key_stride_s = p->key_stride_s;
+    a.rotated_query_stride_s = p->rotated_query_stride_s;
+    a.rotated_key_stride_s = p->rotated_key_stride_s;
+    a.theta = p->theta;
+    a.scaling_factor = p->scaling_factor;
+    a.max_position_embeddings = p->max_position_embeddings;
+    a.scaling_type = p->scaling_type;
+    a.bypass_key = p->bypass_key;
+    if (st) {
+        if (st->head_dim != p->head_dim || st->num_kv_heads != p->num_key_heads || st->batch != p->batch ||
+            st->seqstarts != p->seqstarts || st->start_pos != p->start_pos)
+            return fail(PMXHIP_INVALID_VALUE, "%s: the append part must describe the same rows as the rotation", what);
+        if (int rc = check_cache_layout(what, st->cache_mode, st->page_size, st->cache_stride_s, st->cache_stride_l,
+                                        st->cache_stride_h, st->cache_stride_kv, 8))
+            return rc;
+        if (!st->current_value || !st->cachestarts || !st->cache || !st->scale)
+            return fail(PMXHIP_INVALID_VALUE, "%s: null device pointer", what);
+        if (st->current_value_stride_s % 8 || !aligned16(st->current_value) || (reinterpret_cast<uintptr_t>(st->cache) & 7u))
+            return fail(PMXHIP_UNSUPPORTED, "%s: current_value needs 16-byte aligned rows, cache 8-byte alignment", what);
+        a.value = st->current_value;
+        a.value_stride_s = st->current_value_stride_s;
+        a.cache = static_cast<int8_t*>(st->cache);
+        a.scale = st->scale;
+        a.cachestarts = st->cachestarts;
+        a.layer_idx = st->layer_idx;
+        a.cache_stride_s = st->cache_stride_s;
+        a.cache_stride_l = st->cache_stride_l;
+        a.cache_stride_h = st->cache_stride_h;
+        a.cache_stride_kv = st->cache_stride_kv;
+        a.cachestarts_stride_b = st->cachestarts_stride_b;
+        a.cache_mode = st->cache_mode;
+    }
+    if (pmxhip::launch_rope(a, stream) != 0) return fail(PMXHIP_UNSUPPORTED, "%s: no kernel for this shape", what);
+    return launch_status(what);
+}
+
+int pmxhip_rotary_position_embedding(const pmxhip_rope_params* p, pmxhip_stream_t stream)
+{
+    return rope_common("rotary_position_embedding", p, nullptr, stream);
+}
+
+int pmxhip_rope_kv_cache_quantize(const pmxhip_rope_params* rope, const pmxhip_kvstore_params* store, pmxhip_stream_t stream)
+{
+    if (!store) return fail(PMXHIP_INVALID_VALUE, "rope_kv_cache_quantize: null params");
+    return rope_common("rope_kv_cache_quantize", rope, store, stream);
+}
+
 } // extern "C"

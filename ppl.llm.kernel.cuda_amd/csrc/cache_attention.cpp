@@ -15,6 +15,7 @@
 #include "pmx_hip/c_api.h"
 #include "pmx_hip/key_value_cache.h"
 #include "pmx_hip/kv_cache_reorder.h"
+#include "pmx_hip/rotary_position_embedding.h"
 
 namespace ppl { namespace kernel { namespace llm { namespace cuda { namespace pmx {
 
@@ -404,6 +405,131 @@ ppl::common::RetCode kv_cache_invert_reorder(
     return to_retcode(pmxhip_kv_cache_invert_reorder(stream, outer_mem, static_cast<const int64_t*>(page_ids), &s, &d, page_nums,
                                                      layers, kv_heads, tokens, head_dim, group_size, tp_rank, tp_size, kv_cache,
                                                      kv_scale));
+}
+
+static ppl::common::RetCode fill_rope_params(
+    pmxhip_rope_params& p,
+    const ppl::common::TensorShape* query_shape, const void* query, const ppl::common::TensorShape* key_shape, const void* key,
+    const void* start_pos, const void* seqstarts, const float theta, const int32_t bypass_key, const int64_t rotary_dim,
+    const int64_t batch, const int64_t num_heads, const int64_t num_key_heads, const int64_t max_seqlen,
+    const int64_t max_position_embeddings, const rope_scaling_t scaling_type, const float scaling_factor,
+    const ppl::common::TensorShape* rotated_query_shape, void* rotated_query,
+    const ppl::common::TensorShape* rotated_key_shape, void* rotated_key)
+{
+    // checks of rotary_position_embedding.cu:368-398
+    if (query_shape->GetDataType() != ppl::common::DATATYPE_FLOAT16) {
+        PMX_LOG_ERROR("only support fp16");
+        return ppl::common::RC_UNSUPPORTED;
+    }
+    if (query_shape->GetDimCount() != 3 || key_shape->GetDimCount() != 3 || rotated_query_shape->GetDimCount() != 3 ||
+        (rotated_key && rotated_key_shape->GetDimCount() != 3)) {
+        PMX_LOG_ERROR("query, key, rotated_query and rotated_key must have 3 dims");
+        return ppl::common::RC_INVALID_VALUE;
+    }
+    const int64_t head_dim = query_shape->GetDim(2);
+    if (head_dim % 2 != 0 || rotary_dim % 2 != 0) {
+        PMX_LOG_ERROR("head_dim and rotary_dim should be even numbers");
+        return ppl::common::RC_INVALID_VALUE;
+    }
+    memset(&p, 0, sizeof(p));
+    p.query = query;
+    p.key = key;
+    p.start_pos = static_cast<const int64_t*>(start_pos);
+    p.seqstarts = static_cast<const int64_t*>(seqstarts);
+    p.theta = theta;
+    p.bypass_key = bypass_key;
+    p.rotary_dim = rotary_dim;
+    p.batch = batch;
+    p.num_heads = num_heads;
+    p.num_key_heads = num_key_heads;
+    p.head_dim = head_dim;
+    p.max_seqlen = max_seqlen;
+    p.max_position_embeddings = max_position_embeddings;
+    p.scaling_type = scaling_type;
+    p.scaling_factor = scaling_factor;
+    p.query_stride_s = query_shape->GetDim(1) * head_dim; // lines 411-414: dim[1] is the leading dim of heads
+    p.key_stride_s = key_shape->GetDim(1) * head_dim;
+    p.rotated_query_stride_s = rotated_query_shape->GetDim(1) * head_dim;
+    p.rotated_key_stride_s = rotated_key ? rotated_key_shape->GetDim(1) * head_dim : 0;
+    p.rotated_query = rotated_query;
+    p.rotated_key = rotated_key;
+    return ppl::common::RC_SUCCESS;
+}
+
+ppl::common::RetCode dynamic_batching_rotary_position_embedding(
+    hipStream_t stream,
+    const ppl::common::TensorShape* query_shape, const void* query,
+    const ppl::common::TensorShape* key_shape, const void* key,
+    const void* start_pos, const void* seqstarts,
+    const float theta, const int32_t bypass_key, const int64_t rotary_dim,
+    const int64_t batch, const int64_t num_heads, const int64_t num_key_heads,
+    const int64_t max_seqlen, const int64_t max_position_embeddings,
+    const rope_scaling_t scaling_type, const float scaling_factor,
+    const ppl::common::TensorShape* rotated_query_shape, void* rotated_query,
+    const ppl::common::TensorShape* rotated_key_shape, void* rotated_key)
+{
+    pmxhip_rope_params p;
+    const ppl::common::RetCode rc = fill_rope_params(p, query_shape, query, key_shape, key, start_pos, seqstarts, theta, bypass_key,
+                                                     rotary_dim, batch, num_heads, num_key_heads, max_seqlen,
+                                                     max_position_embeddings, scaling_type, scaling_factor, rotated_query_shape,
+                                                     rotated_query, rotated_key_shape, rotated_key);
+    if (rc != ppl::common::RC_SUCCESS) return rc;
+    return to_retcode(pmxhip_rotary_position_embedding(&p, stream));
+}
+
+ppl::common::RetCode dynamic_batching_rotary_position_embedding_kv_cache(
+    hipStream_t stream,
+    const ppl::common::TensorShape* query_shape, const void* query,
+    const ppl::common::TensorShape* key_shape, const void* key,
+    const ppl::common::TensorShape* value_shape, const void* current_value,
+    const void* start_pos, const void* seqstarts,
+    const float theta, const int32_t bypass_key, const int64_t rotary_dim,
+    const int64_t batch, const int64_t num_heads, const int64_t num_key_heads,
+    const int64_t max_seqlen, const int64_t max_position_embeddings,
+    const rope_scaling_t scaling_type, const float scaling_factor,
+    const ppl::common::TensorShape* rotated_query_shape, void* rotated_query,
+    const ppl::common::TensorShape* rotated_key_shape, void* rotated_key,
+    const void* cachestarts, const int64_t num_layer, const int64_t layer_idx,
+    const int32_t cache_mode, const int64_t page_size,
+    const int64_t cache_stride_s, const int64_t cache_stride_l, const int64_t cache_stride_h,
+    const int64_t cache_stride_kv, const int64_t cachestarts_stride_b,
+    void* cache, void* scale)
+{
+    pmxhip_rope_params p;
+    const ppl::common::RetCode rc = fill_rope_params(p, query_shape, query, key_shape, key, start_pos, seqstarts, theta, bypass_key,
+                                                     rotary_dim, batch, num_heads, num_key_heads, max_seqlen,
+                                                     max_position_embeddings, scaling_type, scaling_factor, rotated_query_shape,
+                                                     rotated_query, rotated_key_shape, rotated_key);
+    if (rc != ppl::common::RC_SUCCESS) return rc;
+    if (value_shape->GetDimCount() != 3) {
+        PMX_LOG_ERROR("current_value's dim should be 3");
+        return ppl::common::RC_INVALID_VALUE;
+    }
+    pmxhip_kvstore_params st;
+    memset(&st, 0, sizeof(st));
+    st.current_key = key;
+    st.current_value = current_value;
+    st.seqstarts = p.seqstarts;
+    st.cachestarts = static_cast<const int64_t*>(cachestarts);
+    st.start_pos = p.start_pos;
+    st.num_layer = num_layer;
+    st.layer_idx = layer_idx;
+    st.num_kv_heads = num_key_heads;
+    st.head_dim = p.head_dim;
+    st.page_size = (int32_t)page_size;
+    st.current_key_stride_s = p.key_stride_s;
+    st.current_value_stride_s = value_shape->GetDim(1) * p.head_dim;
+    st.cache_stride_s = cache_stride_s;
+    st.cache_stride_l = cache_stride_l;
+    st.cache_stride_h = cache_stride_h;
+    st.cache_stride_kv = cache_stride_kv;
+    st.cachestarts_stride_b = cachestarts_stride_b;
+    st.cache = cache;
+    st.scale = scale;
+    st.batch = batch;
+    st.max_seqlen = max_seqlen;
+    st.cache_mode = cache_mode;
+    return to_retcode(pmxhip_rope_kv_cache_quantize(&p, &st, stream));
 }
 
 }}}}} // namespace ppl::kernel::llm::cuda::pmx

@@ -113,7 +113,36 @@ struct PageCopyLaunch {
     int64_t src_stride[5], dst_stride[5];     // layer, K/V plane, kv head, token, byte
 };
 
+// Rotary position embedding of the step's Q and K rows, optionally fused with the quantise/append of
+// the rotated K and of V (cache != nullptr).
+struct RopeLaunch {
+    const void* query;          // half (S, Hq, D)
+    const void* key;            // half (S, KVH, D)
+    const void* value;          // half (S, KVH, D); only read when appending
+    void* rotated_query;        // half; may alias query
+    void* rotated_key;          // half; may be nullptr when appending
+    const int64_t* seqstarts;   // (B + 1)
+    const int64_t* start_pos;   // (B)
+    int64_t batch;
+    int64_t max_tokens;         // upper bound of the number of rows
+    int64_t num_heads, num_key_heads;
+    int32_t head_dim, rotary_dim;
+    int64_t query_stride_s, key_stride_s, value_stride_s, rotated_query_stride_s, rotated_key_stride_s; // in halves
+    float theta, scaling_factor;
+    int64_t max_position_embeddings;
+    int32_t scaling_type;       // 0 none, 1 linear, 2 dynamic
+    int32_t bypass_key;
+    // append part (same meaning as QuantLaunch)
+    int8_t* cache;
+    void* scale;
+    const int64_t* cachestarts;
+    int64_t layer_idx;
+    int64_t cache_stride_s, cache_stride_l, cache_stride_h, cache_stride_kv, cachestarts_stride_b;
+    int32_t cache_mode;
+};
+
 int launch_kv_quantize(const QuantLaunch& a, hipStream_t stream);
+int launch_rope(const RopeLaunch& a, hipStream_t stream);
 void launch_page_copy(const PageCopyLaunch& a, hipStream_t stream);
 int launch_decode(const DecodeLaunch& a, int stage, hipStream_t stream); // stage: 0 both, 1 ranges, 2 combine
 int decode_wg_tokens(int head_dim, int kv_heads_per_group);

@@ -193,6 +193,54 @@ def prefill_attention(query, output, cache, scale, seqstarts, kvstarts, cachesta
     return rc
 
 
+def _rope_params(query, key, start_pos, seqstarts, rotated_query, rotated_key, *, theta, rotary_dim, batch, max_seqlen,
+                 bypass_key=False, max_position_embeddings=2048, scaling_type=0, scaling_factor=1.0):
+    p = _lib.RopeParams()
+    hq, d = int(query.shape[1]), int(query.shape[2])
+    hk = int(key.shape[1])
+    p.query, p.key = _ptr(query), _ptr(key)
+    p.start_pos, p.seqstarts = _ptr(start_pos), _ptr(seqstarts)
+    p.theta, p.bypass_key, p.rotary_dim, p.batch = theta, 1 if bypass_key else 0, rotary_dim, batch
+    p.num_heads, p.num_key_heads, p.head_dim, p.max_seqlen = hq, hk, d, max_seqlen
+    p.max_position_embeddings, p.scaling_type, p.scaling_factor = max_position_embeddings, scaling_type, scaling_factor
+    p.query_stride_s = p.rotated_query_stride_s = hq * d
+    p.key_stride_s = p.rotated_key_stride_s = hk * d
+    p.rotated_query = _ptr(rotated_query)
+    p.rotated_key = _ptr(rotated_key) if rotated_key is not None else None
+    return p
+
+
+def rotary_position_embedding(query, key, start_pos, seqstarts, rotated_query, rotated_key, *, stream=None, check=True, **kw):
+    """Rotates the channel pairs of `query` [S, Hq, D] and `key` [S, KVH, D] (fp16) by their positions."""
+    p = _rope_params(query, key, start_pos, seqstarts, rotated_query, rotated_key, **kw)
+    rc = _lib.lib().pmxhip_rotary_position_embedding(ctypes.byref(p), _stream(stream))
+    if check and rc != RC_SUCCESS:
+        raise PmxError(rc, "rotary_position_embedding")
+    return rc
+
+
+def rope_key_value_cache(query, key, value, start_pos, seqstarts, cachestarts, rotated_query, rotated_key, cache, scale, *,
+                         num_layer, layer_idx, cache_mode, page_size, cache_stride_s, cache_stride_l, cache_stride_h,
+                         cache_stride_kv, cachestarts_stride_b, stream=None, check=True, **kw):
+    """The rotation and, in the same kernel, the quantise/append of the rotated key and of `value`;
+    `rotated_key` may be None."""
+    p = _rope_params(query, key, start_pos, seqstarts, rotated_query, rotated_key, **kw)
+    st = KvstoreParams()
+    st.current_key, st.current_value = _ptr(key), _ptr(value)
+    st.seqstarts, st.cachestarts, st.start_pos = _ptr(seqstarts), _ptr(cachestarts), _ptr(start_pos)
+    st.num_layer, st.layer_idx = num_layer, layer_idx
+    st.num_kv_heads, st.head_dim, st.page_size = p.num_key_heads, p.head_dim, page_size
+    st.current_key_stride_s = st.current_value_stride_s = p.key_stride_s
+    st.cache_stride_s, st.cache_stride_l, st.cache_stride_h = cache_stride_s, cache_stride_l, cache_stride_h
+    st.cache_stride_kv, st.cachestarts_stride_b = cache_stride_kv, cachestarts_stride_b
+    st.cache, st.scale = _ptr(cache), _ptr(scale)
+    st.batch, st.max_seqlen, st.cache_mode = p.batch, p.max_seqlen, cache_mode
+    rc = _lib.lib().pmxhip_rope_kv_cache_quantize(ctypes.byref(p), ctypes.byref(st), _stream(stream))
+    if check and rc != RC_SUCCESS:
+        raise PmxError(rc, "rope_kv_cache_quantize")
+    return rc
+
+
 def kv_cache_reorder(kv_cache, kv_scale, page_ids, src_stride, dst_stride, *, layers, kv_heads, tokens, head_dim,
                      group_size, tp_rank, tp_size, outer_mem, stream=None, check=True):
     """Gathers the pages `page_ids` of the int8 cache and of its scales into `outer_mem`.
