@@ -124,47 +124,57 @@ __global__ __launch_bounds__(kQuantThreads) void kv_quantize_kernel(const QuantL
 template <bool PAGED>
 __global__ __launch_bounds__(kQuantThreads) void rope_append_kernel(const RopeLaunch a)
 {
-    __shared__ float s_cos[128], s_sin[128];
-    const int64_t first = a.seqstarts[0];
-    const int64_t tok = blockIdx.x;
-    if (tok >= a.seqstarts[a.batch] - first) return;
-    const int64_t in_tok = first + tok;
-    const int b = sequence_of(a.seqstarts, (int)a.batch, in_tok);
-    const int64_t seq_pos = in_tok - a.seqstarts[b];
-    const int64_t pos = a.start_pos[b] + seq_pos;
+    // a workgroup takes as many consecutive tokens as its threads can compute coefficients for in one go
+    __shared__ float s_cos[kQuantThreads], s_sin[kQuantThreads];
+    __shared__ int64_t s_row[kQuantThreads / 4];
     const int pairs = a.head_dim >> 1, rd2 = a.rotary_dim >> 1;
+    const int tokens_per_wg = kQuantThreads / pairs; // pairs <= 128
+    const int64_t first = a.seqstarts[0];
+    const int64_t n_tokens = a.seqstarts[a.batch] - first;
+    const int64_t tok0 = (int64_t)blockIdx.x * tokens_per_wg;
+    if (tok0 >= n_tokens) return;
+    const bool append = a.cache != nullptr;
 
-    for (int i = threadIdx.x; i < pairs; i += kQuantThreads) {
-        float c = 1.f, s = 0.f;
-        if (i < rd2) {
-            float th = a.theta;
-            if (a.scaling_type == 2) { // dynamic: rotary_position_embedding.cu:68-91
-                const int64_t pos_end = a.start_pos[b] + (a.seqstarts[b + 1] - a.seqstarts[b]);
-                if (pos_end > a.max_position_embeddings) {
-                    const float base = ((a.scaling_factor * (float)pos_end) / (float)a.max_position_embeddings) - (a.scaling_factor - 1.f);
-                    const float expn = (float)rd2 / (float)(rd2 - 1);
-                    th = a.theta * (float)pow((double)base, (double)expn);
+    {
+        const int tl = threadIdx.x / pairs, i = threadIdx.x - tl * pairs;
+        const int64_t tok = tok0 + tl;
+        if (tl < tokens_per_wg && tok < n_tokens) {
+            const int64_t in_tok = first + tok;
+            const int b = sequence_of(a.seqstarts, (int)a.batch, in_tok);
+            const int64_t pos = a.start_pos[b] + (in_tok - a.seqstarts[b]);
+            float c = 1.f, s = 0.f;
+            if (i < rd2) {
+                float th = a.theta;
+                if (a.scaling_type == 2) { // dynamic: rotary_position_embedding.cu:68-91
+                    const int64_t pos_end = a.start_pos[b] + (a.seqstarts[b + 1] - a.seqstarts[b]);
+                    if (pos_end > a.max_position_embeddings) {
+                        const float base = ((a.scaling_factor * (float)pos_end) / (float)a.max_position_embeddings) - (a.scaling_factor - 1.f);
+                        const float expn = (float)rd2 / (float)(rd2 - 1);
+                        th = a.theta * (float)pow((double)base, (double)expn);
+                    }
                 }
+                const float inv = 1.0f / (float)pow((double)th, (double)((float)i / (float)rd2));
+                const float p = a.scaling_type == 1 ? (float)pos / a.scaling_factor : (float)pos;
+                const float angle = inv * p;
+                c = (float)cos((double)angle);
+                s = (float)sin((double)angle);
             }
-            const float inv = 1.0f / (float)pow((double)th, (double)((float)i / (float)rd2));
-            const float p = a.scaling_type == 1 ? (float)pos / a.scaling_factor : (float)pos;
-            const float angle = inv * p;
-            c = (float)cos((double)angle);
-            s = (float)sin((double)angle);
+            s_cos[threadIdx.x] = c;
+            s_sin[threadIdx.x] = s;
+            if (i == 0 && append)
+                s_row[tl] = token_row<PAGED>(a.cachestarts, PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b, pos);
         }
-        s_cos[i] = c;
-        s_sin[i] = s;
     }
     __syncthreads();
 
-    auto rotate = [&](const u32x4 raw, int d0) -> u32x4 {
+    auto rotate = [&](const u32x4 raw, int d0, int tl) -> u32x4 {
         u32x4 out;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
             const int i = (d0 >> 1) + w;
             const half2_t h = bitcast<half2_t>(raw[w]);
             if (i < rd2) {
-                const float x = (float)h.x, y = (float)h.y, c = s_cos[i], s = s_sin[i];
+                const float x = (float)h.x, y = (float)h.y, c = s_cos[tl * pairs + i], s = s_sin[tl * pairs + i];
                 const half2_t r = {(half_t)(x * c - y * s), (half_t)(y * c + x * s)};
                 out[w] = bitcast<uint32_t>(r);
             } else {
@@ -177,27 +187,29 @@ __global__ __launch_bounds__(kQuantThreads) void rope_append_kernel(const RopeLa
     const int gph = a.head_dim >> 3; // groups of 8 channels per head
     const int q_units = (int)a.num_heads * gph;
     const int k_units = (int)a.num_key_heads * gph;
-    const bool append = a.cache != nullptr;
-    int64_t row = 0;
-    if (append) row = token_row<PAGED>(a.cachestarts, PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b, pos);
-    for (int u = threadIdx.x; u < q_units + k_units; u += kQuantThreads) {
+    const int units = q_units + k_units;
+    int n_here = tokens_per_wg;
+    if (tok0 + n_here > n_tokens) n_here = (int)(n_tokens - tok0);
+    for (int w = threadIdx.x; w < n_here * units; w += kQuantThreads) {
+        const int tl = w / units, u = w - tl * units;
+        const int64_t in_tok = first + tok0 + tl;
         if (u < q_units) {
             const int h = u / gph, d0 = (u - h * gph) << 3;
             const int64_t idx = (int64_t)h * a.head_dim + d0;
             const u32x4 raw = *(const u32x4*)((const half_t*)a.query + in_tok * a.query_stride_s + idx);
-            *(u32x4*)((half_t*)a.rotated_query + in_tok * a.rotated_query_stride_s + idx) = rotate(raw, d0);
+            *(u32x4*)((half_t*)a.rotated_query + in_tok * a.rotated_query_stride_s + idx) = rotate(raw, d0, tl);
         } else {
             const int uk = u - q_units;
             const int h = uk / gph, d0 = (uk - h * gph) << 3;
             const int64_t idx = (int64_t)h * a.head_dim + d0;
             u32x4 kraw = *(const u32x4*)((const half_t*)a.key + in_tok * a.key_stride_s + idx);
-            if (!a.bypass_key) kraw = rotate(kraw, d0);
+            if (!a.bypass_key) kraw = rotate(kraw, d0, tl);
             if (a.rotated_key) *(u32x4*)((half_t*)a.rotated_key + in_tok * a.rotated_key_stride_s + idx) = kraw;
             if (append) {
                 const u32x4 vraw = *(const u32x4*)((const half_t*)a.value + in_tok * a.value_stride_s + idx);
                 const Quantised kq = quantise_group(kraw);
                 const Quantised vq = quantise_group(vraw);
-                const int64_t k_out = row * a.cache_stride_s + a.layer_idx * a.cache_stride_l + (int64_t)h * a.cache_stride_h + d0;
+                const int64_t k_out = s_row[tl] * a.cache_stride_s + a.layer_idx * a.cache_stride_l + (int64_t)h * a.cache_stride_h + d0;
                 const int64_t v_out = k_out + a.cache_stride_kv;
                 *(u32x2*)(a.cache + k_out) = kq.q;
                 *(u32x2*)(a.cache + v_out) = vq.q;
@@ -211,11 +223,11 @@ __global__ __launch_bounds__(kQuantThreads) void rope_append_kernel(const RopeLa
 int launch_rope(const RopeLaunch& a, hipStream_t stream)
 {
     if (a.max_tokens <= 0) return 0;
-    if (a.head_dim > 256) return 1;
-    if (a.cache_mode == 1)
-        hipLaunchKernelGGL(rope_append_kernel<true>, dim3((unsigned)a.max_tokens), dim3(kQuantThreads), 0, stream, a);
-    else
-        hipLaunchKernelGGL(rope_append_kernel<false>, dim3((unsigned)a.max_tokens), dim3(kQuantThreads), 0, stream, a);
+    if (a.head_dim > 256 || a.head_dim < 8) return 1;
+    const int tokens_per_wg = kQuantThreads / (a.head_dim / 2);
+    const unsigned blocks = (unsigned)((a.max_tokens + tokens_per_wg - 1) / tokens_per_wg);
+    if (a.cache_mode == 1) hipLaunchKernelGGL(rope_append_kernel<true>, dim3(blocks), dim3(kQuantThreads), 0, stream, a);
+    else hipLaunchKernelGGL(rope_append_kernel<false>, dim3(blocks), dim3(kQuantThreads), 0, stream, a);
     return 0;
 }
 
