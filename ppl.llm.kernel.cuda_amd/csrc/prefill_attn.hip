@@ -9,13 +9,14 @@
 // bottom-right: row i sees columns < i + 1 + kvlen - qlen (flash_attn2/src/mask.h:186).
 //
 // Decomposition (this file's own):
-//   * one workgroup (4 waves) = one kv head of one sequence x a tile of query
-//     positions x ALL query heads of that kv head.  The (position, head) pairs
-//     are the 128 "columns" of the tile, 32 per wave, so a dequantised K/V tile
-//     is shared by every query head of the group.
+//   * one workgroup (8 waves, two per SIMD) = one kv head of one sequence x a tile
+//     of query positions x ALL query heads of that kv head.  The (position, head)
+//     pairs are the 256 "columns" of the tile, 32 per wave, so a dequantised K/V
+//     tile is shared by every query head of the group.
 //   * K/V tiles of 64 tokens are dequantised int8 -> fp16 into LDS once per
-//     workgroup; raw bytes of the next tile are prefetched into registers while
-//     the current tile is computed.
+//     workgroup, into one of two buffers: while tile i is multiplied, tile i+1 is
+//     dequantised into the other buffer and the raw bytes of tile i+2 travel from
+//     memory into registers.  One barrier per tile.
 //   * S^T = K Q^T (tokens are MFMA rows, columns stay columns): a lane then owns
 //     one column, so the softmax max/sum are register-local apart from one
 //     exchange between the two half-waves, and the S^T accumulator layout is
@@ -34,9 +35,9 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int kPrefillThreads = 256;
+constexpr int kPrefillThreads = 512;
 constexpr int kBN = 64;        // kv tokens per tile
-constexpr int kCols = 128;     // (position, head) columns per workgroup
+constexpr int kCols = 256;     // (position, head) columns per workgroup, 32 per wave
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kNegBig = -1.0e30f;
 constexpr float kPShift = 14.0f;
@@ -70,11 +71,10 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     // trick, p = hi + lo), and O accumulates hi*hi + lo*hi + hi*lo: at |v| ~ 40 a single fp16
     // rounding of either factor already costs ~1e-2 absolute where contributions cancel.
     extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-    half_t* const sK = (half_t*)smem_raw;
+    // two tile buffers; a buffer holds K (hi, lo) row-major and V (hi, lo) transposed
     // (fp16 K/V need no low parts: the tiles are the values themselves)
-    half_t* const sKlo = sK + kBN * K_STRIDE;
-    half_t* const sV = KV16 ? sKlo : sKlo + kBN * K_STRIDE;
-    half_t* const sVlo = sV + D * V_STRIDE;
+    constexpr int TILE_HALVES = (KV16 ? 1 : 2) * (kBN * K_STRIDE + D * V_STRIDE);
+    half_t* const smem = (half_t*)smem_raw;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -82,15 +82,16 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     const int hh = lane >> 5;   // half-wave
     const int l32 = lane & 31;
 
-    const int b = blockIdx.y;
-    const int kvh = blockIdx.z;
+    // grid: x = (sequence, kv head), y = query tile; workgroups are dispatched x first, so every sequence's
+    // last query tile (the one that walks the most kv tokens) starts before any shorter one
+    const int b = blockIdx.x / (int)a.num_kv_heads;
+    const int kvh = blockIdx.x - b * (int)a.num_kv_heads;
     const int G = (int)(a.num_heads / a.num_kv_heads);
     const int ppw = kCols / G > 0 ? kCols / G : 1; // query positions per workgroup
     const int64_t q_row0 = a.seqstarts[b];
     const int qlen = (int)(a.seqstarts[b + 1] - q_row0);
     const int kvlen = (int)(a.kvstarts[b + 1] - a.kvstarts[b]);
-    // query tiles in descending order: the workgroups that walk the most kv tokens are dispatched first
-    const int p0 = (int)(gridDim.x - 1 - blockIdx.x) * ppw;
+    const int p0 = (int)(gridDim.y - 1 - blockIdx.y) * ppw;
     if (p0 >= qlen) return;
 
     // ---- this lane's column ----
@@ -149,8 +150,9 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     const int k_g = tid % GPT;           // channel group of this thread's K units
     const int k_t0 = tid / GPT;          // first token; further units are kPrefillThreads / GPT tokens apart
     const int v_g = tid % GPT;
-    const int v_q = tid / GPT;           // token quad (tokens 4 v_q .. 4 v_q + 3)
-    const bool v_on = tid < V_THREADS;
+    const int v_q = (tid / GPT) % (kBN / 4); // token quad (tokens 4 v_q .. 4 v_q + 3)
+    const int v_half = tid / V_THREADS;      // which four of the group's eight channels this thread transposes
+    const bool v_on = v_half < 2;
 
     u32x2 k_raw[K_UNITS];
     half_t k_sc[K_UNITS];
@@ -241,7 +243,11 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
             }
         }
     };
-    auto store_tile = [&]() {
+    auto store_tile = [&](int buf) {
+        half_t* const sK = smem + buf * TILE_HALVES;
+        half_t* const sKlo = sK + kBN * K_STRIDE;
+        half_t* const sV = KV16 ? sKlo : sKlo + kBN * K_STRIDE;
+        half_t* const sVlo = sV + D * V_STRIDE;
         if (KV16) {
 #pragma unroll
             for (int u = 0; u < K_UNITS; ++u) *(u32x4*)&sK[(k_t0 + u * K_TSTEP) * K_STRIDE + 8 * k_g] = k16[u];
@@ -249,8 +255,8 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
                 const int grp = v_q >> 2;
                 const int posv = 16 * grp + vt_pos16(4 * (v_q & 3));
 #pragma unroll
-                for (int e8 = 0; e8 < 8; ++e8) {
-                    const int e = (e8 + v_g) & 7; // rotated channel order, as below
+                for (int e4 = 0; e4 < 4; ++e4) {
+                    const int e = 4 * v_half + ((e4 + v_g) & 3); // rotated channel order, as below
                     const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u; // half (e & 1) of two words
                     const int w = e >> 1;
                     const uint32_t w0 = w == 0 ? v16[0][0] : (w == 1 ? v16[0][1] : (w == 2 ? v16[0][2] : v16[0][3]));
@@ -291,8 +297,8 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
             const int grp = v_q >> 2;
             const int posv = 16 * grp + vt_pos16(4 * (v_q & 3));
 #pragma unroll
-            for (int e8 = 0; e8 < 8; ++e8) {
-                const int e = (e8 + v_g) & 7; // rotate the channel order per lane: spreads LDS banks
+            for (int e4 = 0; e4 < 4; ++e4) {
+                const int e = 4 * v_half + ((e4 + v_g) & 3); // rotate the channel order per lane: spreads LDS banks
                 // byte e of each of the four tokens; the byte index is a run-time value, so the
                 // v_perm selector is built instead of templated
                 const uint32_t sel = 0x0c000c00u | (uint32_t)(e & 3) | ((uint32_t)(4 + (e & 3)) << 16);
@@ -313,19 +319,20 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         }
     };
 
+    // Prologue: tile 0 dequantised into buffer 0, raw bytes of tile 1 in registers.
     int64_t row_next = 0;
     if (n_tiles > 0) {
         load_tile(0, tile_row(0));
-        row_next = tile_row(1);
+        store_tile(0);
+        if (n_tiles > 1) load_tile(1, tile_row(1));
+        row_next = tile_row(2);
+        __syncthreads();
     }
     for (int tile = 0; tile < n_tiles; ++tile) {
-        __syncthreads(); // everyone is done reading the previous tile
-        store_tile();
-        __syncthreads();
-        if (tile + 1 < n_tiles) {
-            load_tile(tile + 1, row_next);
-            row_next = tile_row(tile + 2);
-        }
+        const half_t* const sK = smem + (tile & 1) * TILE_HALVES;
+        const half_t* const sKlo = sK + kBN * K_STRIDE;
+        const half_t* const sV = KV16 ? sKlo : sKlo + kBN * K_STRIDE;
+        const half_t* const sVlo = sV + D * V_STRIDE;
 
         // ---- S^T = K Q^T : two 32-token blocks ----
         f32x16 s_acc[2];
@@ -342,6 +349,14 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
                 }
                 s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], s_acc[mb], 0, 0, 0);
             }
+        }
+
+        // ---- while those products run: tile + 1 into the other buffer (every wave is past its reads of that
+        // buffer since the barrier that ended the previous iteration), then the raw bytes of tile + 2 ----
+        if (tile + 1 < n_tiles) store_tile((tile & 1) ^ 1);
+        if (tile + 2 < n_tiles) {
+            load_tile(tile + 2, row_next);
+            row_next = tile_row(tile + 3);
         }
 
         // ---- online softmax per column (element i <-> token 32 mb + 8 (i/4) + 4 hh + i%4) ----
@@ -426,6 +441,7 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
                     o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pfl[mb][t], o_acc[cb], 0, 0, 0);
                     o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[mb][t], o_acc[cb], 0, 0, 0);
                 }
+        __syncthreads(); // tile + 1 is complete in its buffer; this tile's buffer may be overwritten
     }
 
     // ---- normalise and store: element i of block cb <-> channel 32 cb + 8 (i/4) + 4 hh + i%4 ----
@@ -449,8 +465,8 @@ template <int D, int SRC, bool EXTRA>
 static void launch_prefill_variant(const PrefillLaunch& a, dim3 grid, hipStream_t stream)
 {
     // int8 source: K hi/lo tiles + transposed V hi/lo tiles (above the 64 KB static limit for D = 128, hence
-    // dynamic); fp16 source: one K tile and one transposed V tile
-    constexpr size_t lds_bytes = (SRC == 2 ? 1 : 2) * (kBN * (D + 8) + D * (kBN + 8)) * sizeof(half_t);
+    // dynamic); fp16 source: one K tile and one transposed V tile; two buffers of each
+    constexpr size_t lds_bytes = 2 * (SRC == 2 ? 1 : 2) * (kBN * (D + 8) + D * (kBN + 8)) * sizeof(half_t); // two tile buffers
     static const hipError_t once = hipFuncSetAttribute((const void*)prefill_attention_kernel<D, SRC, EXTRA>,
                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     (void)once;
@@ -462,7 +478,7 @@ static void launch_prefill_d(const PrefillLaunch& a, hipStream_t stream)
 {
     const int G = (int)(a.num_heads / a.num_kv_heads);
     const int ppw = kCols / G > 0 ? kCols / G : 1;
-    const dim3 grid((unsigned)((a.max_seqlen + ppw - 1) / ppw), (unsigned)a.prefill_batches, (unsigned)a.num_kv_heads);
+    const dim3 grid((unsigned)(a.prefill_batches * a.num_kv_heads), (unsigned)((a.max_seqlen + ppw - 1) / ppw), 1);
     const bool extra = a.attn_mask != nullptr || a.alibi_slopes != nullptr;
     const int src = a.current_key ? 2 : (a.cache_mode == 1 ? 0 : 1);
     if (extra) {
