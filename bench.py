@@ -182,7 +182,7 @@ def main():
         "stages_us": stages,
         "roofline": {
             "kernel": ("decode_attention_quad_kernel" if bt.head_dim == 128 and bt.num_kv_heads % 8 == 0 and
-                       bt.num_heads // bt.num_kv_heads <= 8 else "decode_attention_kernel"),
+                       3 <= bt.num_heads // bt.num_kv_heads <= 8 else "decode_attention_kernel"),
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,

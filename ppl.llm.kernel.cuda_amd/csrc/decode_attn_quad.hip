@@ -1,14 +1,15 @@
-// Decode attention over the int8 group-8 KV cache, variant for head_dim 128, groups of at
-// most eight query heads per kv head and kv heads in multiples of eight (the common GQA
+// Decode attention over the int8 group-8 KV cache, variant for head_dim 128, groups of three
+// to eight query heads per kv head and kv heads in multiples of eight (the common GQA
 // shapes).  Same semantics, token ranges, pieces and workspace as decode_attn.hip
 // (reference: src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/kernel.cu:229-679,
 // 1115-1891); what differs is the lane layout, chosen so that the matrix pipe computes
 // the q.k products while the vector pipe converts and accumulates:
 //
 //   * A wave owns two kv heads and up to four of their query heads; with more than four query
-//     heads per kv head a second set of four waves takes heads 4..7 of the same kv heads (it
-//     requests the same cache lines at about the same time, so they come from the cache levels
-//     and HBM is still read once).  The four lanes of a quad hold four different TOKENS of the
+//     heads per kv head a second set of four waves takes heads 4..7 of the same kv heads; a
+//     barrier per pair of blocks keeps the two sets within a block of each other, so that the
+//     second request for a cache line is served by the cache levels (without it the sets drift
+//     apart and HBM is read twice).  The four lanes of a quad hold four different TOKENS of the
 //     same 16 channels; the eight quads of a half-wave hold the eight 16-channel chunks of
 //     those tokens; the two half-waves hold the two kv heads.  A block is 16 tokens: step j
 //     of a lane is token 4 j + (lane in quad).
@@ -341,6 +342,10 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
         drain_loads(ka.q8, ka.sc);
         drain_loads(va.q8, va.sc);
         for (int i = 0;;) {
+            // With two sets of waves on the same kv heads, a barrier per pair of blocks keeps the sets within a
+            // block of each other, so that the second set's requests find the lines in the cache levels
+            // (every wave of the workgroup runs the same number of blocks).
+            if (GP > 1) __syncthreads();
             int npos = pos + (i + 1 < nb ? kQuadBlock : 0);
             if (tail_partial && i + 2 == nb) clamp_offsets(npos);
             request_k(kb, npos);
@@ -428,9 +433,11 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
 }
 
 // true when the variant above serves the launch; the caller falls back to the general kernel otherwise
+// (with one or two query heads per kv head the general kernel is the faster one: its arithmetic is light
+// enough to hide behind the cache stream)
 bool decode_quad_applicable(const DecodeLaunch& a)
 {
-    return a.head_dim == kQuadD && a.attn_mask == nullptr && a.kv_heads_per_group == kQuadHeads && a.num_kv_repeats <= 8 &&
+    return a.head_dim == kQuadD && a.attn_mask == nullptr && a.kv_heads_per_group == kQuadHeads && a.num_kv_repeats >= 3 && a.num_kv_repeats <= 8 &&
            a.num_passes == 1 && a.wg_tokens == kQuadBlock && a.output_stride_s % 8 == 0 &&
            (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0;
 }

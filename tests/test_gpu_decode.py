@@ -36,7 +36,7 @@ def run_decode(dev, ranges=0, **kw):
 SHAPES = [
     # (Hq, KVH, D)
     (8, 8, 64), (4, 4, 128), (32, 8, 128), (16, 2, 128), (12, 2, 128), (6, 2, 96), (4, 2, 256), (32, 2, 64),
-    (3, 3, 128), (24, 8, 128), (2, 1, 128), (16, 8, 128), (8, 8, 128), (64, 16, 128),
+    (3, 3, 128), (24, 8, 128), (2, 1, 128), (16, 8, 128), (8, 8, 128), (64, 16, 128), (64, 8, 128), (40, 8, 128),
 ]
 
 
