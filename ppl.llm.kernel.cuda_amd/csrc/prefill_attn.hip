@@ -152,7 +152,7 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     const int v_g = tid % GPT;
     const int v_q = (tid / GPT) % (kBN / 4); // token quad (tokens 4 v_q .. 4 v_q + 3)
     const int v_half = tid / V_THREADS;      // which four of the group's eight channels this thread transposes
-    const bool v_on = v_half < 2;
+    const bool v_on = (2 * V_THREADS == kPrefillThreads) || v_half < 2; // compile-time true when every thread has a unit
 
     u32x2 k_raw[K_UNITS];
     half_t k_sc[K_UNITS];
@@ -243,19 +243,25 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
             }
         }
     };
-    auto store_tile = [&](int buf) {
+    // One slice of the dequantise-and-store of a tile: slices [0, K_UNITS) are this thread's K units, slices
+    // K_UNITS + [0, 4) its four V channels.  Sliced so that the work can be spread between the MFMAs of the
+    // previous tile's products.
+    constexpr int N_SLICES = K_UNITS + 4;
+    auto store_slice = [&](int buf, int slice) {
         half_t* const sK = smem + buf * TILE_HALVES;
         half_t* const sKlo = sK + kBN * K_STRIDE;
         half_t* const sV = KV16 ? sKlo : sKlo + kBN * K_STRIDE;
         half_t* const sVlo = sV + D * V_STRIDE;
         if (KV16) {
 #pragma unroll
-            for (int u = 0; u < K_UNITS; ++u) *(u32x4*)&sK[(k_t0 + u * K_TSTEP) * K_STRIDE + 8 * k_g] = k16[u];
+            for (int u = 0; u < K_UNITS; ++u)
+                if (slice == u) *(u32x4*)&sK[(k_t0 + u * K_TSTEP) * K_STRIDE + 8 * k_g] = k16[u];
             if (v_on) {
                 const int grp = v_q >> 2;
                 const int posv = 16 * grp + vt_pos16(4 * (v_q & 3));
 #pragma unroll
                 for (int e4 = 0; e4 < 4; ++e4) {
+                    if (slice != K_UNITS + e4) continue;
                     const int e = 4 * v_half + ((e4 + v_g) & 3); // rotated channel order, as below
                     const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u; // half (e & 1) of two words
                     const int w = e >> 1;
@@ -274,6 +280,7 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         // K: 8 halves of one (token, group) -> one 128-bit LDS store
 #pragma unroll
         for (int u = 0; u < K_UNITS; ++u) {
+            if (slice != u) continue;
             const half2_t sc = {k_sc[u], k_sc[u]};
             const uint32_t f0 = k_raw[u][0] ^ kFlipSigns, f1 = k_raw[u][1] ^ kFlipSigns;
             const half2_t x0 = cvt_bytes01(f0), x1 = cvt_bytes23(f0), x2 = cvt_bytes01(f1), x3 = cvt_bytes23(f1);
@@ -298,6 +305,7 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
             const int posv = 16 * grp + vt_pos16(4 * (v_q & 3));
 #pragma unroll
             for (int e4 = 0; e4 < 4; ++e4) {
+                if (slice != K_UNITS + e4) continue;
                 const int e = 4 * v_half + ((e4 + v_g) & 3); // rotate the channel order per lane: spreads LDS banks
                 // byte e of each of the four tokens; the byte index is a run-time value, so the
                 // v_perm selector is built instead of templated
@@ -319,6 +327,11 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         }
     };
 
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int k = 0; k < N_SLICES; ++k) store_slice(buf, k);
+    };
+
     // Prologue: tile 0 dequantised into buffer 0, raw bytes of tile 1 in registers.
     int64_t row_next = 0;
     if (n_tiles > 0) {
@@ -334,26 +347,48 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         const half_t* const sV = KV16 ? sKlo : sKlo + kBN * K_STRIDE;
         const half_t* const sVlo = sV + D * V_STRIDE;
 
-        // ---- S^T = K Q^T : two 32-token blocks ----
+        // ---- S^T = K Q^T : two 32-token blocks.  The A fragments come from LDS in batches of QB k-steps, the
+        // next batch requested before the current one is multiplied, so that an MFMA never waits for the
+        // read issued just before it ----
         f32x16 s_acc[2];
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb) {
+        for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) s_acc[mb][i] = 0.f;
+        {
+            constexpr int QB = 4;
+            constexpr int PER_MB = KSTEPS / QB;
+            constexpr int NBATCH = 2 * PER_MB;
+            f16x8 fh[2][QB], fl[2][QB];
+            auto read_batch = [&](int bi, f16x8* ph, f16x8* pl) {
+                const int mb = bi / PER_MB, s0 = (bi % PER_MB) * QB;
 #pragma unroll
-            for (int s = 0; s < KSTEPS; ++s) {
-                const f16x8 kf = *(const f16x8*)&sK[(32 * mb + l32) * K_STRIDE + 16 * s + 8 * hh];
-                if (!KV16) {
-                    const f16x8 kl = *(const f16x8*)&sKlo[(32 * mb + l32) * K_STRIDE + 16 * s + 8 * hh];
-                    s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kl, qf[s], s_acc[mb], 0, 0, 0);
+                for (int j = 0; j < QB; ++j) {
+                    ph[j] = *(const f16x8*)&sK[(32 * mb + l32) * K_STRIDE + 16 * (s0 + j) + 8 * hh];
+                    if (!KV16) pl[j] = *(const f16x8*)&sKlo[(32 * mb + l32) * K_STRIDE + 16 * (s0 + j) + 8 * hh];
                 }
-                s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], s_acc[mb], 0, 0, 0);
+            };
+            read_batch(0, fh[0], fl[0]);
+#pragma unroll
+            for (int bi = 0; bi < NBATCH; ++bi) {
+                if (bi + 1 < NBATCH) read_batch(bi + 1, fh[(bi + 1) & 1], fl[(bi + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0); // keep the requests ahead of the products (the scheduler would sink them)
+                const int mb = bi / PER_MB, s0 = (bi % PER_MB) * QB;
+#pragma unroll
+                for (int j = 0; j < QB; ++j) {
+                    if (!KV16) s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl[bi & 1][j], qf[s0 + j], s_acc[mb], 0, 0, 0);
+                    s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fh[bi & 1][j], qf[s0 + j], s_acc[mb], 0, 0, 0);
+                }
+                // between the batches: slices of tile + 1 into the other buffer (every wave is past its reads of
+                // that buffer since the barrier that ended the previous iteration; after the last tile the slices
+                // rewrite stale bytes into the idle buffer, which keeps this code free of branches)
+#pragma unroll
+                for (int k = 0; k < N_SLICES; ++k)
+                    if (bi == k * NBATCH / N_SLICES) store_slice((tile & 1) ^ 1, k);
             }
         }
 
-        // ---- while those products run: tile + 1 into the other buffer (every wave is past its reads of that
-        // buffer since the barrier that ended the previous iteration), then the raw bytes of tile + 2 ----
-        if (tile + 1 < n_tiles) store_tile((tile & 1) ^ 1);
+        // ---- then the raw bytes of tile + 2 ----
         if (tile + 2 < n_tiles) {
             load_tile(tile + 2, row_next);
             row_next = tile_row(tile + 3);
@@ -426,21 +461,31 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
             }
         l_run += lsum;
 
-        // ---- O^T += V^T P^T ----
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
+        // ---- O^T += V^T P^T : fragment batches of one (32-token block, 16-token step) each, read one ahead ----
+        {
+            f16x8 vh[2][CB], vl[2][CB];
+            auto read_batch = [&](int bi, f16x8* ph, f16x8* pl) {
+                const int mb = bi >> 1, t = bi & 1;
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) {
-                    const f16x8 vf = *(const f16x8*)&sV[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
-                    if (!KV16) {
-                        const f16x8 vl = *(const f16x8*)&sVlo[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
-                        o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vl, pf[mb][t], o_acc[cb], 0, 0, 0);
-                    }
-                    o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pfl[mb][t], o_acc[cb], 0, 0, 0);
-                    o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[mb][t], o_acc[cb], 0, 0, 0);
+                    ph[cb] = *(const f16x8*)&sV[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
+                    if (!KV16) pl[cb] = *(const f16x8*)&sVlo[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
                 }
+            };
+            read_batch(0, vh[0], vl[0]);
+#pragma unroll
+            for (int bi = 0; bi < 4; ++bi) {
+                if (bi + 1 < 4) read_batch(bi + 1, vh[(bi + 1) & 1], vl[(bi + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                const int mb = bi >> 1, t = bi & 1;
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) {
+                    if (!KV16) o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vl[bi & 1][cb], pf[mb][t], o_acc[cb], 0, 0, 0);
+                    o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vh[bi & 1][cb], pfl[mb][t], o_acc[cb], 0, 0, 0);
+                    o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vh[bi & 1][cb], pf[mb][t], o_acc[cb], 0, 0, 0);
+                }
+            }
+        }
         __syncthreads(); // tile + 1 is complete in its buffer; this tile's buffer may be overwritten
     }
 
