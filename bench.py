@@ -91,7 +91,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards by kv head "
-              "with no exchange, see DESIGN.md)" % args.gpus, file=sys.stderr)
+              "with no exchange between GPUs)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     import torch
