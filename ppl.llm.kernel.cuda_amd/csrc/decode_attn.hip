@@ -545,15 +545,26 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(const DecodeLaunch a
             }
         }
         const int n = (int)((w1 - wb < 63 ? w1 - wb : 63) + 1);
-        for (int k = 0; k < n; ++k) {
-            const float wk = __shfl(wt, k);
-            if (wk == 0.f) continue; // empty piece (or one without weight): its workspace row may be stale
-            den += wk;
-            const float* src = a.partial_out + ((wb + k + b) * a.num_heads + h) * D;
+        // four pieces per step: their rows are requested together, then accumulated (an empty piece has
+        // weight zero and a possibly stale workspace row, which is read but never enters the sum)
+        for (int k0 = 0; k0 < n; k0 += 4) {
+            float wk[4], row[4][NC];
 #pragma unroll
-            for (int i = 0; i < NC; ++i) {
-                const int c = lane + 64 * i;
-                if (c < D) o[i] += wk * src[c];
+            for (int u = 0; u < 4; ++u) {
+                const int k = k0 + u < n ? k0 + u : n - 1;
+                wk[u] = k0 + u < n ? __shfl(wt, k) : 0.f;
+                const float* src = a.partial_out + ((wb + k + b) * a.num_heads + h) * D;
+#pragma unroll
+                for (int i = 0; i < NC; ++i) {
+                    const int c = lane + 64 * i;
+                    row[u][i] = c < D ? src[c] : 0.f;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                den += wk[u];
+#pragma unroll
+                for (int i = 0; i < NC; ++i) o[i] += wk[u] != 0.f ? wk[u] * row[u][i] : 0.f;
             }
         }
     }
