@@ -485,28 +485,40 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
 #endif
 }
 
-// One wave per (sequence, query head): merges the pieces the decode kernel left in the
-// workspace.  A sequence with a single piece was already written by the decode kernel.
-template <int D>
-__global__ __launch_bounds__(64) void decode_combine_kernel(const DecodeLaunch a)
+// One workgroup of NW waves per (sequence, query head): merges the pieces the decode kernel left in the
+// workspace.  A sequence with a single piece was already written by the decode kernel.  The (max, exp-sum)
+// pairs are read with lanes over ranges (every wave for itself, so no exchange is needed for the maximum
+// and the denominator); the rows are read four channels per lane, so a wave takes 64 / (D/4) pieces per
+// request and keeps four requests in flight, and the waves share the pieces of a long sequence between
+// them.  Their partial rows are added through LDS.
+template <int D, int NW>
+__global__ __launch_bounds__(64 * NW) void decode_combine_kernel(const DecodeLaunch a)
 {
+    constexpr int LPR = D / 4;    // lanes that cover one piece row
+    constexpr int PPW = 64 / LPR; // piece rows per wave and request (D = 96: two, the last 16 lanes idle)
+    constexpr int SLOTS = NW * PPW;
+    constexpr int U = 4;
+    __shared__ float s_part[SLOTS][D];
     const int b = blockIdx.y;
     const int h = blockIdx.x;
-    const int lane = threadIdx.x;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int sub = lane / LPR, c4 = lane % LPR;
+    const int slot = (tid >> 6) * PPW + sub;
     const int64_t kv_base = a.kvstarts[0];
     const int64_t total = a.kvstarts[a.decoding_batches] - kv_base;
     const int64_t s_beg = a.kvstarts[b] - kv_base;
     const int64_t s_end = a.kvstarts[b + 1] - kv_base;
     half_t* out = (half_t*)a.output + (int64_t)b * a.output_stride_s + (int64_t)h * D;
     if (s_end <= s_beg) { // empty sequence: the reference yields 0/(0+1e-6) = 0 (kernel.cu:516)
-        for (int c = lane; c < D; c += 64) out[c] = (half_t)0.f;
+        for (int c = tid; c < D; c += 64 * NW) out[c] = (half_t)0.f;
         return;
     }
     const int64_t per = tokens_per_range(total, a.ranges, a.wg_tokens, a.min_tokens_per_range);
     const int64_t w0 = s_beg / per, w1 = (s_end - 1) / per;
     if (w0 == w1) return; // one range covers the sequence: final output already written
 
-    // lanes over ranges: (max, exp-sum) of every non-empty piece, then the weights of the merge
+    // lanes over ranges: the maximum over the non-empty pieces
     float M = kNegBig;
     int pieces = 0;
     for (int64_t wb = w0; wb <= w1; wb += 64) {
@@ -527,14 +539,11 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(const DecodeLaunch a
 #pragma unroll
     for (int s = 32; s >= 1; s >>= 1) M = fmaxf(M, __shfl_xor(M, s));
 
-    constexpr int NC = (D + 63) / 64;
-    float o[NC];
-#pragma unroll
-    for (int i = 0; i < NC; ++i) o[i] = 0.f;
+    f32x4 o = {0.f, 0.f, 0.f, 0.f};
     float den = 0.f;
     for (int64_t wb = w0; wb <= w1; wb += 64) {
         const int64_t w = wb + lane;
-        float wt = 0.f;
+        float wt = 0.f; // weight of range wb + lane
         if (w <= w1) {
             int64_t pa, pe;
             const int64_t r0 = w * per;
@@ -544,35 +553,39 @@ __global__ __launch_bounds__(64) void decode_combine_kernel(const DecodeLaunch a
                 wt = a.partial_ml[pi * 2 + 1] * __builtin_amdgcn_exp2f(a.partial_ml[pi * 2] - M);
             }
         }
+        den += wt;
         const int n = (int)((w1 - wb < 63 ? w1 - wb : 63) + 1);
-        // four pieces per step: their rows are requested together, then accumulated (an empty piece has
-        // weight zero and a possibly stale workspace row, which is read but never enters the sum)
-        for (int k0 = 0; k0 < n; k0 += 4) {
-            float wk[4], row[4][NC];
+        // U requests per slot in flight; an empty piece has weight zero and a possibly stale workspace row,
+        // which is read but never enters the sum
+        for (int k0 = 0; k0 < n; k0 += SLOTS * U) {
+            float wk[U];
+            f32x4 row[U];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                const int k = k0 + u < n ? k0 + u : n - 1;
-                wk[u] = k0 + u < n ? __shfl(wt, k) : 0.f;
-                const float* src = a.partial_out + ((wb + k + b) * a.num_heads + h) * D;
-#pragma unroll
-                for (int i = 0; i < NC; ++i) {
-                    const int c = lane + 64 * i;
-                    row[u][i] = c < D ? src[c] : 0.f;
-                }
+            for (int u = 0; u < U; ++u) {
+                const int k = k0 + u * SLOTS + slot;
+                const bool mine = k < n && sub < PPW;
+                const int kc = mine ? k : n - 1;
+                wk[u] = __shfl(wt, kc);
+                if (!mine) wk[u] = 0.f;
+                row[u] = *(const f32x4*)(a.partial_out + ((wb + kc + b) * a.num_heads + h) * D + c4 * 4);
             }
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                den += wk[u];
-#pragma unroll
-                for (int i = 0; i < NC; ++i) o[i] += wk[u] != 0.f ? wk[u] * row[u][i] : 0.f;
-            }
+            for (int u = 0; u < U; ++u)
+                if (wk[u] != 0.f) o += row[u] * wk[u];
         }
     }
-    const float inv = den > 0.f ? 1.f / den : 0.f;
 #pragma unroll
-    for (int i = 0; i < NC; ++i) {
-        const int c = lane + 64 * i;
-        if (c < D) out[c] = (half_t)(o[i] * inv);
+    for (int s = 32; s >= 1; s >>= 1) den += __shfl_xor(den, s);
+    if (sub < PPW) *(f32x4*)&s_part[slot][c4 * 4] = o;
+    __syncthreads();
+    if (tid < LPR) {
+        f32x4 r = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < SLOTS; ++i) r += *(const f32x4*)&s_part[i][tid * 4];
+        const float inv = den > 0.f ? 1.f / den : 0.f;
+        r *= inv;
+        typedef half_t half4_t __attribute__((ext_vector_type(4)));
+        *(half4_t*)(out + tid * 4) = half4_t{(half_t)r[0], (half_t)r[1], (half_t)r[2], (half_t)r[3]};
     }
 }
 
@@ -655,7 +668,15 @@ static int launch_decode_d(const DecodeLaunch& a, int stage, hipStream_t stream)
     }
     if (stage == 1) return 0;
     // always run: it also writes the zero rows of empty sequences
-    hipLaunchKernelGGL((decode_combine_kernel<D>), dim3((unsigned)a.num_heads, (unsigned)a.decoding_batches), dim3(64), 0, stream, a);
+    {
+        // waves per (sequence, head) row by the mean number of pieces per sequence: with many rows of a few
+        // pieces each, extra waves only add dispatch work (measured: 8 / 9 / 13 us for 1 / 2 / 4 waves on 128
+        // sequences of about five pieces, 17 / 12 / 9 us on one sequence of 256 pieces)
+        const dim3 cgrid((unsigned)a.num_heads, (unsigned)a.decoding_batches);
+        if (a.ranges <= 16 * a.decoding_batches) hipLaunchKernelGGL((decode_combine_kernel<D, 1>), cgrid, dim3(64), 0, stream, a);
+        else if (a.ranges <= 48 * a.decoding_batches) hipLaunchKernelGGL((decode_combine_kernel<D, 2>), cgrid, dim3(128), 0, stream, a);
+        else hipLaunchKernelGGL((decode_combine_kernel<D, 4>), cgrid, dim3(256), 0, stream, a);
+    }
     return 0;
 }
 

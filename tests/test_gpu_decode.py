@@ -89,6 +89,20 @@ def test_decode_empty_sequence_and_closed_forms(pkg, oracle):
             np.testing.assert_allclose(got[b], want, rtol=2e-3, atol=1e-6)
 
 
+@pytest.mark.parametrize("shape", [(8, 8, 64), (6, 2, 96), (32, 8, 128), (8, 2, 128), (4, 2, 256)])
+def test_decode_many_pieces_per_sequence(pkg, oracle, shape):
+    """Long sequences cut into many pieces: the combine kernel then shares the pieces of a row between
+    two or four waves (chosen from ranges / sequences), for every row width."""
+    hq, hkv, d = shape
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 300 + d, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                         cache_mode=1, dec_kv_lens=[5000, 700], outliers=True)
+    ref = oracle_decode(oracle, bt, q, cache, scale)
+    for ranges in (20, 40, 120):  # one, two and four waves per row
+        got, plan = run_decode(dev, ranges)
+        assert plan.num_token_ranges == ranges
+        assert_attention_close(got, ref, "shape %s ranges %d" % (shape, ranges))
+
+
 def test_decode_gqa_identical_queries_and_mha_equivalence(pkg, oracle):
     bt, dev, q, cache, scale = make_case(pkg, oracle, 78, num_heads=8, num_kv_heads=2, head_dim=128, cache_mode=0,
                                          dec_kv_lens=[333, 64])
