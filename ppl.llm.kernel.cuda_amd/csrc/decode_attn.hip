@@ -98,10 +98,6 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
     const int64_t r0 = (int64_t)blockIdx.x * per;
     if (r0 >= total) return;
     const int64_t r1 = (r0 + per < total) ? r0 + per : total;
-#ifdef PMX_WG_TRACE
-    const unsigned long long trace_t0 = wall_clock64();
-    const unsigned long long trace_c0 = clock64();
-#endif
 
     // Addressing: a wave-uniform 64-bit base per block (scalar registers) plus a 32-bit per-lane
     // offset: (token in block) * stride_s + (head in group) * stride_h + channel.
@@ -470,19 +466,6 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
         }
         __syncthreads(); // the next piece overwrites the LDS partials
     }
-#ifdef PMX_WG_TRACE
-    if (tid == 0) {
-        unsigned long long* tr = (unsigned long long*)(a.partial_ml + (int64_t)(a.ranges + a.decoding_batches) * a.num_heads * 2);
-        const int64_t wg = blockIdx.x + (int64_t)gridDim.x * (blockIdx.y + (int64_t)gridDim.y * blockIdx.z);
-        unsigned xcc = 0, hwid = 0;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-        tr[wg * 4 + 0] = trace_t0;
-        tr[wg * 4 + 1] = wall_clock64();
-        tr[wg * 4 + 2] = clock64() - trace_c0;
-        tr[wg * 4 + 3] = ((unsigned long long)xcc << 32) | hwid;
-    }
-#endif
 }
 
 // One workgroup of NW waves per (sequence, query head): merges the pieces the decode kernel left in the
