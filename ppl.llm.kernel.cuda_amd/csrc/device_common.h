@@ -110,6 +110,22 @@ __device__ __forceinline__ float dot2_init(half2_t a, half2_t b, float c)
     return r;
 }
 
+// p - float(h.x) and p - float(h.y) in one instruction each: the mixed-precision fused multiply-add reads the
+// half operand in place (exact: the conversion and the subtraction round once, and the result is representable
+// whenever h is p rounded to half)
+__device__ __forceinline__ float sub_half_lo(float p, half2_t h)
+{
+    float r;
+    asm("v_fma_mix_f32 %0, %1, -1.0, %2 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(h), "v"(p));
+    return r;
+}
+__device__ __forceinline__ float sub_half_hi(float p, half2_t h)
+{
+    float r;
+    asm("v_fma_mix_f32 %0, %1, -1.0, %2 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(h), "v"(p));
+    return r;
+}
+
 // Index arrays (kvstarts, cachestarts) are read-only for the whole launch and are read at
 // wave-uniform addresses: viewing them through the constant address space lets the compiler use
 // scalar loads (scalar cache, no vector registers, no vector wait count) for them.

@@ -396,7 +396,8 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
 
         // ---- online softmax per column (element i <-> token 32 mb + 8 (i/4) + 4 hh + i%4) ----
         const int t_base = tile * kBN;
-        const bool need_mask = t_base + kBN > lim;
+        // only the tiles that reach beyond a column's limit need the per-element test (wave-uniform branch)
+        const bool need_mask = __builtin_amdgcn_ballot_w64(t_base + kBN > lim) != 0;
         float mx = kNegBig;
         if (EXTRA) {
             // additive terms per element (log2 units): mask value and alibi distance of (query row, token)
@@ -417,16 +418,19 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
                 }
         } else {
             // maximum of the raw dot products; the (positive) logit scale is applied to it afterwards
+            if (need_mask) {
 #pragma unroll
-            for (int mb = 0; mb < 2; ++mb)
+                for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    if (need_mask) {
+                    for (int i = 0; i < 16; ++i) {
                         const int t = t_base + 32 * mb + 8 * (i >> 2) + 4 * hh + (i & 3);
                         if (t >= lim) s_acc[mb][i] = -INFINITY;
                     }
-                    mx = fmaxf(mx, s_acc[mb][i]);
-                }
+            }
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[mb][i]);
             mx *= sm_scale;
         }
         mx = fmaxf(mx, __shfl_xor(mx, 32));
@@ -453,7 +457,7 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
                 const float p1 = __builtin_amdgcn_exp2f(EXTRA ? s_acc[mb][i + 1] + bias : __builtin_fmaf(s_acc[mb][i + 1], sm_scale, bias));
                 lsum += p0 + p1;
                 const half2_t ph = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(p0, p1));
-                const half2_t pl = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(p0 - (float)ph.x, p1 - (float)ph.y));
+                const half2_t pl = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(sub_half_lo(p0, ph), sub_half_hi(p1, ph)));
                 pf[mb][i >> 3][i & 7] = ph.x;
                 pf[mb][i >> 3][(i & 7) + 1] = ph.y;
                 pfl[mb][i >> 3][i & 7] = pl.x;
