@@ -337,6 +337,16 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
             }
         };
 
+        // An empty statement that every accumulator passes through at the end of a block.  Without it the
+        // register allocator keeps the accumulators of the two unrolled blocks in different registers and
+        // copies all 64 of them twice per loop iteration (8 % of the loop's instructions).
+        auto pin_acc = [&]() {
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int c = 0; c < 16; ++c) asm volatile("" : "+v"(acc[s][c]));
+        };
+
         // software pipeline as in decode_attn.hip: K of block i+1 is requested before the logits of
         // block i, V of block i+1 before the PV of block i; the last block re-requests itself
         drain_loads(ka.q8, ka.sc);
@@ -352,6 +362,7 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
             logits_softmax(ka);
             request_v(vb, kb.boff);
             accumulate_pv(va);
+            pin_acc();
             pos = npos;
             if (++i == nb) break;
             npos = pos + (i + 1 < nb ? kQuadBlock : 0);
@@ -360,6 +371,7 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
             logits_softmax(kb);
             request_v(va, ka.boff);
             accumulate_pv(vb);
+            pin_acc();
             pos = npos;
             if (++i == nb) break;
         }

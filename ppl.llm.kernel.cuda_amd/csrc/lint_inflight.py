@@ -5,7 +5,10 @@ Their cache loads are inline assembly with explicit wait counts, so the compiler
 registers are the target of a load still in flight.  This script reads the gfx950 assembly of a
 translation unit (hipcc -S) and, with the in-order completion model of vector memory operations,
 reports every instruction that reads or writes such a register before a wait covers it (a spill, a
-copy, a reuse).  Exit status 1 when it finds one: such a kernel must not run.
+copy, a reuse).  It also reports an inline-assembly vector instruction that reads the result of the
+transcendental instruction (v_exp_f32, v_rcp_f32, ...) issued directly before it: that use needs a wait
+state, which the compiler inserts for its own instructions but not for the opaque text of an asm
+statement.  Exit status 1 when it finds either: such a kernel must not run.
 
     hipcc ... --cuda-device-only -S file.hip -o file.s && python3 lint_inflight.py file.s
 """
@@ -22,6 +25,7 @@ def registers(text):
     return out
 
 
+TRANS = ('v_exp_', 'v_log_', 'v_rcp_', 'v_rsq_', 'v_sqrt_', 'v_sin_', 'v_cos_')
 LOADS = ('global_load', 'scratch_load', 'buffer_load', 'flat_load')
 STORES = ('global_store', 'scratch_store', 'buffer_store', 'flat_store', 'global_atomic', 'flat_atomic', 'buffer_atomic')
 
@@ -30,7 +34,9 @@ def lint(name, lines):
     queue = []  # outstanding vector memory operations, oldest first: (destination registers, from inline asm)
     in_asm = False
     problems = 0
+    hazards = 0
     asm_loads = 0
+    trans_dst = set()  # destination of the previous instruction when that was a transcendental one
     for no, raw in enumerate(lines):
         t = raw.strip()
         if t.startswith(';;#ASMSTART'):
@@ -43,6 +49,10 @@ def lint(name, lines):
             continue
         t = t.split(';')[0].strip()
         op = t.split()[0]
+        if in_asm and op.startswith('v_') and ',' in t and registers(t.split(',', 1)[1]) & trans_dst:
+            print("  %s:%d: asm instruction reads a transcendental result without a wait state: %s" % (name, no, t[:90]))
+            hazards += 1
+        trans_dst = registers(t.split(',')[0]) if op.startswith(TRANS) else set()
         if op == 's_waitcnt':
             m = re.search(r'vmcnt\((\d+)\)', t)
             if m:
@@ -74,7 +84,7 @@ def lint(name, lines):
         if bad:
             print("  %s:%d: touches v%s with a load in flight: %s" % (name, no, sorted(bad)[:6], t[:90]))
             problems += 1
-    return problems, asm_loads
+    return problems, asm_loads, hazards
 
 
 def main():
@@ -89,10 +99,10 @@ def main():
                 j = i + 1
                 while j < len(src) and 's_endpgm' not in src[j]:
                     j += 1
-                problems, asm_loads = lint(m.group(1), src[i:j])
+                problems, asm_loads, hazards = lint(m.group(1), src[i:j])
                 if asm_loads:
                     checked += 1
-                total += problems if asm_loads else 0
+                total += (problems if asm_loads else 0) + hazards
                 i = j
             i += 1
     print("lint_inflight: %d hand-scheduled kernels checked, %d problems" % (checked, total))
