@@ -231,7 +231,7 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
             for (int c = 0; c < 16; ++c) acc[s][c] = 0.f;
 
         float prob[4][kTB]; // [slot][step]: probabilities of this lane's own tokens
-        auto logits_softmax = [&](KBlock& kx) {
+        auto logits_softmax = [&](KBlock& kx, bool beyond_piece) { // beyond_piece: the block reaches past the piece (wave-uniform)
             float part[4][kTB]; // [head][step], over this lane's 16 channels, log2 units
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
@@ -249,8 +249,7 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
                     else d1 = __builtin_amdgcn_mfma_f32_4x4x4f16(qa[w], kh, d1, 0, 0, 0);
                 }
                 const half2_t sc = bitcast<half2_t>(kx.sc[j]);
-                const float s0 = (float)sc.x * logit_scale;
-                const float s1 = (float)sc.y * logit_scale;
+                const float s0 = (float)sc.x, s1 = (float)sc.y; // the logit scale is applied to the two complete logits below
 #pragma unroll
                 for (int g = 0; g < 4; ++g) part[g][j] = __builtin_fmaf(d1[g], s1, d0[g] * s0);
             }
@@ -267,12 +266,14 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
                 }
                 swap_rows(rb[0], rb[1]);
                 swap_rows(rb[2], rb[3]);
-                l0 = rb[0] + rb[1];
-                l1 = rb[2] + rb[3];
+                l0 = (rb[0] + rb[1]) * logit_scale;
+                l1 = (rb[2] + rb[3]) * logit_scale;
             }
-            const int tk = kx.pos + 4 * row_odd + t4;
-            l0 = tk < pe32 ? l0 : -INFINITY; // only in the last block: tokens beyond the piece
-            l1 = tk + 8 < pe32 ? l1 : -INFINITY;
+            if (beyond_piece) { // only the last block of a piece
+                const int tk = kx.pos + 4 * row_odd + t4;
+                l0 = tk < pe32 ? l0 : -INFINITY;
+                l1 = tk + 8 < pe32 ? l1 : -INFINITY;
+            }
             // block max of the head: both lanes of the row pair
             float mx = fmaxf(l0, l1), my = mx;
             swap_rows(mx, my);
@@ -359,7 +360,7 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
             int npos = pos + (i + 1 < nb ? kQuadBlock : 0);
             if (tail_partial && i + 2 == nb) clamp_offsets(npos);
             request_k(kb, npos);
-            logits_softmax(ka);
+            logits_softmax(ka, tail_partial && i + 1 == nb);
             request_v(vb, kb.boff);
             accumulate_pv(va);
             pin_acc();
@@ -368,7 +369,7 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
             npos = pos + (i + 1 < nb ? kQuadBlock : 0);
             if (tail_partial && i + 2 == nb) clamp_offsets(npos);
             request_k(ka, npos);
-            logits_softmax(kb);
+            logits_softmax(kb, tail_partial && i + 1 == nb);
             request_v(va, ka.boff);
             accumulate_pv(vb);
             pin_acc();
