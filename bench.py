@@ -9,7 +9,9 @@ tile.  Inputs are resident in HBM before the timed region.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3]
 
 Prints one JSON line.  `value` = algorithmic decode bytes of the batch divided by
-the whole step time (GB/s); `roofline` prices the dominant kernel alone (the
+the whole step time (GB/s).  The K timed steps are K layer calls recorded once into a HIP
+graph and replayed (`launch`; `--eager` times host-launched kernels instead, which is
+also reported as `us_per_layer_eager`); `roofline` prices the dominant kernel alone (the
 token-range decode kernel), timed with events on the stream it is launched on;
 `cpu_baseline` is the CPU oracle on a bounded sample of the same batch.
 """
@@ -84,6 +86,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C3m0", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--eager", action="store_true", help="time host-launched kernels only (no HIP graph)")
     ap.add_argument("--ranges", type=int, default=0, help="token ranges for decode (0 = planned)")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (known traffic, for scaling rocprofv3 "
@@ -127,7 +130,28 @@ def main():
     for _ in range(args.steps):
         step()
     torch.cuda.synchronize()
-    step_s = (time.perf_counter() - t0) / args.steps
+    eager_s = (time.perf_counter() - t0) / args.steps
+    step_s, launch = eager_s, "one launch per kernel from the host (eager)"
+    if not args.eager:
+        # The same K layer calls recorded once into a HIP graph and replayed: the way a serving loop runs a
+        # decode step (all layers in one graph).  Every kernel still runs on every replay.
+        side = torch.cuda.Stream()
+        side.wait_stream(stream)
+        with torch.cuda.stream(side):
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(args.steps):
+                    rc = op.forward(side)
+                    if rc != 0:
+                        raise RuntimeError("forward() returned %d during capture" % rc)
+            graph.replay()  # untimed
+            side.synchronize()
+            t0 = time.perf_counter()
+            graph.replay()
+            side.synchronize()
+            step_s = (time.perf_counter() - t0) / args.steps
+        stream.wait_stream(side)
+        launch = "HIP graph of %d layer calls, replayed once" % args.steps
 
     # per-kernel durations: events on the launch stream around each stage
     def time_stage(fn, n):
@@ -168,6 +192,8 @@ def main():
         "warmup": args.warmup,
         "ms_per_step": step_s * 1e3,
         "us_per_layer": step_s * 1e6,
+        "us_per_layer_eager": eager_s * 1e6,
+        "launch": launch,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

@@ -55,6 +55,41 @@ def test_scaled_c5_through_the_operator(pkg, oracle):
     full_step(pkg, oracle, bt, rng)
 
 
+def test_forward_in_a_hip_graph(pkg, oracle):
+    """forward() records no memory-set node and allocates nothing, so a caller can capture it: every replay,
+    with eager calls between the replays, gives the rows of the eager call bit for bit."""
+    bt, rng = pkg.workloads.custom_batch(404, num_heads=32, num_kv_heads=8, head_dim=128, cache_mode=1,
+                                         dec_kv_lens=[700, 2, 1900, 130, 1], prefill_q_lens=[70], prefill_prior=[300],
+                                         outliers=True)
+    cache, scale = host_cache(bt)
+    dev = pkg.harness.DeviceBatch(bt)
+    for b, pos, k_rows, v_rows in oracle_fill_history(oracle, pkg, bt, rng, cache, scale):
+        dev.append_rows(b, pos, k_rows, v_rows)
+    q, k, v = pkg.workloads.step_inputs(bt, rng)
+    dev.set_step_inputs(q, k, v)
+    op = dev.make_operator(specify_decoding_multi_block=1)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        assert op.forward(side) == 0  # also sets the kernels' attributes before the capture
+        side.synchronize()
+        eager = dev.output.clone()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            assert op.forward(side) == 0
+            assert op.forward(side) == 0
+        for rep in range(3):
+            dev.output.fill_(float("nan"))
+            graph.replay()
+            side.synchronize()
+            assert torch.equal(dev.output.view(torch.int16), eager.view(torch.int16)), "replay %d" % rep
+            assert op.forward(side) == 0
+            side.synchronize()
+    oracle_append_step(oracle, bt, k, v, cache, scale)
+    ref = oracle_prefill(oracle, bt, q, cache, scale)
+    ref[:bt.decoding_batches] = oracle_decode(oracle, bt, q, cache, scale)
+    assert_attention_close(eager.float().cpu().numpy(), ref, "eager rows")
+
+
 def test_contiguous_mode_and_stagewise_calls(pkg, oracle):
     bt, rng = pkg.workloads.custom_batch(402, num_heads=8, num_kv_heads=8, head_dim=64, cache_mode=0,
                                          dec_kv_lens=[200, 31], prefill_q_lens=[40], prefill_prior=[9])
