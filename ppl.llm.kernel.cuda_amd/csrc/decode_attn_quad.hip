@@ -123,7 +123,7 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
     const char* const scale_v = scale_k + (a.cache_stride_kv >> 3) * 2;
     const float logit_scale = a.attn_scale * kLog2e;
 
-    int b = find_sequence(kvstarts, (int)a.decoding_batches, r0);
+    int b = find_sequence(kvstarts, a.kvstarts, (int)a.decoding_batches, r0, (int)(threadIdx.x & 63));
     for (; b < a.decoding_batches; ++b) {
         const int64_t s_beg = kvstarts[b] - kv_base;
         if (s_beg >= r1) break;

@@ -84,9 +84,23 @@ __device__ __forceinline__ void piece_bounds(int64_t r0, int64_t r1, int64_t s_b
 }
 
 // first b in [0, n) with starts[b + 1] - starts[0] > g   (starts is non-decreasing)
-__device__ __forceinline__ int find_sequence(const_i64_ptr starts, int n, int64_t g)
+// Every workgroup runs this before it can request its first cache block, so the whole chip waits on it at the
+// start of the kernel.  Up to kCountedSequences entries are counted by the lanes (the answer is the number of
+// entries <= g): independent loads, one memory latency; beyond that, bisection with scalar loads (one latency
+// per halving).
+constexpr int kCountedSequences = 1024;
+__device__ __forceinline__ int find_sequence(const_i64_ptr starts, const int64_t* starts_global, int n, int64_t g, int lane)
 {
     const int64_t base = starts[0];
+    if (n <= kCountedSequences) {
+        int count = 0;
+        for (int i0 = 0; i0 < n; i0 += kWave) {
+            const int i = i0 + lane;
+            const bool below = i < n && starts_global[i + 1] - base <= g;
+            count += __builtin_popcountll(__builtin_amdgcn_ballot_w64(below));
+        }
+        return count;
+    }
     int lo = 0, hi = n; // answer in [lo, hi]
     while (lo < hi) {
         const int mid = (lo + hi) >> 1;
