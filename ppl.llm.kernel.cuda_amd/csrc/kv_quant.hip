@@ -92,7 +92,11 @@ __global__ __launch_bounds__(kQuantThreads) void kv_quantize_kernel(const QuantL
         const int h = gi / groups_per_head;
         const int d0 = (gi - h * groups_per_head) << 3;
         const int64_t in_tok = first + tok;
-        const int b = sequence_of(a.seqstarts, (int)a.batch, in_tok);
+        // decode steps have one new token per sequence: token i then belongs to sequence i, which two independent
+        // loads confirm; otherwise the sequence is found by bisection (a chain of dependent loads)
+        int b;
+        if (tok < a.batch && a.seqstarts[tok] == in_tok && a.seqstarts[tok + 1] > in_tok) b = (int)tok;
+        else b = sequence_of(a.seqstarts, (int)a.batch, in_tok);
         const int64_t pos = a.start_pos[b] + (in_tok - a.seqstarts[b]);
         const int64_t row = token_row<PAGED>(a.cachestarts, PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b, pos);
 
