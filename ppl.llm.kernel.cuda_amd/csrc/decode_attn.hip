@@ -93,7 +93,7 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
     const const_i64_ptr kvstarts = as_constant(a.kvstarts);
     const const_i64_ptr cachestarts = as_constant(a.cachestarts);
     const int64_t kv_base = kvstarts[0];
-    const int64_t total = kvstarts[a.decoding_batches] - kv_base;
+    const int64_t total = stream_length(kvstarts[a.decoding_batches] - kv_base, a.decoding_batches);
     const int64_t per = tokens_per_range(total, a.ranges, wg_tokens, a.min_tokens_per_range);
     const int64_t r0 = (int64_t)blockIdx.x * per;
     if (r0 >= total) return;
@@ -112,9 +112,10 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
 
     int b = find_sequence(kvstarts, a.kvstarts, (int)a.decoding_batches, r0, (int)(threadIdx.x & 63));
     for (; b < a.decoding_batches; ++b) {
-        const int64_t s_beg = kvstarts[b] - kv_base;
-        if (s_beg >= r1) break;
-        const int64_t len = kvstarts[b + 1] - kv_base - s_beg;
+        const int64_t first_token = kvstarts[b] - kv_base;
+        if (stream_length(first_token, b) >= r1) break; // the sequence's interval starts beyond the range
+        const int64_t len = kvstarts[b + 1] - kv_base - first_token;
+        const int64_t s_beg = sequence_origin(first_token, b);
         int64_t pa, pe; // this workgroup's piece [pa, pe) of the sequence, in sequence coordinates
         piece_bounds(r0, r1, s_beg, len, wg_tokens, pa, pe);
         if (pe <= pa) continue;
@@ -489,9 +490,9 @@ __global__ __launch_bounds__(64 * NW) void decode_combine_kernel(const DecodeLau
     const int sub = lane / LPR, c4 = lane % LPR;
     const int slot = (tid >> 6) * PPW + sub;
     const int64_t kv_base = a.kvstarts[0];
-    const int64_t total = a.kvstarts[a.decoding_batches] - kv_base;
-    const int64_t s_beg = a.kvstarts[b] - kv_base;
-    const int64_t s_end = a.kvstarts[b + 1] - kv_base;
+    const int64_t total = stream_length(a.kvstarts[a.decoding_batches] - kv_base, a.decoding_batches);
+    const int64_t s_beg = sequence_origin(a.kvstarts[b] - kv_base, b);
+    const int64_t s_end = s_beg + (a.kvstarts[b + 1] - a.kvstarts[b]);
     half_t* out = (half_t*)a.output + (int64_t)b * a.output_stride_s + (int64_t)h * D;
     if (s_end <= s_beg) { // empty sequence: the reference yields 0/(0+1e-6) = 0 (kernel.cu:516)
         for (int c = tid; c < D; c += 64 * NW) out[c] = (half_t)0.f;

@@ -108,7 +108,7 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
     const const_i64_ptr kvstarts = as_constant(a.kvstarts);
     const const_i64_ptr cachestarts = as_constant(a.cachestarts);
     const int64_t kv_base = kvstarts[0];
-    const int64_t total = kvstarts[a.decoding_batches] - kv_base;
+    const int64_t total = stream_length(kvstarts[a.decoding_batches] - kv_base, a.decoding_batches);
     const int64_t per = tokens_per_range(total, a.ranges, kQuadBlock, a.min_tokens_per_range);
     const int64_t r0 = (int64_t)blockIdx.x * per;
     if (r0 >= total) return;
@@ -125,9 +125,10 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
 
     int b = find_sequence(kvstarts, a.kvstarts, (int)a.decoding_batches, r0, (int)(threadIdx.x & 63));
     for (; b < a.decoding_batches; ++b) {
-        const int64_t s_beg = kvstarts[b] - kv_base;
-        if (s_beg >= r1) break;
-        const int64_t len = kvstarts[b + 1] - kv_base - s_beg;
+        const int64_t first_token = kvstarts[b] - kv_base;
+        if (stream_length(first_token, b) >= r1) break; // the sequence's interval starts beyond the range
+        const int64_t len = kvstarts[b + 1] - kv_base - first_token;
+        const int64_t s_beg = sequence_origin(first_token, b);
         int64_t pa, pe;
         piece_bounds(r0, r1, s_beg, len, kQuadBlock, pa, pe);
         if (pe <= pa) continue;
