@@ -103,6 +103,25 @@ def test_decode_many_pieces_per_sequence(pkg, oracle, shape):
         assert_attention_close(got, ref, "shape %s ranges %d" % (shape, ranges))
 
 
+@pytest.mark.parametrize("shape", [(32, 8, 128), (8, 8, 64)])
+def test_decode_more_sequences_than_the_counted_lookup(pkg, oracle, shape):
+    """1500 short sequences (some empty): a range's first sequence is then found by bisection instead of the
+    one-round count, and most ranges hold many whole sequences."""
+    hq, hkv, d = shape
+    lens = np.random.default_rng(9).integers(1, 40, 1500)
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 500 + d, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                         cache_mode=1, dec_kv_lens=lens.tolist())
+    for b in (0, 7, 700, 1499):
+        bt.kv_lens[b] = 0
+    bt.kvstarts = np.concatenate([[0], np.cumsum(bt.kv_lens)]).astype(np.int64)
+    dev.kvstarts.copy_(torch.from_numpy(bt.kvstarts))
+    ref = oracle_decode(oracle, bt, q, cache, scale)
+    for ranges in (0, 64, 1):
+        got, plan = run_decode(dev, ranges)
+        assert_attention_close(got, ref, "shape %s ranges %d" % (shape, plan.num_token_ranges))
+        assert (got[[0, 7, 700, 1499]] == 0).all()
+
+
 def test_decode_gqa_identical_queries_and_mha_equivalence(pkg, oracle):
     bt, dev, q, cache, scale = make_case(pkg, oracle, 78, num_heads=8, num_kv_heads=2, head_dim=128, cache_mode=0,
                                          dec_kv_lens=[333, 64])
