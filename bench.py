@@ -42,6 +42,16 @@ def read_traffic(workload):
     return None
 
 
+def dominant_kernel(bt):
+    """Name of the token-range kernel the library picks for the batch's shape."""
+    g = bt.num_heads // bt.num_kv_heads
+    if bt.head_dim == 128 and 5 <= g <= 32 and bt.num_kv_heads % 4 == 0:
+        return "decode_attention_mfma_kernel"
+    if bt.head_dim == 128 and bt.num_kv_heads % 8 == 0 and 3 <= g <= 8:
+        return "decode_attention_quad_kernel"
+    return "decode_attention_kernel"
+
+
 def cpu_baseline(oracle, bt, q, cache_host, scale_host, budget_s=2.0):
     """The oracle's decode attention over the first sequences of the batch, sized to the time budget."""
     lay = bt.layout
@@ -218,8 +228,7 @@ def main():
         },
         "stages_us": stages,
         "roofline": {
-            "kernel": ("decode_attention_quad_kernel" if bt.head_dim == 128 and bt.num_kv_heads % 8 == 0 and
-                       3 <= bt.num_heads // bt.num_kv_heads <= 8 else "decode_attention_kernel"),
+            "kernel": dominant_kernel(bt),
             "bound": "hbm",
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,

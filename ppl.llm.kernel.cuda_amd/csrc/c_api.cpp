@@ -155,11 +155,15 @@ int pmxhip_decode_plan_make(int64_t decoding_batches, int64_t num_heads, int64_t
     const int64_t repeats = num_heads / num_kv_heads;
     const int lanes_per_slot = head_dim == 64 ? 4 : (head_dim == 256 ? 16 : 8);
     const int slots_per_wave = 64 / lanes_per_slot;
-    const int kvhb = largest_pow2_divisor_upto(num_kv_heads, slots_per_wave < 8 ? slots_per_wave : 8);
+    // many query heads per kv head: the MFMA kernel, four kv heads per workgroup, all query heads in one pass
+    const bool mfma = pmxhip::decode_mfma_shape(head_dim, num_heads, num_kv_heads);
+    const int kvhb = mfma ? pmxhip::kDecodeMfmaKvHeads
+                          : largest_pow2_divisor_upto(num_kv_heads, slots_per_wave < 8 ? slots_per_wave : 8);
     int gt = 1;
     while (gt < repeats && gt < 8) gt *= 2;
+    if (mfma) gt = pmxhip::kDecodeMfmaColumns;
     const int passes = (int)((repeats + gt - 1) / gt);
-    const int wg_tokens = pmxhip::decode_wg_tokens((int)head_dim, kvhb);
+    const int wg_tokens = mfma ? pmxhip::kDecodeMfmaTokens : pmxhip::decode_wg_tokens((int)head_dim, kvhb);
     const int min_tokens = wg_tokens > 128 ? wg_tokens : 128;
 
     int64_t ranges = num_token_ranges_hint;
@@ -226,7 +230,9 @@ int pmxhip_decode_attention_stage(const pmxhip_decode_params* p, int32_t stage, 
     }
 
     {   // per-lane cache offsets are 32-bit: (tokens of one wave block) * stride_s + (kv heads of a group) * stride_h
-        const int wg_tok = pmxhip::decode_wg_tokens((int)p->head_dim, plan.kv_heads_per_group);
+        const int wg_tok = plan.q_heads_per_pass == pmxhip::kDecodeMfmaColumns
+                               ? pmxhip::kDecodeMfmaTokens
+                               : pmxhip::decode_wg_tokens((int)p->head_dim, plan.kv_heads_per_group);
         const double span = (double)wg_tok * (double)p->cache_stride_s + (double)plan.kv_heads_per_group * (double)p->cache_stride_h;
         if (p->cache_stride_s < 0 || p->cache_stride_h < 0 || span >= 2147483648.0)
             return fail(PMXHIP_UNSUPPORTED, "decode_attention: cache_stride_s/cache_stride_h too large for 32-bit lane offsets");
@@ -263,7 +269,9 @@ int pmxhip_decode_attention_stage(const pmxhip_decode_params* p, int32_t stage, 
     a.kv_heads_per_group = plan.kv_heads_per_group;
     a.q_heads_per_pass = plan.q_heads_per_pass;
     a.num_passes = plan.num_passes;
-    a.wg_tokens = pmxhip::decode_wg_tokens((int)p->head_dim, plan.kv_heads_per_group);
+    a.wg_tokens = plan.q_heads_per_pass == pmxhip::kDecodeMfmaColumns
+                      ? pmxhip::kDecodeMfmaTokens
+                      : pmxhip::decode_wg_tokens((int)p->head_dim, plan.kv_heads_per_group);
     a.min_tokens_per_range = a.wg_tokens > 128 ? a.wg_tokens : 128;
     if (pmxhip::launch_decode(a, stage, stream) != 0) return fail(PMXHIP_UNSUPPORTED, "decode_attention: no kernel for this shape");
     return launch_status("decode_attention");

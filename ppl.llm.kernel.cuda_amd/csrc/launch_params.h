@@ -148,6 +148,13 @@ int launch_decode(const DecodeLaunch& a, int stage, hipStream_t stream); // stag
 int decode_wg_tokens(int head_dim, int kv_heads_per_group);
 bool decode_quad_applicable(const DecodeLaunch& a); // head_dim 128, <= 4 query heads per kv head, kv heads in eights
 void launch_decode_quad(const DecodeLaunch& a, hipStream_t stream);
+// head_dim 128, 5 to 32 query heads per kv head, kv heads in fours: MFMA kernel, groups of four kv heads, 32-token blocks
+bool decode_mfma_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads);
+bool decode_mfma_applicable(const DecodeLaunch& a);
+void launch_decode_mfma(const DecodeLaunch& a, hipStream_t stream);
+constexpr int kDecodeMfmaKvHeads = 4;
+constexpr int kDecodeMfmaTokens = 32;
+constexpr int kDecodeMfmaColumns = 32;
 void launch_splitkv_combine_rows(const float* partial_out, const float* partial_ml, const int64_t* piece_begin,
                                  const int64_t* piece_end, int64_t rows, int64_t head_dim, void* output,
                                  hipStream_t stream);

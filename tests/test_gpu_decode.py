@@ -37,6 +37,7 @@ SHAPES = [
     # (Hq, KVH, D)
     (8, 8, 64), (4, 4, 128), (32, 8, 128), (16, 2, 128), (12, 2, 128), (6, 2, 96), (4, 2, 256), (32, 2, 64),
     (3, 3, 128), (24, 8, 128), (2, 1, 128), (16, 8, 128), (8, 8, 128), (64, 16, 128), (64, 8, 128), (40, 8, 128),
+    (28, 4, 128), (64, 4, 128), (128, 4, 128), (96, 8, 128),
 ]
 
 
@@ -133,9 +134,10 @@ def test_decode_gqa_identical_queries_and_mha_equivalence(pkg, oracle):
         assert np.array_equal(got[:, g], got[:, 0])
 
 
-def test_decode_with_mask(pkg, oracle):
-    bt, dev, q, cache, scale = make_case(pkg, oracle, 79, num_heads=8, num_kv_heads=4, head_dim=128, cache_mode=1,
-                                         dec_kv_lens=[70, 300, 5])
+@pytest.mark.parametrize("heads", [(8, 4), (32, 4)])
+def test_decode_with_mask(pkg, oracle, heads):
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 79, num_heads=heads[0], num_kv_heads=heads[1], head_dim=128,
+                                         cache_mode=1, dec_kv_lens=[70, 300, 5])
     total = int(bt.kvstarts[-1])
     width = (total + 7) // 8 * 8
     rng = np.random.default_rng(3)
