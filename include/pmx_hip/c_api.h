@@ -129,8 +129,8 @@ typedef struct pmxhip_decode_plan {
     int32_t num_token_ranges;   /* workgroups along the kv-token stream */
     int32_t kv_heads_per_group; /* kv heads one workgroup serves */
     int32_t q_heads_per_pass;   /* query heads per kv head served at once: up to 8 from registers, or the 32
-                                   MFMA columns when head_dim is 128, num_kv_repeats is 5..32 and kv heads come
-                                   in fours (then kv_heads_per_group is 4) */
+                                   MFMA columns when head_dim is 128 and num_kv_repeats is 5..32 (3..32 when
+                                   the kv heads do not come in eights); kv_heads_per_group is then 4, 2 or 1 */
     int32_t num_passes;         /* ceil(num_kv_repeats / q_heads_per_pass) */
     int64_t partial_out_size;   /* bytes: float32 partial outputs */
     int64_t partial_ml_size;    /* bytes: float32 (running max, exp-sum) pairs */

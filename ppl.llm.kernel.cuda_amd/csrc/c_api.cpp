@@ -155,9 +155,9 @@ int pmxhip_decode_plan_make(int64_t decoding_batches, int64_t num_heads, int64_t
     const int64_t repeats = num_heads / num_kv_heads;
     const int lanes_per_slot = head_dim == 64 ? 4 : (head_dim == 256 ? 16 : 8);
     const int slots_per_wave = 64 / lanes_per_slot;
-    // many query heads per kv head: the MFMA kernel, four kv heads per workgroup, all query heads in one pass
+    // many query heads per kv head: the MFMA kernels, a wave per kv head, all query heads in one pass
     const bool mfma = pmxhip::decode_mfma_shape(head_dim, num_heads, num_kv_heads);
-    const int kvhb = mfma ? pmxhip::kDecodeMfmaKvHeads
+    const int kvhb = mfma ? pmxhip::decode_mfma_kv_heads(num_kv_heads)
                           : largest_pow2_divisor_upto(num_kv_heads, slots_per_wave < 8 ? slots_per_wave : 8);
     int gt = 1;
     while (gt < repeats && gt < 8) gt *= 2;
@@ -170,7 +170,9 @@ int pmxhip_decode_plan_make(int64_t decoding_batches, int64_t num_heads, int64_t
     if (ranges == 0) {
         const int64_t groups = (num_kv_heads / kvhb) * passes;
         const int cus = compute_units > 0 ? compute_units : 256;
-        ranges = ((int64_t)cus * 2 + groups - 1) / groups;
+        // workgroups that a CU holds at once: two, or as many as its eight MFMA-kernel waves make
+        const int wgs_per_cu = mfma ? pmxhip::kDecodeMfmaWavesPerCu / kvhb : 2;
+        ranges = ((int64_t)cus * wgs_per_cu + groups - 1) / groups;
         const int64_t max_tokens = decoding_batches * (max_kvlen > 0 ? max_kvlen : 1);
         const int64_t useful = (max_tokens + min_tokens - 1) / min_tokens;
         if (ranges > useful) ranges = useful;

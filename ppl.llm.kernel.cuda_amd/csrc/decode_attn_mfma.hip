@@ -15,8 +15,8 @@
 // Exactness follows the prefill kernel: K^ = int8 * scale, V^ and p are kept as hi + lo pairs of halves
 // (2 MFMAs per QK step, 3 per PV step), so no fp16 rounding of the dequantised cache enters the result.
 //
-// Ranges, pieces and the workspace are those of decode_attn.hip: one workgroup (four waves = four kv heads)
-// per token range, cuts on multiples of 32 tokens, float32 pieces merged by decode_combine_kernel.
+// Ranges, pieces and the workspace are those of decode_attn.hip: one workgroup (a wave per kv head: four, or two
+// or one when the kv heads do not come in fours) per token range, cuts on multiples of 32 tokens, float32 pieces merged by decode_combine_kernel.
 #include <cstdlib>
 
 #include "decode_common.h"
@@ -31,7 +31,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kMfmaD = 128;
 constexpr int kMfmaBlock = 32;  // tokens per wave iteration (rows of one MFMA block)
-constexpr int kMfmaHeads = 4;   // kv heads (= waves) per workgroup
+constexpr int kMfmaMaxHeads = 4; // kv heads (= waves) per workgroup: four, or two or one when the kv heads do not come in fours
 constexpr int kMfmaCols = 32;   // columns of the MFMA block: query heads of the kv head, padded
 constexpr int kMfma16Cols = 16; // columns of the narrow variant
 constexpr float kPShift = 14.0f; // p is kept as 2^14 * exp2(logit - max): its half parts stay normal numbers
@@ -59,11 +59,11 @@ __device__ __forceinline__ int vt_index(int row /* from vt_row */, int pos /* 0.
 
 } // namespace
 
-template <bool PAGED, bool MASK>
-__global__ __launch_bounds__(kMfmaHeads * kWave, 2) void decode_attention_mfma_kernel(const DecodeLaunch a)
+template <int NW, bool PAGED, bool MASK>
+__global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(const DecodeLaunch a)
 {
     constexpr int D = kMfmaD;
-    __shared__ __attribute__((aligned(16))) half_t s_vt[kMfmaHeads][2][D * kMfmaBlock]; // [wave][hi, lo]
+    __shared__ __attribute__((aligned(16))) half_t s_vt[NW][2][D * kMfmaBlock]; // [wave][hi, lo]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -71,7 +71,7 @@ __global__ __launch_bounds__(kMfmaHeads * kWave, 2) void decode_attention_mfma_k
     const int l32 = lane & 31; // token row (K operand), channel row (V operand) or column (query head)
     const int hh = lane >> 5;
     const int G = (int)a.num_kv_repeats;
-    const int kvh = blockIdx.y * kMfmaHeads + wave;
+    const int kvh = blockIdx.y * NW + wave;
     half_t* const sV = s_vt[wave][0];
     half_t* const sVlo = s_vt[wave][1];
 
@@ -358,11 +358,11 @@ __global__ __launch_bounds__(kMfmaHeads * kWave, 2) void decode_attention_mfma_k
 //   O^T tile (16 channels x 16 columns, eight per block): A = row `channel 16 cb + r` of the V^T tile,
 //     16-byte block qq, whose eight positions are the tokens of the lane's two S^T accumulators in order:
 //     position 8 qq + 4 tile + i <-> token 16 tile + 4 qq + i; the accumulator holds channels 16 cb + 4 qq + i
-template <bool PAGED, bool MASK>
-__global__ __launch_bounds__(kMfmaHeads * kWave, 2) void decode_attention_mfma16_kernel(const DecodeLaunch a)
+template <int NW, bool PAGED, bool MASK>
+__global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(const DecodeLaunch a)
 {
     constexpr int D = kMfmaD;
-    __shared__ __attribute__((aligned(16))) half_t s_vt[kMfmaHeads][2][D * kMfmaBlock]; // [wave][hi, lo]
+    __shared__ __attribute__((aligned(16))) half_t s_vt[NW][2][D * kMfmaBlock]; // [wave][hi, lo]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -370,7 +370,7 @@ __global__ __launch_bounds__(kMfmaHeads * kWave, 2) void decode_attention_mfma16
     const int r16 = lane & 15;
     const int qq = lane >> 4;
     const int G = (int)a.num_kv_repeats;
-    const int kvh = blockIdx.y * kMfmaHeads + wave;
+    const int kvh = blockIdx.y * NW + wave;
     half_t* const sV = s_vt[wave][0];
     half_t* const sVlo = s_vt[wave][1];
 
@@ -685,43 +685,60 @@ static bool wide_columns_forced()
     return on;
 }
 
-// true when the variants above serve the shape (the plan chooses its grouping from the same test)
+// kv heads per workgroup for a shape that these kernels serve
+int decode_mfma_kv_heads(int64_t num_kv_heads)
+{
+    return num_kv_heads % 4 == 0 ? 4 : (num_kv_heads % 2 == 0 ? 2 : 1);
+}
+
+// true when the variants above serve the shape (the plan chooses its grouping from the same test): five or more query
+// heads per kv head, and three or four where the kv heads do not come in eights (those have decode_attn_quad.hip)
 bool decode_mfma_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads)
 {
     if (!mfma_kernel_enabled()) return false;
     if (head_dim != kMfmaD || num_kv_heads <= 0 || num_heads % num_kv_heads != 0) return false;
     const int64_t g = num_heads / num_kv_heads;
-    return g >= 5 && g <= kMfmaCols && num_kv_heads % kMfmaHeads == 0;
+    return g <= kMfmaCols && (g >= 5 || (g >= 3 && num_kv_heads % 8 != 0));
 }
 
 bool decode_mfma_applicable(const DecodeLaunch& a)
 {
-    return decode_mfma_shape(a.head_dim, a.num_heads, a.num_kv_heads) && a.kv_heads_per_group == kMfmaHeads &&
-           a.num_passes == 1 && a.wg_tokens == kMfmaBlock && a.output_stride_s % 4 == 0 &&
-           (reinterpret_cast<uintptr_t>(a.output) & 7u) == 0;
+    return decode_mfma_shape(a.head_dim, a.num_heads, a.num_kv_heads) &&
+           a.kv_heads_per_group == decode_mfma_kv_heads(a.num_kv_heads) && a.num_passes == 1 &&
+           a.wg_tokens == kMfmaBlock && a.output_stride_s % 4 == 0 && (reinterpret_cast<uintptr_t>(a.output) & 7u) == 0;
 }
 
-void launch_decode_mfma(const DecodeLaunch& a, hipStream_t stream)
+template <int NW>
+static void launch_decode_mfma_nw(const DecodeLaunch& a, hipStream_t stream)
 {
-    const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / kMfmaHeads), 1);
-    const dim3 block(kMfmaHeads * kWave);
+    const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / NW), 1);
+    const dim3 block(NW * kWave);
     const bool paged = a.cache_mode == 1, mask = a.attn_mask != nullptr;
     if (a.num_kv_repeats <= kMfma16Cols && !wide_columns_forced()) {
         if (paged) {
-            if (mask) hipLaunchKernelGGL((decode_attention_mfma16_kernel<true, true>), grid, block, 0, stream, a);
-            else hipLaunchKernelGGL((decode_attention_mfma16_kernel<true, false>), grid, block, 0, stream, a);
+            if (mask) hipLaunchKernelGGL((decode_attention_mfma16_kernel<NW, true, true>), grid, block, 0, stream, a);
+            else hipLaunchKernelGGL((decode_attention_mfma16_kernel<NW, true, false>), grid, block, 0, stream, a);
         } else {
-            if (mask) hipLaunchKernelGGL((decode_attention_mfma16_kernel<false, true>), grid, block, 0, stream, a);
-            else hipLaunchKernelGGL((decode_attention_mfma16_kernel<false, false>), grid, block, 0, stream, a);
+            if (mask) hipLaunchKernelGGL((decode_attention_mfma16_kernel<NW, false, true>), grid, block, 0, stream, a);
+            else hipLaunchKernelGGL((decode_attention_mfma16_kernel<NW, false, false>), grid, block, 0, stream, a);
         }
         return;
     }
     if (paged) {
-        if (mask) hipLaunchKernelGGL((decode_attention_mfma_kernel<true, true>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((decode_attention_mfma_kernel<true, false>), grid, block, 0, stream, a);
+        if (mask) hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, true, true>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, true, false>), grid, block, 0, stream, a);
     } else {
-        if (mask) hipLaunchKernelGGL((decode_attention_mfma_kernel<false, true>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((decode_attention_mfma_kernel<false, false>), grid, block, 0, stream, a);
+        if (mask) hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, false, true>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, false, false>), grid, block, 0, stream, a);
+    }
+}
+
+void launch_decode_mfma(const DecodeLaunch& a, hipStream_t stream)
+{
+    switch (decode_mfma_kv_heads(a.num_kv_heads)) {
+    case 4: launch_decode_mfma_nw<4>(a, stream); break;
+    case 2: launch_decode_mfma_nw<2>(a, stream); break;
+    default: launch_decode_mfma_nw<1>(a, stream); break;
     }
 }
 

@@ -152,7 +152,8 @@ void launch_decode_quad(const DecodeLaunch& a, hipStream_t stream);
 bool decode_mfma_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads);
 bool decode_mfma_applicable(const DecodeLaunch& a);
 void launch_decode_mfma(const DecodeLaunch& a, hipStream_t stream);
-constexpr int kDecodeMfmaKvHeads = 4;
+int decode_mfma_kv_heads(int64_t num_kv_heads); // kv heads (= waves) per workgroup: 4, 2 or 1
+constexpr int kDecodeMfmaWavesPerCu = 8;         // 16 KB of LDS per wave
 constexpr int kDecodeMfmaTokens = 32;
 constexpr int kDecodeMfmaColumns = 32;
 void launch_splitkv_combine_rows(const float* partial_out, const float* partial_ml, const int64_t* piece_begin,

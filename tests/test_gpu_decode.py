@@ -38,6 +38,8 @@ SHAPES = [
     (8, 8, 64), (4, 4, 128), (32, 8, 128), (16, 2, 128), (12, 2, 128), (6, 2, 96), (4, 2, 256), (32, 2, 64),
     (3, 3, 128), (24, 8, 128), (2, 1, 128), (16, 8, 128), (8, 8, 128), (64, 16, 128), (64, 8, 128), (40, 8, 128),
     (28, 4, 128), (64, 4, 128), (128, 4, 128), (96, 8, 128),
+    # the MFMA kernels with one or two kv heads (the share of one GPU under tensor parallelism)
+    (8, 1, 128), (4, 1, 128), (40, 2, 128), (24, 1, 128), (12, 4, 128),
 ]
 
 
