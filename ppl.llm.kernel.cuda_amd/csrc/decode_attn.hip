@@ -181,8 +181,8 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
                 if (kHandScheduled) {
-                    load_b128(kb.q8[j], vo[j], bk);
-                    load_b32(kb.sc[j], vo_sc[j], sk);
+                    load_b128<false>(kb.q8[j], vo[j], bk);
+                    load_b32<false>(kb.sc[j], vo_sc[j], sk);
                 } else {
                     kb.q8[j] = *(const u32x4*)(bk + vo[j]);
                     kb.sc[j] = *(const uint32_t*)(sk + vo_sc[j]);
@@ -195,8 +195,8 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
                 if (kHandScheduled) {
-                    load_b128(vb.q8[j], vo[j], bv);
-                    load_b32(vb.sc[j], vo_sc[j], sv);
+                    load_b128<false>(vb.q8[j], vo[j], bv);
+                    load_b32<false>(vb.sc[j], vo_sc[j], sv);
                 } else {
                     vb.q8[j] = *(const u32x4*)(bv + vo[j]);
                     vb.sc[j] = *(const uint32_t*)(sv + vo_sc[j]);

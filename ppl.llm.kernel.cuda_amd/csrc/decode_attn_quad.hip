@@ -176,8 +176,8 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
             const char* sk = scale_k + (boff >> 3) * 2;
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
-                load_b128(kb.q8[j], vo[j], bk);
-                load_b32(kb.sc[j], vo_sc[j], sk);
+                load_b128<true>(kb.q8[j], vo[j], bk);
+                load_b32<false>(kb.sc[j], vo_sc[j], sk);
             }
         };
         auto request_v = [&](VBlock& vb, int64_t boff) {
@@ -185,8 +185,8 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
             const char* sv = scale_v + (boff >> 3) * 2;
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
-                load_b128(vb.q8[j], vo[j], bv);
-                load_b32(vb.sc[j], vo_sc[j], sv);
+                load_b128<true>(vb.q8[j], vo[j], bv);
+                load_b32<false>(vb.sc[j], vo_sc[j], sv);
             }
         };
 

@@ -23,13 +23,22 @@ static_assert(kTB == 4, "the quad reduce-scatter and the explicit wait counts as
 // staging registers for temporaries and then waits for loads issued only moments earlier, which
 // serialises the memory latency into every iteration.  Vector memory operations complete in issue
 // order, so "at most N still outstanding" identifies exactly which loads have landed.
+// STREAM adds the non-temporal hint.  Every cache byte is read once per step, and a plain read stream runs at
+// 6.7 TB/s with the hint against 6.0 TB/s without it on this chip; but a hinted line does not stay in the
+// cache for a second instruction, so the hint is for loads whose instruction covers whole 128-byte lines that
+// nobody else reads: the int8 rows of the quad kernel (6 % faster; with its scale loads hinted too only 4 %),
+// not the general kernel, whose lanes of a quad read different tokens (60 % slower with the hint).
+template <bool STREAM>
 __device__ __forceinline__ void load_b128(u32x4& dst, uint32_t lane_off, const char* wave_base)
 {
-    asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(dst) : "v"(lane_off), "s"(wave_base) : "memory");
+    if (STREAM) asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=&v"(dst) : "v"(lane_off), "s"(wave_base) : "memory");
+    else asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(dst) : "v"(lane_off), "s"(wave_base) : "memory");
 }
+template <bool STREAM>
 __device__ __forceinline__ void load_b32(uint32_t& dst, uint32_t lane_off, const char* wave_base)
 {
-    asm volatile("global_load_dword %0, %1, %2" : "=&v"(dst) : "v"(lane_off), "s"(wave_base) : "memory");
+    if (STREAM) asm volatile("global_load_dword %0, %1, %2 nt" : "=&v"(dst) : "v"(lane_off), "s"(wave_base) : "memory");
+    else asm volatile("global_load_dword %0, %1, %2" : "=&v"(dst) : "v"(lane_off), "s"(wave_base) : "memory");
 }
 // waits until at most N vector memory operations are outstanding; the values pass through the
 // statement so that no use of them can be scheduled before the wait
