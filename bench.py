@@ -47,7 +47,7 @@ def dominant_kernel(bt):
     g = bt.num_heads // bt.num_kv_heads
     if bt.head_dim == 128 and g <= 32 and (g >= 5 or (g >= 3 and bt.num_kv_heads % 8 != 0)):
         return "decode_attention_mfma16_kernel" if g <= 16 else "decode_attention_mfma_kernel"
-    if bt.head_dim == 128 and bt.num_kv_heads % 8 == 0 and 3 <= g <= 8:
+    if bt.head_dim == 128 and bt.num_kv_heads % 8 == 0 and g <= 8:
         return "decode_attention_quad_kernel"
     return "decode_attention_kernel"
 

@@ -1,6 +1,5 @@
-// Decode attention over the int8 group-8 KV cache, variant for head_dim 128, groups of three
-// to eight query heads per kv head and kv heads in multiples of eight (the common GQA
-// shapes).  Same semantics, token ranges, pieces and workspace as decode_attn.hip
+// Decode attention over the int8 group-8 KV cache, variant for head_dim 128, up to eight query
+// heads per kv head and kv heads in multiples of eight (MHA and the common GQA shapes).  Same semantics, token ranges, pieces and workspace as decode_attn.hip
 // (reference: src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/kernel.cu:229-679,
 // 1115-1891); what differs is the lane layout, chosen so that the matrix pipe computes
 // the q.k products while the vector pipe converts and accumulates:
@@ -446,12 +445,12 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
     }
 }
 
-// true when the variant above serves the launch; the caller falls back to the general kernel otherwise
-// (with one or two query heads per kv head the general kernel is the faster one: its arithmetic is light
-// enough to hide behind the cache stream)
+// true when the variant above serves the launch; the caller falls back to the general kernel otherwise.
+// One or two query heads per kv head leave rows of the 4x4x4 products and three quarters or half of the PV
+// arithmetic unused, but this kernel's row loads take the non-temporal hint, which the general kernel's cannot.
 bool decode_quad_applicable(const DecodeLaunch& a)
 {
-    return a.head_dim == kQuadD && a.attn_mask == nullptr && a.kv_heads_per_group == kQuadHeads && a.num_kv_repeats >= 3 && a.num_kv_repeats <= 8 &&
+    return a.head_dim == kQuadD && a.attn_mask == nullptr && a.kv_heads_per_group == kQuadHeads && a.num_kv_repeats >= 1 && a.num_kv_repeats <= 8 &&
            a.num_passes == 1 && a.wg_tokens == kQuadBlock && a.output_stride_s % 8 == 0 &&
            (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0;
 }
