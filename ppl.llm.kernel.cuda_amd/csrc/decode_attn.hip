@@ -502,60 +502,114 @@ __global__ __launch_bounds__(64 * NW) void decode_combine_kernel(const DecodeLau
     const int64_t w0 = s_beg / per, w1 = (s_end - 1) / per;
     if (w0 == w1) return; // one range covers the sequence: final output already written
 
-    // lanes over ranges: the maximum over the non-empty pieces
-    float M = kNegBig;
-    int pieces = 0;
-    for (int64_t wb = w0; wb <= w1; wb += 64) {
-        const int64_t w = wb + lane;
-        float m = kNegBig;
+    f32x4 o = {0.f, 0.f, 0.f, 0.f};
+    float den = 0.f;
+    if (w1 - w0 < 64) {
+        // at most 64 ranges (one per lane): the first rows are requested together with the (max, sum) pairs,
+        // before their weights are known, so that the two round trips to memory overlap
+        const int n = (int)(w1 - w0) + 1;
+        f32x4 row[U];
+        int src[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k = u * SLOTS + slot;
+            const bool mine = k < n && sub < PPW;
+            src[u] = mine ? k : -1;
+            row[u] = *(const f32x4*)(a.partial_out + ((w0 + (mine ? k : n - 1) + b) * a.num_heads + h) * D + c4 * 4);
+        }
+        float m = kNegBig, l = 0.f;
         bool live = false;
-        if (w <= w1) {
+        if (lane < n) {
+            const int64_t w = w0 + lane;
             int64_t pa, pe;
             const int64_t r0 = w * per;
             piece_bounds(r0, (r0 + per < total) ? r0 + per : total, s_beg, s_end - s_beg, a.wg_tokens, pa, pe);
             live = pe > pa;
-            if (live) m = a.partial_ml[((w + b) * a.num_heads + h) * 2];
-        }
-        pieces += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live));
-        M = fmaxf(M, m);
-    }
-    if (pieces <= 1) return; // the cuts moved onto one boundary: the decode kernel wrote the final output
-#pragma unroll
-    for (int s = 32; s >= 1; s >>= 1) M = fmaxf(M, __shfl_xor(M, s));
-
-    f32x4 o = {0.f, 0.f, 0.f, 0.f};
-    float den = 0.f;
-    for (int64_t wb = w0; wb <= w1; wb += 64) {
-        const int64_t w = wb + lane;
-        float wt = 0.f; // weight of range wb + lane
-        if (w <= w1) {
-            int64_t pa, pe;
-            const int64_t r0 = w * per;
-            piece_bounds(r0, (r0 + per < total) ? r0 + per : total, s_beg, s_end - s_beg, a.wg_tokens, pa, pe);
-            if (pe > pa) {
-                const int64_t pi = (w + b) * a.num_heads + h;
-                wt = a.partial_ml[pi * 2 + 1] * __builtin_amdgcn_exp2f(a.partial_ml[pi * 2] - M);
+            if (live) {
+                const float2 ml = *(const float2*)(a.partial_ml + ((w + b) * a.num_heads + h) * 2);
+                m = ml.x;
+                l = ml.y;
             }
         }
-        den += wt;
-        const int n = (int)((w1 - wb < 63 ? w1 - wb : 63) + 1);
-        // U requests per slot in flight; an empty piece has weight zero and a possibly stale workspace row,
-        // which is read but never enters the sum
-        for (int k0 = 0; k0 < n; k0 += SLOTS * U) {
-            float wk[U];
-            f32x4 row[U];
+        if (__builtin_popcountll(__builtin_amdgcn_ballot_w64(live)) <= 1) return; // the decode kernel wrote the final output
+        float M = m;
+#pragma unroll
+        for (int s = 32; s >= 1; s >>= 1) M = fmaxf(M, __shfl_xor(M, s));
+        const float wt = live ? l * __builtin_amdgcn_exp2f(m - M) : 0.f; // an empty piece's row may be stale: weight zero
+        den = wt;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const float wk = __shfl(wt, src[u] < 0 ? 0 : src[u]);
+            if (src[u] >= 0 && wk != 0.f) o += row[u] * wk;
+        }
+        for (int k0 = SLOTS * U; k0 < n; k0 += SLOTS * U) {
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int k = k0 + u * SLOTS + slot;
                 const bool mine = k < n && sub < PPW;
-                const int kc = mine ? k : n - 1;
-                wk[u] = __shfl(wt, kc);
-                if (!mine) wk[u] = 0.f;
-                row[u] = *(const f32x4*)(a.partial_out + ((wb + kc + b) * a.num_heads + h) * D + c4 * 4);
+                src[u] = mine ? k : -1;
+                row[u] = *(const f32x4*)(a.partial_out + ((w0 + (mine ? k : n - 1) + b) * a.num_heads + h) * D + c4 * 4);
             }
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-                if (wk[u] != 0.f) o += row[u] * wk[u];
+            for (int u = 0; u < U; ++u) {
+                const float wk = __shfl(wt, src[u] < 0 ? 0 : src[u]);
+                if (src[u] >= 0 && wk != 0.f) o += row[u] * wk;
+            }
+        }
+    } else {
+        // lanes over ranges: the maximum over the non-empty pieces
+        float M = kNegBig;
+        int pieces = 0;
+        for (int64_t wb = w0; wb <= w1; wb += 64) {
+            const int64_t w = wb + lane;
+            float m = kNegBig;
+            bool live = false;
+            if (w <= w1) {
+                int64_t pa, pe;
+                const int64_t r0 = w * per;
+                piece_bounds(r0, (r0 + per < total) ? r0 + per : total, s_beg, s_end - s_beg, a.wg_tokens, pa, pe);
+                live = pe > pa;
+                if (live) m = a.partial_ml[((w + b) * a.num_heads + h) * 2];
+            }
+            pieces += __builtin_popcountll(__builtin_amdgcn_ballot_w64(live));
+            M = fmaxf(M, m);
+        }
+        if (pieces <= 1) return; // the cuts moved onto one boundary: the decode kernel wrote the final output
+#pragma unroll
+        for (int s = 32; s >= 1; s >>= 1) M = fmaxf(M, __shfl_xor(M, s));
+
+        for (int64_t wb = w0; wb <= w1; wb += 64) {
+            const int64_t w = wb + lane;
+            float wt = 0.f; // weight of range wb + lane
+            if (w <= w1) {
+                int64_t pa, pe;
+                const int64_t r0 = w * per;
+                piece_bounds(r0, (r0 + per < total) ? r0 + per : total, s_beg, s_end - s_beg, a.wg_tokens, pa, pe);
+                if (pe > pa) {
+                    const int64_t pi = (w + b) * a.num_heads + h;
+                    wt = a.partial_ml[pi * 2 + 1] * __builtin_amdgcn_exp2f(a.partial_ml[pi * 2] - M);
+                }
+            }
+            den += wt;
+            const int n = (int)((w1 - wb < 63 ? w1 - wb : 63) + 1);
+            // U requests per slot in flight; an empty piece has weight zero and a possibly stale workspace row,
+            // which is read but never enters the sum
+            for (int k0 = 0; k0 < n; k0 += SLOTS * U) {
+                float wk[U];
+                f32x4 row[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int k = k0 + u * SLOTS + slot;
+                    const bool mine = k < n && sub < PPW;
+                    const int kc = mine ? k : n - 1;
+                    wk[u] = __shfl(wt, kc);
+                    if (!mine) wk[u] = 0.f;
+                    row[u] = *(const f32x4*)(a.partial_out + ((wb + kc + b) * a.num_heads + h) * D + c4 * 4);
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    if (wk[u] != 0.f) o += row[u] * wk[u];
+            }
         }
     }
 #pragma unroll
