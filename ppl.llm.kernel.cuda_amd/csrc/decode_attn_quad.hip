@@ -167,6 +167,7 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
                 vo_sc[j] = vo[j] >> 2;
             }
         };
+        // (the row loads carry the non-temporal hint unless a second set of waves reads the same lines)
         auto request_k = [&](KBlock& kb, int pos) {
             kb.pos = pos;
             const int64_t boff = row_base_of(pos) * a.cache_stride_s;
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
             const char* sk = scale_k + (boff >> 3) * 2;
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
-                load_b128<true>(kb.q8[j], vo[j], bk);
+                load_b128<GP == 1>(kb.q8[j], vo[j], bk);
                 load_b32<false>(kb.sc[j], vo_sc[j], sk);
             }
         };
@@ -184,7 +185,7 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
             const char* sv = scale_v + (boff >> 3) * 2;
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
-                load_b128<true>(vb.q8[j], vo[j], bv);
+                load_b128<GP == 1>(vb.q8[j], vo[j], bv);
                 load_b32<false>(vb.sc[j], vo_sc[j], sv);
             }
         };
