@@ -127,7 +127,8 @@ typedef struct pmxhip_decode_params {
 
 typedef struct pmxhip_decode_plan {
     int32_t num_token_ranges;   /* workgroups along the kv-token stream */
-    int32_t kv_heads_per_group; /* kv heads one workgroup serves */
+    int32_t kv_heads_per_group; /* kv heads one workgroup serves (the largest power of two up to 8 that divides
+                                   num_kv_heads, fewer for head_dim 256) */
     int32_t q_heads_per_pass;   /* query heads per kv head served at once: up to 8 from registers, or the 32
                                    MFMA columns when head_dim is 128 and num_kv_repeats is 5..32 (3..32 when
                                    the kv heads do not come in eights); kv_heads_per_group is then 4, 2 or 1 */

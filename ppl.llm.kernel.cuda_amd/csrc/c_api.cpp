@@ -170,8 +170,10 @@ int pmxhip_decode_plan_make(int64_t decoding_batches, int64_t num_heads, int64_t
     if (ranges == 0) {
         const int64_t groups = (num_kv_heads / kvhb) * passes;
         const int cus = compute_units > 0 ? compute_units : 256;
-        // workgroups that a CU holds at once: two, or as many as its eight MFMA-kernel waves make
-        const int wgs_per_cu = mfma ? pmxhip::kDecodeMfmaWavesPerCu / kvhb : 2;
+        // workgroups that a CU holds at once: two of four waves, or as many as eight waves make where a kernel with
+        // smaller workgroups serves the shape (a wave per kv head, or per two)
+        const bool quad = !mfma && pmxhip::decode_quad_shape(head_dim, num_heads, num_kv_heads);
+        const int wgs_per_cu = mfma ? pmxhip::kDecodeMfmaWavesPerCu / kvhb : (quad ? 16 / kvhb : 2);
         ranges = ((int64_t)cus * wgs_per_cu + groups - 1) / groups;
         const int64_t max_tokens = decoding_batches * (max_kvlen > 0 ? max_kvlen : 1);
         const int64_t useful = (max_tokens + min_tokens - 1) / min_tokens;
@@ -271,9 +273,10 @@ int pmxhip_decode_attention_stage(const pmxhip_decode_params* p, int32_t stage, 
     a.kv_heads_per_group = plan.kv_heads_per_group;
     a.q_heads_per_pass = plan.q_heads_per_pass;
     a.num_passes = plan.num_passes;
-    a.wg_tokens = plan.q_heads_per_pass == pmxhip::kDecodeMfmaColumns
-                      ? pmxhip::kDecodeMfmaTokens
-                      : pmxhip::decode_wg_tokens((int)p->head_dim, plan.kv_heads_per_group);
+    // tokens that a workgroup takes per step, the unit of the range cuts: a property of the kernel that will run
+    if (plan.q_heads_per_pass == pmxhip::kDecodeMfmaColumns) a.wg_tokens = pmxhip::kDecodeMfmaTokens;
+    else if (!p->attn_mask && pmxhip::decode_quad_shape(p->head_dim, p->num_heads, p->num_kv_heads)) a.wg_tokens = pmxhip::kDecodeQuadTokens;
+    else a.wg_tokens = pmxhip::decode_wg_tokens((int)p->head_dim, plan.kv_heads_per_group);
     a.min_tokens_per_range = a.wg_tokens > 128 ? a.wg_tokens : 128;
     if (pmxhip::launch_decode(a, stage, stream) != 0) return fail(PMXHIP_UNSUPPORTED, "decode_attention: no kernel for this shape");
     return launch_status("decode_attention");

@@ -680,7 +680,7 @@ static void launch_decode_dgt(const DecodeLaunch& a, dim3 grid, hipStream_t stre
 }
 
 // PMX_HIP_DECODE_GENERAL=1 keeps every shape on the general kernel (for comparisons)
-static bool general_kernel_forced()
+bool decode_general_forced()
 {
     static const bool forced = [] {
         const char* e = getenv("PMX_HIP_DECODE_GENERAL");
@@ -693,9 +693,9 @@ template <int D>
 static int launch_decode_d(const DecodeLaunch& a, int stage, hipStream_t stream)
 {
     const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / a.kv_heads_per_group), (unsigned)a.num_passes);
-    if (stage != 2 && D == 128 && decode_mfma_applicable(a) && !general_kernel_forced()) {
+    if (stage != 2 && D == 128 && decode_mfma_applicable(a) && !decode_general_forced()) {
         launch_decode_mfma(a, stream);
-    } else if (stage != 2 && D == 128 && decode_quad_applicable(a) && !general_kernel_forced()) {
+    } else if (stage != 2 && D == 128 && decode_quad_applicable(a) && !decode_general_forced()) {
         launch_decode_quad(a, stream);
     } else if (stage != 2) {
         switch (a.q_heads_per_pass) {

@@ -692,13 +692,13 @@ int decode_mfma_kv_heads(int64_t num_kv_heads)
 }
 
 // true when the variants above serve the shape (the plan chooses its grouping from the same test): five or more query
-// heads per kv head, and three or four where the kv heads do not come in eights (those have decode_attn_quad.hip)
+// heads per kv head, and three or four with an odd number of kv heads (the others have decode_attn_quad.hip)
 bool decode_mfma_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads)
 {
     if (!mfma_kernel_enabled()) return false;
     if (head_dim != kMfmaD || num_kv_heads <= 0 || num_heads % num_kv_heads != 0) return false;
     const int64_t g = num_heads / num_kv_heads;
-    return g <= kMfmaCols && (g >= 5 || (g >= 3 && num_kv_heads % 8 != 0));
+    return g <= kMfmaCols && (g >= 5 || (g >= 3 && num_kv_heads % 2 != 0));
 }
 
 bool decode_mfma_applicable(const DecodeLaunch& a)

@@ -36,7 +36,7 @@ typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int kQuadD = 128;
-constexpr int kQuadHeads = 8;   // kv heads per workgroup (two per wave)
+constexpr int kQuadMaxHeads = 8; // kv heads per workgroup (two per wave): eight, or four or two when the kv heads do not come in eights
 constexpr int kQuadBlock = 16;  // tokens per block
 constexpr int kDppRor8 = 0x128; // row_ror:8 = lane ^ 8 inside a row of 16
 
@@ -85,16 +85,17 @@ __device__ __forceinline__ float quad_lane(float v)
 
 } // namespace
 
-// GP: sets of four query heads per kv head (1 or 2); the workgroup has 4 * GP waves.
-template <bool PAGED, int GP>
-__global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_kernel(const DecodeLaunch a)
+// GP: sets of four query heads per kv head (1 or 2); WP: pairs of kv heads per workgroup (4, 2 or 1); the workgroup
+// has WP * GP waves.
+template <bool PAGED, int GP, int WP>
+__global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kernel(const DecodeLaunch a)
 {
     constexpr int D = kQuadD;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wave = wave_id & 3;      // which pair of kv heads
-    const int g_first = (wave_id >> 2) * 4; // first query head (within the kv head's group) of this wave
+    const int wave = wave_id % WP;      // which pair of kv heads
+    const int g_first = (wave_id / WP) * 4; // first query head (within the kv head's group) of this wave
     const int t4 = lane & 3;           // token within a step
     const int chunk = (lane >> 2) & 7; // channels [16 chunk, 16 chunk + 16)
     const int hsel = lane >> 5;        // which of the wave's two kv heads
@@ -102,7 +103,7 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
     const int g_own = (((lane >> 2) & 1) << 1) | ((lane >> 3) & 1);
     const int row_odd = (lane >> 4) & 1;
     const int G = (int)a.num_kv_repeats; // <= 4 * GP
-    const int kvh = blockIdx.y * kQuadHeads + wave * 2 + hsel;
+    const int kvh = blockIdx.y * (2 * WP) + wave * 2 + hsel;
 
     const const_i64_ptr kvstarts = as_constant(a.kvstarts);
     const const_i64_ptr cachestarts = as_constant(a.cachestarts);
@@ -113,7 +114,7 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
     if (r0 >= total) return;
     const int64_t r1 = (r0 + per < total) ? r0 + per : total;
 
-    const int64_t group_off = a.layer_idx * a.cache_stride_l + (int64_t)(blockIdx.y * kQuadHeads) * a.cache_stride_h;
+    const int64_t group_off = a.layer_idx * a.cache_stride_l + (int64_t)(blockIdx.y * (2 * WP)) * a.cache_stride_h;
     const uint32_t stride_s32 = (uint32_t)a.cache_stride_s; // the host checks that a block's span fits 32 bits
     const uint32_t lane_base = (uint32_t)((int64_t)(wave * 2 + hsel) * a.cache_stride_h + chunk * 16);
     const char* const cache_k = (const char*)a.cache + group_off;
@@ -446,26 +447,53 @@ __global__ __launch_bounds__(kDecodeThreads * GP, 2) void decode_attention_quad_
     }
 }
 
-// true when the variant above serves the launch; the caller falls back to the general kernel otherwise.
+// kv heads per workgroup for a shape that this kernel serves
+int decode_quad_kv_heads(int64_t num_kv_heads)
+{
+    return num_kv_heads % 8 == 0 ? 8 : (num_kv_heads % 4 == 0 ? 4 : 2);
+}
+
+// true when the variant above serves the shape: head_dim 128, an even number of kv heads, up to four query heads
+// per kv head (up to eight with kv heads in eights; decode_attn_mfma.hip takes five and more first).
 // One or two query heads per kv head leave rows of the 4x4x4 products and three quarters or half of the PV
 // arithmetic unused, but this kernel's row loads take the non-temporal hint, which the general kernel's cannot.
+bool decode_quad_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads)
+{
+    if (decode_general_forced()) return false;
+    if (head_dim != kQuadD || num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || num_kv_heads % 2 != 0) return false;
+    const int64_t g = num_heads / num_kv_heads;
+    return g <= 4 || (g <= 8 && num_kv_heads % 8 == 0);
+}
+
+// true when it serves the launch (no attn_mask); the caller falls back to the general kernel otherwise
 bool decode_quad_applicable(const DecodeLaunch& a)
 {
-    return a.head_dim == kQuadD && a.attn_mask == nullptr && a.kv_heads_per_group == kQuadHeads && a.num_kv_repeats >= 1 && a.num_kv_repeats <= 8 &&
-           a.num_passes == 1 && a.wg_tokens == kQuadBlock && a.output_stride_s % 8 == 0 &&
-           (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0;
+    return decode_quad_shape(a.head_dim, a.num_heads, a.num_kv_heads) && a.attn_mask == nullptr &&
+           a.kv_heads_per_group == decode_quad_kv_heads(a.num_kv_heads) && a.num_passes == 1 && a.wg_tokens == kQuadBlock &&
+           a.output_stride_s % 8 == 0 && (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0;
+}
+
+template <int WP>
+static void launch_decode_quad_wp(const DecodeLaunch& a, hipStream_t stream)
+{
+    const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / (2 * WP)), 1);
+    const bool paged = a.cache_mode == 1;
+    if (paged) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1, WP>), grid, dim3(kWave * WP), 0, stream, a);
+    else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1, WP>), grid, dim3(kWave * WP), 0, stream, a);
 }
 
 void launch_decode_quad(const DecodeLaunch& a, hipStream_t stream)
 {
-    const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / kQuadHeads), 1);
-    const bool paged = a.cache_mode == 1;
-    if (a.num_kv_repeats <= 4) {
-        if (paged) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1>), grid, dim3(kDecodeThreads), 0, stream, a);
-        else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1>), grid, dim3(kDecodeThreads), 0, stream, a);
-    } else {
-        if (paged) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 2>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
-        else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 2>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
+    if (a.num_kv_repeats > 4) { // two sets of four waves on eight kv heads
+        const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / kQuadMaxHeads), 1);
+        if (a.cache_mode == 1) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 2, 4>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
+        else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 2, 4>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
+        return;
+    }
+    switch (decode_quad_kv_heads(a.num_kv_heads)) {
+    case 8: launch_decode_quad_wp<4>(a, stream); break;
+    case 4: launch_decode_quad_wp<2>(a, stream); break;
+    default: launch_decode_quad_wp<1>(a, stream); break;
     }
 }
 

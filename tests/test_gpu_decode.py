@@ -40,6 +40,8 @@ SHAPES = [
     (28, 4, 128), (64, 4, 128), (128, 4, 128), (96, 8, 128),
     # the MFMA kernels with one or two kv heads (the share of one GPU under tensor parallelism)
     (8, 1, 128), (4, 1, 128), (40, 2, 128), (24, 1, 128), (12, 4, 128),
+    # the quad kernel with four and two kv heads per workgroup
+    (8, 2, 128), (6, 6, 128), (24, 12, 128), (16, 4, 128),
 ]
 
 

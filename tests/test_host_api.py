@@ -120,6 +120,8 @@ def test_decode_plan(pkg, hip_lib):
     assert plan.q_heads_per_pass == 32 and plan.kv_heads_per_group == 1 and plan.num_token_ranges == 2048
     plan = pkg.ops.decode_plan(64, 16, 2, 128, 8192, cus=256)
     assert plan.q_heads_per_pass == 32 and plan.kv_heads_per_group == 2 and plan.num_token_ranges == 1024
+    plan = pkg.ops.decode_plan(64, 16, 4, 128, 8192, cus=256)  # four kv heads: two waves per workgroup, four workgroups per CU
+    assert plan.q_heads_per_pass == 4 and plan.kv_heads_per_group == 4 and plan.num_token_ranges == 1024
     plan = pkg.ops.decode_plan(4, 48, 3, 64, 512, cus=256)  # G = 16 -> two passes of 8; 3 kv heads -> 1 per group
     assert plan.q_heads_per_pass == 8 and plan.num_passes == 2 and plan.kv_heads_per_group == 1
     plan = pkg.ops.decode_plan(1, 8, 8, 64, 100, cus=256)   # tiny: one range, no workspace
