@@ -43,11 +43,11 @@ def read_traffic(workload):
 
 
 def dominant_kernel(bt):
-    """Name of the token-range kernel the library picks for the batch's shape."""
+    """Name of the token-range kernel the library picks for the batch's shape (no attn_mask)."""
     g = bt.num_heads // bt.num_kv_heads
-    if bt.head_dim == 128 and g <= 32 and (g >= 5 or (g >= 3 and bt.num_kv_heads % 8 != 0)):
+    if bt.head_dim == 128 and g <= 32 and (g >= 5 or (g >= 3 and bt.num_kv_heads % 2 != 0)):
         return "decode_attention_mfma16_kernel" if g <= 16 else "decode_attention_mfma_kernel"
-    if bt.head_dim == 128 and bt.num_kv_heads % 8 == 0 and g <= 8:
+    if bt.head_dim == 128 and bt.num_kv_heads % 2 == 0 and g <= 4:
         return "decode_attention_quad_kernel"
     return "decode_attention_kernel"
 
