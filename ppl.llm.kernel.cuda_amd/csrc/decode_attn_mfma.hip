@@ -695,7 +695,7 @@ int decode_mfma_kv_heads(int64_t num_kv_heads)
 // heads per kv head, and three or four with an odd number of kv heads (the others have decode_attn_quad.hip)
 bool decode_mfma_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads)
 {
-    if (!mfma_kernel_enabled()) return false;
+    if (!mfma_kernel_enabled() || decode_general_forced()) return false;
     if (head_dim != kMfmaD || num_kv_heads <= 0 || num_heads % num_kv_heads != 0) return false;
     const int64_t g = num_heads / num_kv_heads;
     return g <= kMfmaCols && (g >= 5 || (g >= 3 && num_kv_heads % 2 != 0));
