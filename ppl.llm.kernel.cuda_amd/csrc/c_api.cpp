@@ -275,7 +275,9 @@ int pmxhip_decode_attention_stage(const pmxhip_decode_params* p, int32_t stage, 
     a.num_passes = plan.num_passes;
     // tokens that a workgroup takes per step, the unit of the range cuts: a property of the kernel that will run
     if (plan.q_heads_per_pass == pmxhip::kDecodeMfmaColumns) a.wg_tokens = pmxhip::kDecodeMfmaTokens;
-    else if (!p->attn_mask && pmxhip::decode_quad_shape(p->head_dim, p->num_heads, p->num_kv_heads)) a.wg_tokens = pmxhip::kDecodeQuadTokens;
+    else if (pmxhip::decode_quad_shape(p->head_dim, p->num_heads, p->num_kv_heads) &&
+             (!p->attn_mask || pmxhip::decode_quad_mask_ok(p->num_heads, p->num_kv_repeats, p->mask_stride_h)))
+        a.wg_tokens = pmxhip::kDecodeQuadTokens;
     else a.wg_tokens = pmxhip::decode_wg_tokens((int)p->head_dim, plan.kv_heads_per_group);
     a.min_tokens_per_range = a.wg_tokens > 128 ? a.wg_tokens : 128;
     if (pmxhip::launch_decode(a, stage, stream) != 0) return fail(PMXHIP_UNSUPPORTED, "decode_attention: no kernel for this shape");

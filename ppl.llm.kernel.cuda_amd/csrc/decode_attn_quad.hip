@@ -86,8 +86,8 @@ __device__ __forceinline__ float quad_lane(float v)
 } // namespace
 
 // GP: sets of four query heads per kv head (1 or 2); WP: pairs of kv heads per workgroup (4, 2 or 1); the workgroup
-// has WP * GP waves.
-template <bool PAGED, int GP, int WP>
+// has WP * GP waves.  MASK: the additive attn_mask (kernel.cu:319-325), two more requests per block and lane.
+template <bool PAGED, int GP, int WP, bool MASK>
 __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kernel(const DecodeLaunch a)
 {
     constexpr int D = kQuadD;
@@ -159,6 +159,19 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
             vo[j] = (uint32_t)(4 * j + t4) * stride_s32 + lane_base;
             vo_sc[j] = vo[j] >> 2;
         }
+        // attn_mask: this lane's two complete logits belong to head g_own and the tokens 4 row_odd + t4 and + 8 of the
+        // block; byte offsets against a wave-uniform base (the host checks that they fit 32 bits)
+        const char* mask_base = nullptr;
+        uint32_t mo[2] = {0, 0};
+        uint32_t mask_head = 0;
+        if (MASK) {
+            const int g = g_first + g_own;
+            const int h = kvh * G + (g < G ? g : 0);
+            mask_head = (uint32_t)((int64_t)h * a.mask_stride_h * 2);
+            mask_base = (const char*)a.attn_mask + ((int64_t)b * a.mask_stride_s + kvstarts[b]) * 2;
+            mo[0] = mask_head + (uint32_t)(4 * row_odd + t4) * 2;
+            mo[1] = mo[0] + 16;
+        }
         auto clamp_offsets = [&](int pos) { // tokens beyond the piece re-read its last token; their logits are masked
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
@@ -167,9 +180,16 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
                 vo[j] = (uint32_t)(tc - pos) * stride_s32 + lane_base;
                 vo_sc[j] = vo[j] >> 2;
             }
+            if (MASK) {
+#pragma unroll
+                for (int r = 0; r < 2; ++r) {
+                    const int t = pos + 4 * row_odd + t4 + 8 * r;
+                    mo[r] = mask_head + (uint32_t)((t < pe32 ? t : pe32 - 1) - pos) * 2;
+                }
+            }
         };
         // (the row loads carry the non-temporal hint unless a second set of waves reads the same lines)
-        auto request_k = [&](KBlock& kb, int pos) {
+        auto request_k = [&](KBlock& kb, uint32_t (&mk)[2], int pos) {
             kb.pos = pos;
             const int64_t boff = row_base_of(pos) * a.cache_stride_s;
             kb.boff = boff;
@@ -179,6 +199,10 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
             for (int j = 0; j < kTB; ++j) {
                 load_b128<GP == 1>(kb.q8[j], vo[j], bk);
                 load_b32<false>(kb.sc[j], vo_sc[j], sk);
+            }
+            if (MASK) {
+                load_u16(mk[0], mo[0], mask_base + (int64_t)pos * 2);
+                load_u16(mk[1], mo[1], mask_base + (int64_t)pos * 2);
             }
         };
         auto request_v = [&](VBlock& vb, int64_t boff) {
@@ -193,9 +217,10 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
 
         KBlock ka, kb;
         VBlock va, vb;
+        uint32_t mka[2] = {0, 0}, mkb[2] = {0, 0}; // the blocks' mask values (halves)
         int pos = pa32;
         if (nb == 1 && tail_partial) clamp_offsets(pos);
-        request_k(ka, pos);
+        request_k(ka, mka, pos);
         request_v(va, ka.boff);
 
         // ---- A operands: this lane supplies row t4 = query head t4, its chunk's 16 channels ----
@@ -233,14 +258,17 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
             for (int c = 0; c < 16; ++c) acc[s][c] = 0.f;
 
         float prob[4][kTB]; // [slot][step]: probabilities of this lane's own tokens
-        auto logits_softmax = [&](KBlock& kx, bool beyond_piece) { // beyond_piece: the block reaches past the piece (wave-uniform)
+        // loads in flight when a block's logits start: its own, the V block before it and the next K block;
+        // a K block has two more requests with the mask
+        constexpr int kMoreK = MASK ? 4 : 0, kMoreV = MASK ? 2 : 0;
+        auto logits_softmax = [&](KBlock& kx, uint32_t (&mk)[2], bool beyond_piece) { // beyond_piece: the block reaches past the piece (wave-uniform)
             float part[4][kTB]; // [head][step], over this lane's 16 channels, log2 units
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
-                if (j == 0) wait_loads<22>(kx.q8[0], kx.sc[0]);
-                if (j == 1) wait_loads<20>(kx.q8[1], kx.sc[1]);
-                if (j == 2) wait_loads<18>(kx.q8[2], kx.sc[2]);
-                if (j == 3) wait_loads<16>(kx.q8[3], kx.sc[3]);
+                if (j == 0) wait_loads<22 + kMoreK>(kx.q8[0], kx.sc[0]);
+                if (j == 1) wait_loads<20 + kMoreK>(kx.q8[1], kx.sc[1]);
+                if (j == 2) wait_loads<18 + kMoreK>(kx.q8[2], kx.sc[2]);
+                if (j == 3) wait_loads<16 + kMoreK>(kx.q8[3], kx.sc[3]);
                 f32x4 d0 = qbias0, d1 = qbias1;
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
@@ -270,6 +298,11 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
                 swap_rows(rb[2], rb[3]);
                 l0 = (rb[0] + rb[1]) * logit_scale;
                 l1 = (rb[2] + rb[3]) * logit_scale;
+            }
+            if (MASK) { // the block's two mask requests follow its eight cache requests
+                wait_loads<18>(mk[0], mk[1]);
+                l0 += (float)bitcast<half2_t>(mk[0]).x * kLog2e;
+                l1 += (float)bitcast<half2_t>(mk[1]).x * kLog2e;
             }
             if (beyond_piece) { // only the last block of a piece
                 const int tk = kx.pos + 4 * row_odd + t4;
@@ -314,10 +347,10 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
         auto accumulate_pv = [&](VBlock& vx) {
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
-                if (j == 0) wait_loads<22>(vx.q8[0], vx.sc[0]);
-                if (j == 1) wait_loads<20>(vx.q8[1], vx.sc[1]);
-                if (j == 2) wait_loads<18>(vx.q8[2], vx.sc[2]);
-                if (j == 3) wait_loads<16>(vx.q8[3], vx.sc[3]);
+                if (j == 0) wait_loads<22 + kMoreV>(vx.q8[0], vx.sc[0]);
+                if (j == 1) wait_loads<20 + kMoreV>(vx.q8[1], vx.sc[1]);
+                if (j == 2) wait_loads<18 + kMoreV>(vx.q8[2], vx.sc[2]);
+                if (j == 3) wait_loads<16 + kMoreV>(vx.q8[3], vx.sc[3]);
                 float x[16];
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
@@ -354,6 +387,7 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
         // block i, V of block i+1 before the PV of block i; the last block re-requests itself
         drain_loads(ka.q8, ka.sc);
         drain_loads(va.q8, va.sc);
+        if (MASK) wait_loads<0>(mka[0], mka[1]);
         for (int i = 0;;) {
             // With two sets of waves on the same kv heads, a barrier per pair of blocks keeps the sets within a
             // block of each other, so that the second set's requests find the lines in the cache levels
@@ -361,8 +395,8 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
             if (GP > 1) __syncthreads();
             int npos = pos + (i + 1 < nb ? kQuadBlock : 0);
             if (tail_partial && i + 2 == nb) clamp_offsets(npos);
-            request_k(kb, npos);
-            logits_softmax(ka, tail_partial && i + 1 == nb);
+            request_k(kb, mkb, npos);
+            logits_softmax(ka, mka, tail_partial && i + 1 == nb);
             request_v(vb, kb.boff);
             accumulate_pv(va);
             pin_acc();
@@ -370,8 +404,8 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
             if (++i == nb) break;
             npos = pos + (i + 1 < nb ? kQuadBlock : 0);
             if (tail_partial && i + 2 == nb) clamp_offsets(npos);
-            request_k(ka, npos);
-            logits_softmax(kb, tail_partial && i + 1 == nb);
+            request_k(ka, mka, npos);
+            logits_softmax(kb, mkb, tail_partial && i + 1 == nb);
             request_v(va, ka.boff);
             accumulate_pv(vb);
             pin_acc();
@@ -382,6 +416,10 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
         drain_loads(kb.q8, kb.sc);
         drain_loads(va.q8, va.sc);
         drain_loads(vb.q8, vb.sc);
+        if (MASK) {
+            wait_loads<0>(mka[0], mka[1]);
+            wait_loads<0>(mkb[0], mkb[1]);
+        }
 
         // ---- end of the piece: exp-sum of the head over the row pair, (max, sum) of the four slots,
         // then the four token streams of the quad are merged ----
@@ -465,11 +503,20 @@ bool decode_quad_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads
     return g <= 4 || (g <= 8 && num_kv_heads % 8 == 0);
 }
 
-// true when it serves the launch (no attn_mask); the caller falls back to the general kernel otherwise
+// attn_mask: one set of waves only, and the mask's byte offsets inside a sequence's rows (heads x mask_stride_h, plus
+// a block) fit 32 bits
+bool decode_quad_mask_ok(int64_t num_heads, int64_t num_kv_repeats, int64_t mask_stride_h)
+{
+    if (num_kv_repeats > 4 || mask_stride_h < 0) return false;
+    return ((double)num_heads * (double)mask_stride_h + 64.0) * 2.0 < 4294967296.0;
+}
+
+// true when it serves the launch; the caller falls back to the general kernel otherwise
 bool decode_quad_applicable(const DecodeLaunch& a)
 {
-    return decode_quad_shape(a.head_dim, a.num_heads, a.num_kv_heads) && a.attn_mask == nullptr &&
-           a.kv_heads_per_group == decode_quad_kv_heads(a.num_kv_heads) && a.num_passes == 1 && a.wg_tokens == kQuadBlock &&
+    if (!decode_quad_shape(a.head_dim, a.num_heads, a.num_kv_heads)) return false;
+    if (a.attn_mask != nullptr && !decode_quad_mask_ok(a.num_heads, a.num_kv_repeats, a.mask_stride_h)) return false;
+    return a.kv_heads_per_group == decode_quad_kv_heads(a.num_kv_heads) && a.num_passes == 1 && a.wg_tokens == kQuadBlock &&
            a.output_stride_s % 8 == 0 && (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0;
 }
 
@@ -477,17 +524,22 @@ template <int WP>
 static void launch_decode_quad_wp(const DecodeLaunch& a, hipStream_t stream)
 {
     const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / (2 * WP)), 1);
-    const bool paged = a.cache_mode == 1;
-    if (paged) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1, WP>), grid, dim3(kWave * WP), 0, stream, a);
-    else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1, WP>), grid, dim3(kWave * WP), 0, stream, a);
+    const bool paged = a.cache_mode == 1, mask = a.attn_mask != nullptr;
+    if (paged) {
+        if (mask) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1, WP, true>), grid, dim3(kWave * WP), 0, stream, a);
+        else hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1, WP, false>), grid, dim3(kWave * WP), 0, stream, a);
+    } else {
+        if (mask) hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1, WP, true>), grid, dim3(kWave * WP), 0, stream, a);
+        else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1, WP, false>), grid, dim3(kWave * WP), 0, stream, a);
+    }
 }
 
 void launch_decode_quad(const DecodeLaunch& a, hipStream_t stream)
 {
     if (a.num_kv_repeats > 4) { // two sets of four waves on eight kv heads
         const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / kQuadMaxHeads), 1);
-        if (a.cache_mode == 1) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 2, 4>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
-        else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 2, 4>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
+        if (a.cache_mode == 1) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 2, 4, false>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
+        else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 2, 4, false>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
         return;
     }
     switch (decode_quad_kv_heads(a.num_kv_heads)) {

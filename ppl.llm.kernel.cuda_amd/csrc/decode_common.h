@@ -47,6 +47,16 @@ __device__ __forceinline__ void wait_loads(u32x4& a, uint32_t& b)
 {
     asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
 }
+template <int N>
+__device__ __forceinline__ void wait_loads(uint32_t& a, uint32_t& b)
+{
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
+}
+// one half (an attn_mask value) per lane, zero-extended
+__device__ __forceinline__ void load_u16(uint32_t& dst, uint32_t lane_off, const char* wave_base)
+{
+    asm volatile("global_load_ushort %0, %1, %2" : "=&v"(dst) : "v"(lane_off), "s"(wave_base) : "memory");
+}
 // Waits for every outstanding load.  A register that is the target of an in-flight load must stay
 // allocated until a wait covers it, even when its value is never used (the redundant request of
 // the last block): passing it through this statement keeps it reserved, so that nothing else can

@@ -149,7 +149,8 @@ int decode_wg_tokens(int head_dim, int kv_heads_per_group);
 bool decode_general_forced(); // PMX_HIP_DECODE_GENERAL=1 in the environment: every shape on the general kernel
 bool decode_quad_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads); // head_dim 128, an even number of kv heads, <= 4 query heads each
 int decode_quad_kv_heads(int64_t num_kv_heads);                                    // kv heads per workgroup: 8, 4 or 2
-bool decode_quad_applicable(const DecodeLaunch& a);                                // the shape, and no attn_mask
+bool decode_quad_mask_ok(int64_t num_heads, int64_t num_kv_repeats, int64_t mask_stride_h); // attn_mask within its reach
+bool decode_quad_applicable(const DecodeLaunch& a);
 constexpr int kDecodeQuadTokens = 16;
 void launch_decode_quad(const DecodeLaunch& a, hipStream_t stream);
 // head_dim 128, 5 to 32 query heads per kv head, kv heads in fours: MFMA kernel, groups of four kv heads, 32-token blocks

@@ -138,7 +138,7 @@ def test_decode_gqa_identical_queries_and_mha_equivalence(pkg, oracle):
         assert np.array_equal(got[:, g], got[:, 0])
 
 
-@pytest.mark.parametrize("heads", [(8, 4), (32, 4), (96, 4)])
+@pytest.mark.parametrize("heads", [(8, 4), (32, 4), (96, 4), (8, 8), (32, 8), (6, 2), (2, 1), (24, 8)])
 def test_decode_with_mask(pkg, oracle, heads):
     bt, dev, q, cache, scale = make_case(pkg, oracle, 79, num_heads=heads[0], num_kv_heads=heads[1], head_dim=128,
                                          cache_mode=1, dec_kv_lens=[70, 300, 5])
