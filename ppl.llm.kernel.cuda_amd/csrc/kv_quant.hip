@@ -92,6 +92,10 @@ __global__ __launch_bounds__(kQuantThreads) void kv_quantize_kernel(const QuantL
         const int h = gi / groups_per_head;
         const int d0 = (gi - h * groups_per_head) << 3;
         const int64_t in_tok = first + tok;
+        // the rows to quantise do not depend on the sequence: requested first, they travel during the index lookups
+        const int64_t in_idx = (int64_t)h * a.head_dim + d0;
+        const u32x4 kraw = *(const u32x4*)((const half_t*)a.current_key + in_tok * a.current_key_stride_s + in_idx);
+        const u32x4 vraw = *(const u32x4*)((const half_t*)a.current_value + in_tok * a.current_value_stride_s + in_idx);
         // decode steps have one new token per sequence: token i then belongs to sequence i, which two independent
         // loads confirm; otherwise the sequence is found by bisection (a chain of dependent loads)
         int b;
@@ -100,9 +104,6 @@ __global__ __launch_bounds__(kQuantThreads) void kv_quantize_kernel(const QuantL
         const int64_t pos = a.start_pos[b] + (in_tok - a.seqstarts[b]);
         const int64_t row = token_row<PAGED>(a.cachestarts, PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b, pos);
 
-        const int64_t in_idx = (int64_t)h * a.head_dim + d0;
-        const u32x4 kraw = *(const u32x4*)((const half_t*)a.current_key + in_tok * a.current_key_stride_s + in_idx);
-        const u32x4 vraw = *(const u32x4*)((const half_t*)a.current_value + in_tok * a.current_value_stride_s + in_idx);
         const Quantised kq = quantise_group(kraw);
         const Quantised vq = quantise_group(vraw);
 
