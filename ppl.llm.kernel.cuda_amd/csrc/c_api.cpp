@@ -173,7 +173,7 @@ int pmxhip_decode_plan_make(int64_t decoding_batches, int64_t num_heads, int64_t
         // workgroups that a CU holds at once: two of four waves, or as many as eight waves make where a kernel with
         // smaller workgroups serves the shape (a wave per kv head, or per two)
         const bool quad = !mfma && pmxhip::decode_quad_shape(head_dim, num_heads, num_kv_heads);
-        const int wgs_per_cu = mfma ? pmxhip::kDecodeMfmaWavesPerCu / kvhb : (quad ? 16 / kvhb : 2);
+        const int wgs_per_cu = mfma ? pmxhip::kDecodeMfmaWavesPerCu / kvhb : (quad ? (head_dim == 256 ? 8 : 16) / kvhb : 2);
         ranges = ((int64_t)cus * wgs_per_cu + groups - 1) / groups;
         const int64_t max_tokens = decoding_batches * (max_kvlen > 0 ? max_kvlen : 1);
         const int64_t useful = (max_tokens + min_tokens - 1) / min_tokens;

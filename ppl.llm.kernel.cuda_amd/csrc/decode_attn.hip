@@ -695,7 +695,7 @@ static int launch_decode_d(const DecodeLaunch& a, int stage, hipStream_t stream)
     const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / a.kv_heads_per_group), (unsigned)a.num_passes);
     if (stage != 2 && D == 128 && decode_mfma_applicable(a) && !decode_general_forced()) {
         launch_decode_mfma(a, stream);
-    } else if (stage != 2 && D == 128 && decode_quad_applicable(a) && !decode_general_forced()) {
+    } else if (stage != 2 && (D == 128 || D == 256) && decode_quad_applicable(a) && !decode_general_forced()) {
         launch_decode_quad(a, stream);
     } else if (stage != 2) {
         switch (a.q_heads_per_pass) {

@@ -1,5 +1,6 @@
-// Decode attention over the int8 group-8 KV cache, variant for head_dim 128, up to eight query
-// heads per kv head and kv heads in multiples of eight (MHA and the common GQA shapes).  Same semantics, token ranges, pieces and workspace as decode_attn.hip
+// Decode attention over the int8 group-8 KV cache, variant for head_dim 128 (an even number of kv heads)
+// and 256, up to four query heads per kv head (MHA and the common GQA shapes; up to eight at head_dim 128
+// with kv heads in eights).  Same semantics, token ranges, pieces and workspace as decode_attn.hip
 // (reference: src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/kernel.cu:229-679,
 // 1115-1891); what differs is the lane layout, chosen so that the matrix pipe computes
 // the q.k products while the vector pipe converts and accumulates:
@@ -76,6 +77,12 @@ __device__ __forceinline__ float fold_xor8(float lo, float hi)
         : "v"(lo), "v"(hi));
     return r;
 }
+// v + v(lane ^ 32): the swap hands every lane the value of its own lane in the lower and in the upper half-wave
+__device__ __forceinline__ float sum_halves(float v)
+{
+    const u32x2_t r = __builtin_amdgcn_permlane32_swap(bitcast<uint32_t>(v), bitcast<uint32_t>(v), false, false);
+    return bitcast<float>(r[0]) + bitcast<float>(r[1]);
+}
 // value held by quad lane i (compile-time i)
 template <int I>
 __device__ __forceinline__ float quad_lane(float v)
@@ -87,10 +94,13 @@ __device__ __forceinline__ float quad_lane(float v)
 
 // GP: sets of four query heads per kv head (1 or 2); WP: pairs of kv heads per workgroup (4, 2 or 1); the workgroup
 // has WP * GP waves.  MASK: the additive attn_mask (kernel.cu:319-325), two more requests per block and lane.
-template <bool PAGED, int GP, int WP, bool MASK>
+// HD: head_dim 128, or 256: the two half-waves then hold the two halves of ONE kv head's channels instead of two kv
+// heads, and a logit is the sum of the two half-waves' sums.
+template <bool PAGED, int GP, int WP, bool MASK, int HD>
 __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kernel(const DecodeLaunch a)
 {
-    constexpr int D = kQuadD;
+    constexpr int D = HD;
+    constexpr int KPW = HD == 256 ? 1 : 2; // kv heads per wave
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -98,12 +108,13 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
     const int g_first = (wave_id / WP) * 4; // first query head (within the kv head's group) of this wave
     const int t4 = lane & 3;           // token within a step
     const int chunk = (lane >> 2) & 7; // channels [16 chunk, 16 chunk + 16)
-    const int hsel = lane >> 5;        // which of the wave's two kv heads
+    const int hsel = lane >> 5;        // which of the wave's two kv heads (head_dim 256: which half of the channels)
     // the head whose complete logits this lane receives from the reduce-scatter
     const int g_own = (((lane >> 2) & 1) << 1) | ((lane >> 3) & 1);
     const int row_odd = (lane >> 4) & 1;
     const int G = (int)a.num_kv_repeats; // <= 4 * GP
-    const int kvh = blockIdx.y * (2 * WP) + wave * 2 + hsel;
+    const int kvh = blockIdx.y * (KPW * WP) + wave * KPW + (KPW == 2 ? hsel : 0);
+    const int ch0 = chunk * 16 + (KPW == 1 ? hsel * 128 : 0); // this lane's 16 channels
 
     const const_i64_ptr kvstarts = as_constant(a.kvstarts);
     const const_i64_ptr cachestarts = as_constant(a.cachestarts);
@@ -114,9 +125,9 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
     if (r0 >= total) return;
     const int64_t r1 = (r0 + per < total) ? r0 + per : total;
 
-    const int64_t group_off = a.layer_idx * a.cache_stride_l + (int64_t)(blockIdx.y * (2 * WP)) * a.cache_stride_h;
+    const int64_t group_off = a.layer_idx * a.cache_stride_l + (int64_t)(blockIdx.y * (KPW * WP)) * a.cache_stride_h;
     const uint32_t stride_s32 = (uint32_t)a.cache_stride_s; // the host checks that a block's span fits 32 bits
-    const uint32_t lane_base = (uint32_t)((int64_t)(wave * 2 + hsel) * a.cache_stride_h + chunk * 16);
+    const uint32_t lane_base = (uint32_t)((int64_t)(wave * KPW + (KPW == 2 ? hsel : 0)) * a.cache_stride_h + ch0);
     const char* const cache_k = (const char*)a.cache + group_off;
     const char* const cache_v = cache_k + a.cache_stride_kv;
     const char* const scale_k = (const char*)a.scale + (group_off >> 3) * 2;
@@ -229,7 +240,7 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
         {
             const bool on = g_first + t4 < G;
             const int h = kvh * G + (on ? g_first + t4 : 0);
-            const u32x4* qp = (const u32x4*)((const half_t*)a.query + (int64_t)b * a.query_stride_s + (int64_t)h * D + chunk * 16);
+            const u32x4* qp = (const u32x4*)((const half_t*)a.query + (int64_t)b * a.query_stride_s + (int64_t)h * D + ch0);
             u32x4 lo = qp[0], hi = qp[1];
             if (!on) { lo = u32x4{0, 0, 0, 0}; hi = lo; }
             qa[0] = bitcast<half4_t>(u32x2_t{lo[0], lo[1]});
@@ -296,8 +307,14 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
                 }
                 swap_rows(rb[0], rb[1]);
                 swap_rows(rb[2], rb[3]);
-                l0 = (rb[0] + rb[1]) * logit_scale;
-                l1 = (rb[2] + rb[3]) * logit_scale;
+                l0 = rb[0] + rb[1];
+                l1 = rb[2] + rb[3];
+                if (KPW == 1) { // the other half of the channels
+                    l0 = sum_halves(l0);
+                    l1 = sum_halves(l1);
+                }
+                l0 *= logit_scale;
+                l1 *= logit_scale;
             }
             if (MASK) { // the block's two mask requests follow its eight cache requests
                 wait_loads<18>(mk[0], mk[1]);
@@ -462,7 +479,7 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
                 const int h = kvh * G + g;
                 if (whole) {
                     typedef half_t half8_t __attribute__((ext_vector_type(8)));
-                    half_t* out = (half_t*)a.output + (int64_t)b * a.output_stride_s + (int64_t)h * D + chunk * 16;
+                    half_t* out = (half_t*)a.output + (int64_t)b * a.output_stride_s + (int64_t)h * D + ch0;
                     half8_t v0, v1;
 #pragma unroll
                     for (int c = 0; c < 8; ++c) {
@@ -472,7 +489,7 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
                     *(half8_t*)out = v0;
                     *(half8_t*)(out + 8) = v1;
                 } else {
-                    float* out = a.partial_out + (piece * a.num_heads + h) * D + chunk * 16;
+                    float* out = a.partial_out + (piece * a.num_heads + h) * D + ch0;
 #pragma unroll
                     for (int c = 0; c < 16; c += 4) *(f32x4*)(out + c) = f32x4{o[c], o[c + 1], o[c + 2], o[c + 3]};
                     if (chunk == 0) {
@@ -485,21 +502,26 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
     }
 }
 
-// kv heads per workgroup for a shape that this kernel serves
-int decode_quad_kv_heads(int64_t num_kv_heads)
+// kv heads per workgroup for a shape that this kernel serves (a wave holds two kv heads of 128 channels, one of 256)
+int decode_quad_kv_heads(int64_t head_dim, int64_t num_kv_heads)
 {
-    return num_kv_heads % 8 == 0 ? 8 : (num_kv_heads % 4 == 0 ? 4 : 2);
+    const int per_wave = head_dim == 256 ? 1 : 2;
+    const int64_t pairs = num_kv_heads / per_wave;
+    return per_wave * (pairs % 4 == 0 ? 4 : (pairs % 2 == 0 ? 2 : 1));
 }
 
-// true when the variant above serves the shape: head_dim 128, an even number of kv heads, up to four query heads
-// per kv head (up to eight with kv heads in eights; decode_attn_mfma.hip takes five and more first).
+// true when the variant above serves the shape: head_dim 128 with an even number of kv heads or head_dim 256, up to
+// four query heads per kv head (head_dim 128: up to eight with kv heads in eights; decode_attn_mfma.hip takes five and
+// more first).
 // One or two query heads per kv head leave rows of the 4x4x4 products and three quarters or half of the PV
 // arithmetic unused, but this kernel's row loads take the non-temporal hint, which the general kernel's cannot.
 bool decode_quad_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads)
 {
     if (decode_general_forced()) return false;
-    if (head_dim != kQuadD || num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || num_kv_heads % 2 != 0) return false;
+    if (num_kv_heads <= 0 || num_heads % num_kv_heads != 0) return false;
     const int64_t g = num_heads / num_kv_heads;
+    if (head_dim == 256) return g <= 4;
+    if (head_dim != kQuadD || num_kv_heads % 2 != 0) return false;
     return g <= 4 || (g <= 8 && num_kv_heads % 8 == 0);
 }
 
@@ -516,21 +538,22 @@ bool decode_quad_applicable(const DecodeLaunch& a)
 {
     if (!decode_quad_shape(a.head_dim, a.num_heads, a.num_kv_heads)) return false;
     if (a.attn_mask != nullptr && !decode_quad_mask_ok(a.num_heads, a.num_kv_repeats, a.mask_stride_h)) return false;
-    return a.kv_heads_per_group == decode_quad_kv_heads(a.num_kv_heads) && a.num_passes == 1 && a.wg_tokens == kQuadBlock &&
-           a.output_stride_s % 8 == 0 && (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0;
+    return a.kv_heads_per_group == decode_quad_kv_heads(a.head_dim, a.num_kv_heads) && a.num_passes == 1 &&
+           a.wg_tokens == kQuadBlock && a.output_stride_s % 8 == 0 && (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0;
 }
 
-template <int WP>
+template <int WP, int HD>
 static void launch_decode_quad_wp(const DecodeLaunch& a, hipStream_t stream)
 {
-    const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / (2 * WP)), 1);
+    constexpr int KPW = HD == 256 ? 1 : 2;
+    const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / (KPW * WP)), 1);
     const bool paged = a.cache_mode == 1, mask = a.attn_mask != nullptr;
     if (paged) {
-        if (mask) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1, WP, true>), grid, dim3(kWave * WP), 0, stream, a);
-        else hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1, WP, false>), grid, dim3(kWave * WP), 0, stream, a);
+        if (mask) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1, WP, true, HD>), grid, dim3(kWave * WP), 0, stream, a);
+        else hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1, WP, false, HD>), grid, dim3(kWave * WP), 0, stream, a);
     } else {
-        if (mask) hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1, WP, true>), grid, dim3(kWave * WP), 0, stream, a);
-        else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1, WP, false>), grid, dim3(kWave * WP), 0, stream, a);
+        if (mask) hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1, WP, true, HD>), grid, dim3(kWave * WP), 0, stream, a);
+        else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1, WP, false, HD>), grid, dim3(kWave * WP), 0, stream, a);
     }
 }
 
@@ -538,14 +561,23 @@ void launch_decode_quad(const DecodeLaunch& a, hipStream_t stream)
 {
     if (a.num_kv_repeats > 4) { // two sets of four waves on eight kv heads
         const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / kQuadMaxHeads), 1);
-        if (a.cache_mode == 1) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 2, 4, false>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
-        else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 2, 4, false>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
+        if (a.cache_mode == 1) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 2, 4, false, 128>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
+        else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 2, 4, false, 128>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
         return;
     }
-    switch (decode_quad_kv_heads(a.num_kv_heads)) {
-    case 8: launch_decode_quad_wp<4>(a, stream); break;
-    case 4: launch_decode_quad_wp<2>(a, stream); break;
-    default: launch_decode_quad_wp<1>(a, stream); break;
+    const int waves = decode_quad_kv_heads(a.head_dim, a.num_kv_heads) / (a.head_dim == 256 ? 1 : 2);
+    if (a.head_dim == 256) {
+        switch (waves) {
+        case 4: launch_decode_quad_wp<4, 256>(a, stream); break;
+        case 2: launch_decode_quad_wp<2, 256>(a, stream); break;
+        default: launch_decode_quad_wp<1, 256>(a, stream); break;
+        }
+    } else {
+        switch (waves) {
+        case 4: launch_decode_quad_wp<4, 128>(a, stream); break;
+        case 2: launch_decode_quad_wp<2, 128>(a, stream); break;
+        default: launch_decode_quad_wp<1, 128>(a, stream); break;
+        }
     }
 }
 

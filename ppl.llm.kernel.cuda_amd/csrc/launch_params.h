@@ -147,8 +147,8 @@ void launch_page_copy(const PageCopyLaunch& a, hipStream_t stream);
 int launch_decode(const DecodeLaunch& a, int stage, hipStream_t stream); // stage: 0 both, 1 ranges, 2 combine
 int decode_wg_tokens(int head_dim, int kv_heads_per_group);
 bool decode_general_forced(); // PMX_HIP_DECODE_GENERAL=1 in the environment: every shape on the general kernel
-bool decode_quad_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads); // head_dim 128, an even number of kv heads, <= 4 query heads each
-int decode_quad_kv_heads(int64_t num_kv_heads);                                    // kv heads per workgroup: 8, 4 or 2
+bool decode_quad_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads); // head_dim 128 (even number of kv heads) or 256, <= 4 query heads each
+int decode_quad_kv_heads(int64_t head_dim, int64_t num_kv_heads);                  // kv heads per workgroup: 8, 4 or 2 (head_dim 256: 4, 2 or 1)
 bool decode_quad_mask_ok(int64_t num_heads, int64_t num_kv_repeats, int64_t mask_stride_h); // attn_mask within its reach
 bool decode_quad_applicable(const DecodeLaunch& a);
 constexpr int kDecodeQuadTokens = 16;

@@ -42,6 +42,8 @@ SHAPES = [
     (8, 1, 128), (4, 1, 128), (40, 2, 128), (24, 1, 128), (12, 4, 128),
     # the quad kernel with four and two kv heads per workgroup
     (8, 2, 128), (6, 6, 128), (24, 12, 128), (16, 4, 128),
+    # ... and with head_dim 256 (a wave per kv head)
+    (16, 8, 256), (16, 16, 256), (3, 1, 256), (8, 2, 256), (5, 1, 256),
 ]
 
 
@@ -138,9 +140,10 @@ def test_decode_gqa_identical_queries_and_mha_equivalence(pkg, oracle):
         assert np.array_equal(got[:, g], got[:, 0])
 
 
-@pytest.mark.parametrize("heads", [(8, 4), (32, 4), (96, 4), (8, 8), (32, 8), (6, 2), (2, 1), (24, 8)])
+@pytest.mark.parametrize("heads", [(8, 4), (32, 4), (96, 4), (8, 8), (32, 8), (6, 2), (2, 1), (24, 8), (8, 4, 256), (2, 1, 256)])
 def test_decode_with_mask(pkg, oracle, heads):
-    bt, dev, q, cache, scale = make_case(pkg, oracle, 79, num_heads=heads[0], num_kv_heads=heads[1], head_dim=128,
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 79, num_heads=heads[0], num_kv_heads=heads[1],
+                                         head_dim=heads[2] if len(heads) > 2 else 128,
                                          cache_mode=1, dec_kv_lens=[70, 300, 5])
     total = int(bt.kvstarts[-1])
     width = (total + 7) // 8 * 8
