@@ -341,7 +341,17 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         row_next = tile_row(2);
         __syncthreads();
     }
+    // tokens this wave's columns attend to: beyond them (a tile past its columns' limits, or a wave whose columns lie
+    // beyond the query rows: short chunks leave most waves without any) the wave only helps to stage the tiles
+    int wave_lim = lim;
+#pragma unroll
+    for (int sh = 32; sh >= 1; sh >>= 1) {
+        const int o = __shfl_xor(wave_lim, sh);
+        wave_lim = o > wave_lim ? o : wave_lim;
+    }
+    wave_lim = __builtin_amdgcn_readfirstlane(wave_lim);
     for (int tile = 0; tile < n_tiles; ++tile) {
+        const bool work = tile * kBN < wave_lim;
         const half_t* const sK = smem + (tile & 1) * TILE_HALVES;
         const half_t* const sKlo = sK + kBN * K_STRIDE;
         const half_t* const sV = KV16 ? sKlo : sKlo + kBN * K_STRIDE;
@@ -355,7 +365,7 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) s_acc[mb][i] = 0.f;
-        {
+        if (work) {
             constexpr int QB = 4;
             constexpr int PER_MB = KSTEPS / QB;
             constexpr int NBATCH = 2 * PER_MB;
@@ -386,6 +396,9 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
                 for (int k = 0; k < N_SLICES; ++k)
                     if (bi == k * NBATCH / N_SLICES) store_slice((tile & 1) ^ 1, k);
             }
+        } else {
+#pragma unroll
+            for (int k = 0; k < N_SLICES; ++k) store_slice((tile & 1) ^ 1, k);
         }
 
         // ---- then the raw bytes of tile + 2 ----
@@ -394,99 +407,101 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
             row_next = tile_row(tile + 3);
         }
 
-        // ---- online softmax per column (element i <-> token 32 mb + 8 (i/4) + 4 hh + i%4) ----
-        const int t_base = tile * kBN;
-        // only the tiles that reach beyond a column's limit need the per-element test (wave-uniform branch)
-        const bool need_mask = __builtin_amdgcn_ballot_w64(t_base + kBN > lim) != 0;
-        float mx = kNegBig;
-        if (EXTRA) {
-            // additive terms per element (log2 units): mask value and alibi distance of (query row, token)
-#pragma unroll
-            for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int t = t_base + 32 * mb + 8 * (i >> 2) + 4 * hh + (i & 3);
-                    float v = -INFINITY;
-                    if (t < lim) {
-                        float add = 0.f;
-                        if (mask_row) add = (float)mask_row[t];
-                        if (a.alibi_slopes) add += a.is_causal ? slope * (float)t : -slope * fabsf((float)(pos_c + kvlen - qlen - t));
-                        v = __builtin_fmaf(s_acc[mb][i], sm_scale, add * kLog2e);
-                    }
-                    s_acc[mb][i] = v;
-                    mx = fmaxf(mx, v);
-                }
-        } else {
-            // maximum of the raw dot products; the (positive) logit scale is applied to it afterwards
-            if (need_mask) {
+        if (work) {
+            // ---- online softmax per column (element i <-> token 32 mb + 8 (i/4) + 4 hh + i%4) ----
+            const int t_base = tile * kBN;
+            // only the tiles that reach beyond a column's limit need the per-element test (wave-uniform branch)
+            const bool need_mask = __builtin_amdgcn_ballot_w64(t_base + kBN > lim) != 0;
+            float mx = kNegBig;
+            if (EXTRA) {
+                // additive terms per element (log2 units): mask value and alibi distance of (query row, token)
 #pragma unroll
                 for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
                         const int t = t_base + 32 * mb + 8 * (i >> 2) + 4 * hh + (i & 3);
-                        if (t >= lim) s_acc[mb][i] = -INFINITY;
+                        float v = -INFINITY;
+                        if (t < lim) {
+                            float add = 0.f;
+                            if (mask_row) add = (float)mask_row[t];
+                            if (a.alibi_slopes) add += a.is_causal ? slope * (float)t : -slope * fabsf((float)(pos_c + kvlen - qlen - t));
+                            v = __builtin_fmaf(s_acc[mb][i], sm_scale, add * kLog2e);
+                        }
+                        s_acc[mb][i] = v;
+                        mx = fmaxf(mx, v);
                     }
+            } else {
+                // maximum of the raw dot products; the (positive) logit scale is applied to it afterwards
+                if (need_mask) {
+#pragma unroll
+                    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) {
+                            const int t = t_base + 32 * mb + 8 * (i >> 2) + 4 * hh + (i & 3);
+                            if (t >= lim) s_acc[mb][i] = -INFINITY;
+                        }
+                }
+#pragma unroll
+                for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[mb][i]);
+                mx *= sm_scale;
             }
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_run, mx);
+            // the running max moves rarely once a few tiles have been seen: rescale only then (wave-uniform)
+            if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                l_run *= alpha;
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) o_acc[cb][i] *= alpha;
+                m_run = m_new;
+            }
+            const float bias = kPShift - m_run;
+            // p = hi + lo in halves: hi = p rounded toward zero (two at a time), lo = the exact remainder
+            f16x8 pf[2][2], pfl[2][2];
+            float lsum = 0.f;
 #pragma unroll
             for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[mb][i]);
-            mx *= sm_scale;
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);
-        // the running max moves rarely once a few tiles have been seen: rescale only then (wave-uniform)
-        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-            l_run *= alpha;
-#pragma unroll
-            for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) o_acc[cb][i] *= alpha;
-            m_run = m_new;
-        }
-        const float bias = kPShift - m_run;
-        // p = hi + lo in halves: hi = p rounded toward zero (two at a time), lo = the exact remainder
-        f16x8 pf[2][2], pfl[2][2];
-        float lsum = 0.f;
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-            for (int i = 0; i < 16; i += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(EXTRA ? s_acc[mb][i] + bias : __builtin_fmaf(s_acc[mb][i], sm_scale, bias));
-                const float p1 = __builtin_amdgcn_exp2f(EXTRA ? s_acc[mb][i + 1] + bias : __builtin_fmaf(s_acc[mb][i + 1], sm_scale, bias));
-                lsum += p0 + p1;
-                const half2_t ph = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(p0, p1));
-                const half2_t pl = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(sub_half_lo(p0, ph), sub_half_hi(p1, ph)));
-                pf[mb][i >> 3][i & 7] = ph.x;
-                pf[mb][i >> 3][(i & 7) + 1] = ph.y;
-                pfl[mb][i >> 3][i & 7] = pl.x;
-                pfl[mb][i >> 3][(i & 7) + 1] = pl.y;
-            }
-        l_run += lsum;
-
-        // ---- O^T += V^T P^T : fragment batches of one (32-token block, 16-token step) each, read one ahead ----
-        {
-            f16x8 vh[2][CB], vl[2][CB];
-            auto read_batch = [&](int bi, f16x8* ph, f16x8* pl) {
-                const int mb = bi >> 1, t = bi & 1;
-#pragma unroll
-                for (int cb = 0; cb < CB; ++cb) {
-                    ph[cb] = *(const f16x8*)&sV[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
-                    if (!KV16) pl[cb] = *(const f16x8*)&sVlo[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
+                for (int i = 0; i < 16; i += 2) {
+                    const float p0 = __builtin_amdgcn_exp2f(EXTRA ? s_acc[mb][i] + bias : __builtin_fmaf(s_acc[mb][i], sm_scale, bias));
+                    const float p1 = __builtin_amdgcn_exp2f(EXTRA ? s_acc[mb][i + 1] + bias : __builtin_fmaf(s_acc[mb][i + 1], sm_scale, bias));
+                    lsum += p0 + p1;
+                    const half2_t ph = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(p0, p1));
+                    const half2_t pl = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(sub_half_lo(p0, ph), sub_half_hi(p1, ph)));
+                    pf[mb][i >> 3][i & 7] = ph.x;
+                    pf[mb][i >> 3][(i & 7) + 1] = ph.y;
+                    pfl[mb][i >> 3][i & 7] = pl.x;
+                    pfl[mb][i >> 3][(i & 7) + 1] = pl.y;
                 }
-            };
-            read_batch(0, vh[0], vl[0]);
+            l_run += lsum;
+
+            // ---- O^T += V^T P^T : fragment batches of one (32-token block, 16-token step) each, read one ahead ----
+            {
+                f16x8 vh[2][CB], vl[2][CB];
+                auto read_batch = [&](int bi, f16x8* ph, f16x8* pl) {
+                    const int mb = bi >> 1, t = bi & 1;
 #pragma unroll
-            for (int bi = 0; bi < 4; ++bi) {
-                if (bi + 1 < 4) read_batch(bi + 1, vh[(bi + 1) & 1], vl[(bi + 1) & 1]);
-                __builtin_amdgcn_sched_barrier(0);
-                const int mb = bi >> 1, t = bi & 1;
+                    for (int cb = 0; cb < CB; ++cb) {
+                        ph[cb] = *(const f16x8*)&sV[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
+                        if (!KV16) pl[cb] = *(const f16x8*)&sVlo[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
+                    }
+                };
+                read_batch(0, vh[0], vl[0]);
 #pragma unroll
-                for (int cb = 0; cb < CB; ++cb) {
-                    if (!KV16) o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vl[bi & 1][cb], pf[mb][t], o_acc[cb], 0, 0, 0);
-                    o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vh[bi & 1][cb], pfl[mb][t], o_acc[cb], 0, 0, 0);
-                    o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vh[bi & 1][cb], pf[mb][t], o_acc[cb], 0, 0, 0);
+                for (int bi = 0; bi < 4; ++bi) {
+                    if (bi + 1 < 4) read_batch(bi + 1, vh[(bi + 1) & 1], vl[(bi + 1) & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    const int mb = bi >> 1, t = bi & 1;
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb) {
+                        if (!KV16) o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vl[bi & 1][cb], pf[mb][t], o_acc[cb], 0, 0, 0);
+                        o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vh[bi & 1][cb], pfl[mb][t], o_acc[cb], 0, 0, 0);
+                        o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vh[bi & 1][cb], pf[mb][t], o_acc[cb], 0, 0, 0);
+                    }
                 }
             }
         }
