@@ -51,6 +51,19 @@ def test_prefill_matches_oracle(pkg, oracle, shape, cache_mode):
     assert_attention_close(got[n_dec:], ref[n_dec:], "prefill %s mode %d" % (shape, cache_mode))
 
 
+@pytest.mark.parametrize("shape", [(32, 8, 128), (8, 1, 128), (8, 8, 64), (64, 8, 128)])
+def test_prefill_short_chunks_over_long_histories(pkg, oracle, shape):
+    """A few query tokens per sequence over many kv tiles: most waves of a workgroup have no live column."""
+    hq, hkv, d = shape
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 340 + hq + d, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                         cache_mode=1, dec_kv_lens=[],
+                                         prefill_q_lens=[2, 4, 8, 16, 3, 1], prefill_prior=[1500, 700, 900, 33, 2047, 640],
+                                         outliers=True)
+    ref = oracle_prefill(oracle, bt, q, cache, scale)
+    got = run_prefill(pkg, dev)
+    assert_attention_close(got, ref, "short chunks %s" % (shape,))
+
+
 def test_prefill_non_causal_and_single_row_equals_decode(pkg, oracle):
     bt, dev, q, cache, scale = make_case(pkg, oracle, 320, num_heads=8, num_kv_heads=2, head_dim=128, cache_mode=1,
                                          dec_kv_lens=[], prefill_q_lens=[1, 65], prefill_prior=[300, 10],
