@@ -6,10 +6,11 @@
 //   absmax over the group in half; scale = half(float(absmax) / 127.0f);
 //   scale = scale > eps ? scale : eps with eps = half(1e-5f) (a half subnormal);
 //   q = (int8) round-half-even( half(x / scale) ).
-// The half quotient is formed as the correctly rounded binary32 quotient rounded
-// once more to binary16, which equals the correctly rounded half quotient
-// (24 >= 2*11 + 2), and the integer rounding is v_rndne -- HIP's __half2short_rn
-// truncates, so it is not used.
+// The half quotient is the correctly rounded binary32 quotient rounded once more to
+// binary16, which equals the correctly rounded half quotient (24 >= 2*11 + 2); the
+// binary32 quotient comes from one division per group (the reciprocal of the scale) and
+// a residual correction per element, see quantise_group.  The integer rounding is
+// v_rndne -- HIP's __half2short_rn truncates, so it is not used.
 //
 // Decomposition (this file's own): a flat grid over (new token, group of 8
 // channels); one lane owns one group of K and the same group of V: two 128-bit
@@ -49,10 +50,17 @@ __device__ __forceinline__ Quantised quantise_group(const u32x4 raw)
     half_t s = (half_t)((float)amax / 127.0f);
     s = s > eps ? s : eps;
     const float sf = (float)s;
+    // One correctly rounded reciprocal per group, then a residual step per element:
+    //   q0 = x * rcp, e = fma(-q0, sf, x), quotient = fma(e, rcp, q0).
+    // Rounded to half this equals the correctly rounded quotient for every pair of a finite half x and a half
+    // scale >= eps (all 2.0e9 pairs compared on the CPU; the one difference, -0 / s -> +0, yields the same int8 0).
+    const float rcp = 1.0f / sf;
     uint32_t packed[2] = {0u, 0u};
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const half_t quo = (half_t)((float)x[i] / sf);
+        const float xf = (float)x[i];
+        const float q0 = xf * rcp;
+        const half_t quo = (half_t)__builtin_fmaf(__builtin_fmaf(-q0, sf, xf), rcp, q0);
         const int qi = (int)__builtin_rintf((float)quo);
         packed[i >> 2] |= ((uint32_t)qi & 0xffu) << (8 * (i & 3));
     }
@@ -98,10 +106,19 @@ __global__ __launch_bounds__(kQuantThreads) void kv_quantize_kernel(const QuantL
         const u32x4 vraw = *(const u32x4*)((const half_t*)a.current_value + in_tok * a.current_value_stride_s + in_idx);
         // decode steps have one new token per sequence: token i then belongs to sequence i, which two independent
         // loads confirm; otherwise the sequence is found by bisection (a chain of dependent loads)
+        // (the sequence's start_pos is requested together with them, so that the decode step's chain of dependent
+        // loads is index arrays -> page table -> stores)
         int b;
-        if (tok < a.batch && a.seqstarts[tok] == in_tok && a.seqstarts[tok + 1] > in_tok) b = (int)tok;
-        else b = sequence_of(a.seqstarts, (int)a.batch, in_tok);
-        const int64_t pos = a.start_pos[b] + (in_tok - a.seqstarts[b]);
+        int64_t pos;
+        const int64_t ti = tok < a.batch ? tok : 0;
+        const int64_t s0 = a.seqstarts[ti], s1 = a.seqstarts[ti + 1], sp = a.start_pos[ti];
+        if (tok < a.batch && s0 == in_tok && s1 > in_tok) {
+            b = (int)tok;
+            pos = sp;
+        } else {
+            b = sequence_of(a.seqstarts, (int)a.batch, in_tok);
+            pos = a.start_pos[b] + (in_tok - a.seqstarts[b]);
+        }
         const int64_t row = token_row<PAGED>(a.cachestarts, PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b, pos);
 
         const Quantised kq = quantise_group(kraw);
