@@ -62,6 +62,8 @@ def lib():
         _lib.pmx_oracle_splitkv_combine.restype = ctypes.c_int
         _lib.pmx_oracle_splitkv_combine.argtypes = [_vp] * 3 + [_i64, _i64, _vp]
         _lib.pmx_oracle_num_threads.restype = ctypes.c_int
+        _lib.pmx_oracle_count_reciprocal_quotient_mismatches.restype = ctypes.c_int64
+        _lib.pmx_oracle_count_reciprocal_quotient_mismatches.argtypes = [_vp]
         _lib.pmx_oracle_rotary_position_embedding.restype = ctypes.c_int
         _lib.pmx_oracle_rotary_position_embedding.argtypes = (
             [_vp] * 4 + [_f32, _i32] + [_i64] * 6 + [_i32, _f32] + [_i64] * 4 + [_vp] * 2)
@@ -253,6 +255,14 @@ def splitkv_combine(partial_out, partial_max, partial_sum):
     out = np.zeros(d, dtype=np.float32)
     lib().pmx_oracle_splitkv_combine(_p(partial_out), _p(partial_max), _p(partial_sum), n, d, _p(out))
     return out
+
+
+def count_reciprocal_quotient_mismatches():
+    """(pairs whose int8 results differ, pairs whose half quotients differ in bits) over every
+    finite half numerator and every half scale >= eps."""
+    half_differs = ctypes.c_int64(0)
+    bad = lib().pmx_oracle_count_reciprocal_quotient_mismatches(ctypes.byref(half_differs))
+    return int(bad), int(half_differs.value)
 
 
 def num_threads():

@@ -527,6 +527,37 @@ int pmx_oracle_splitkv_combine(
     return 0;
 }
 
+/* Quotient identity that a quantiser may use instead of one division per channel (not from the
+ * reference; a property of the arithmetic above that tests check): with rcp = 1.0f / s,
+ * q0 = x * rcp, e = fmaf(-q0, s, x), quo = fmaf(e, rcp, q0), the int8 result
+ * rint_even(half(quo)) equals rint_even(half(x / s)).  Compared here for EVERY finite half x and
+ * every half scale s >= eps (2.0e9 pairs); returns the number of pairs whose int8 results differ
+ * and, through *half_differs, the number whose half quotients differ in bits (-0 / s gives +0). */
+int64_t pmx_oracle_count_reciprocal_quotient_mismatches(int64_t* half_differs)
+{
+    const int eps_bits = pmx_oracle_float_to_half(1e-5f);
+    int64_t bad_q = 0, bad_h = 0;
+#pragma omp parallel for reduction(+ : bad_q, bad_h) schedule(dynamic, 64)
+    for (int sb = eps_bits; sb < 0x7C00; ++sb) {
+        const float s = pmx_oracle_half_to_float((uint16_t)sb);
+        const float rcp = 1.0f / s;
+        for (int xb = 0; xb < 0x10000; ++xb) {
+            if ((xb & 0x7C00) == 0x7C00) continue; /* inf, nan */
+            const float x = pmx_oracle_half_to_float((uint16_t)xb);
+            const uint16_t a = pmx_oracle_float_to_half(x / s);
+            const float q0 = x * rcp;
+            const uint16_t b = pmx_oracle_float_to_half(fmaf(fmaf(-q0, s, x), rcp, q0));
+            if (a == b) continue;
+            ++bad_h;
+            const float fa = pmx_oracle_half_to_float(a), fb = pmx_oracle_half_to_float(b);
+            if (fabsf(fa) < 1e9f && fabsf(fb) < 1e9f && (int)nearbyintf(fa) == (int)nearbyintf(fb)) continue;
+            ++bad_q;
+        }
+    }
+    if (half_differs) *half_differs = bad_h;
+    return bad_q;
+}
+
 /* Host threads the OpenMP loops above will use (reported beside CPU timings). */
 int pmx_oracle_num_threads(void)
 {

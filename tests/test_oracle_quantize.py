@@ -78,6 +78,16 @@ def test_c_equals_numpy_on_every_absmax(oracle):
     assert (qn[:, 0] == -qn[:, 1]).all()               # sign symmetry
 
 
+def test_reciprocal_quotient_identity_over_every_pair(oracle):
+    """The HIP quantiser divides once per group (rcp = 1/scale) and corrects each channel's x * rcp with a
+    residual step; over every finite half x and every half scale >= eps the int8 result is that of the
+    reference's half division (kernel.cu:144-148).  The half quotients differ in bits only for x = -0
+    (one pair per scale), which quantises to 0 either way."""
+    bad, half_differs = oracle.count_reciprocal_quotient_mismatches()
+    assert bad == 0
+    assert half_differs == 0x7C00 - 0x00A8
+
+
 def test_random_groups_c_equals_numpy_and_error_bound(oracle):
     rng = np.random.default_rng(5)
     x = (rng.standard_normal((20000, 8)) * 10.0 ** rng.integers(-6, 3, (20000, 1))).astype(np.float16)
