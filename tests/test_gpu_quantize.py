@@ -98,6 +98,31 @@ def test_append_empty_and_single(pkg, oracle):
     assert np.array_equal(got_c, ref_c) and np.array_equal(_bits(got_s), _bits(ref_s))
 
 
+@pytest.mark.parametrize("cache_mode", [0, 1])
+@pytest.mark.parametrize("n_seq,hkv,d", [(300, 1, 8), (1500, 1, 8), (700, 2, 64)])
+def test_append_many_short_sequences(pkg, oracle, cache_mode, n_seq, hkv, d):
+    """Sequences of 0-5 new tokens behind a few decode sequences: a wave's lanes span many sequences (one 8-channel
+    group per token at head_dim 8), empty ones among them; more than 1024 sequences take the bisected lookup."""
+    rng0 = np.random.default_rng(n_seq + d)
+    q_lens = rng0.integers(1, 6, size=n_seq).tolist()
+    prior = rng0.integers(0, 200, size=n_seq).tolist()
+    bt, rng = pkg.workloads.custom_batch(n_seq, num_heads=hkv, num_kv_heads=hkv, head_dim=d, cache_mode=cache_mode,
+                                         dec_kv_lens=[7, 1, 300], prefill_q_lens=q_lens, prefill_prior=prior,
+                                         outliers=False)
+    empty = 3 + np.flatnonzero(rng0.random(n_seq) < 0.3)
+    bt.kv_lens[empty] -= bt.q_lens[empty]
+    bt.q_lens[empty] = 0
+    bt.seqstarts = np.concatenate([[0], np.cumsum(bt.q_lens)]).astype(np.int64)
+    bt.start_pos = (bt.kv_lens - bt.q_lens).astype(np.int64)
+    n = int(bt.q_lens.sum())
+    k = rng.standard_normal((n, hkv, d)).astype(np.float16)
+    v = rng.standard_normal((n, hkv, d)).astype(np.float16)
+    got_c, got_s = run_append(pkg, bt, k, v)
+    ref_c, ref_s = host_cache(bt, canary=(0x5A, 1.5))
+    oracle_append_step(oracle, bt, k, v, ref_c, ref_s)
+    assert np.array_equal(got_c, ref_c) and np.array_equal(_bits(got_s), _bits(ref_s))
+
+
 def test_key_value_cache_flat_entry_point(pkg, oracle):
     """pmxhip_key_value_cache (flattened argument list) writes the same bytes."""
     import ctypes
