@@ -55,6 +55,22 @@ def test_scaled_c5_through_the_operator(pkg, oracle):
     full_step(pkg, oracle, bt, rng)
 
 
+@pytest.mark.parametrize("heads", [(32, 8, 128), (64, 8, 128), (8, 8, 64)])
+def test_cache_beyond_4_gib(pkg, oracle, heads):
+    """A cache of many layers whose last layer lies more than 4 GiB into the allocation (a serving cache on a
+    288 GB part is tens of GiB): every kernel's element offsets must be 64-bit.  The whole cache is compared, so
+    a write at a wrapped offset shows as a damaged canary in another layer."""
+    hq, hkv, d = heads
+    kw = dict(num_heads=hq, num_kv_heads=hkv, head_dim=d, cache_mode=1, dec_kv_lens=[600, 33, 1500, 129, 1, 256],
+              prefill_q_lens=[100, 17], prefill_prior=[150, 0], outliers=True)
+    probe, _ = pkg.workloads.custom_batch(405, num_layer=1, layer_idx=0, **kw)
+    layer_bytes = 2 * probe.layout.pool_tokens * hkv * d
+    layers = (4 << 30) // layer_bytes + 3
+    bt, rng = pkg.workloads.custom_batch(405, num_layer=layers, layer_idx=layers - 1, **kw)
+    assert bt.layer_idx * layer_bytes > (4 << 30)
+    full_step(pkg, oracle, bt, rng)
+
+
 def test_forward_in_a_hip_graph(pkg, oracle):
     """forward() records no memory-set node and allocates nothing, so a caller can capture it: every replay,
     with eager calls between the replays, gives the rows of the eager call bit for bit."""
