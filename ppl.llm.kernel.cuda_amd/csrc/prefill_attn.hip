@@ -46,6 +46,99 @@ constexpr float kPShift = 14.0f;
 // token bits (a, h, r1, r0) -> position bits (h, a, r1, r0)
 __device__ __forceinline__ int vt_pos16(int o) { return ((o & 4) << 1) | ((o & 8) >> 1) | (o & 3); }
 
+// sum over the wave of small non-negative integers, one ballot per bit (every lane of the wave must be here)
+__device__ __forceinline__ int wave_sum_small(int v)
+{
+    int sum = 0;
+    for (int bit = 0; __builtin_amdgcn_ballot_w64((v >> bit) != 0) != 0; ++bit)
+        sum += __builtin_popcountll(__builtin_amdgcn_ballot_w64(((v >> bit) & 1) != 0)) << bit;
+    return sum;
+}
+
+// Which query tile a workgroup takes.  The tiles of a ragged batch cost very different amounts (a tile walks the kv
+// tokens up to its last query row: prior context + rows so far), a CU holds one workgroup, and workgroups start in
+// the order of their numbers, so the order decides how long the last CUs run alone: with the dear tiles first the
+// cheap ones fill the gaps at the end.  Tile t of sequence s gets the level t + ceil(prior_s / ppw) (its cost in
+// units of ppw tokens) and item i of the launch is the i-th tile in the order of falling level (sequences in
+// index order inside a level).  Every wave finds its tile by itself from seqstarts/kvstarts: a lane holds the
+// level interval [lo, lo + n) of up to kPickSlots sequences, the number of tiles at or above a level is a sum over
+// the lanes, and the item's level follows by bisection.  Beyond 64 * kPickSlots sequences the order is the plain
+// one (last tiles first, sequences in index order).  Returns false for an item beyond the batch's tiles.
+constexpr int kPickSlots = 16;
+__device__ __forceinline__ bool pick_query_tile(const PrefillLaunch& a, int ppw, int item, int lane, int& b_out, int& tile_out)
+{
+    const int nseq = (int)a.prefill_batches;
+    if (nseq > 64 * kPickSlots) {
+        const int tiles_max = (int)((a.max_seqlen + ppw - 1) / ppw);
+        const int y = item / nseq;
+        b_out = item - y * nseq;
+        tile_out = tiles_max - 1 - y;
+        return y < tiles_max;
+    }
+    const int kmax = (nseq + 63) >> 6;
+    int lo[kPickSlots], n[kPickSlots];
+    int hi_lane = 0;
+#pragma unroll
+    for (int k = 0; k < kPickSlots; ++k) {
+        lo[k] = 0;
+        n[k] = 0;
+        if (k < kmax) {
+            const int s = 64 * k + lane;
+            if (s < nseq) {
+                const int qlen = (int)(a.seqstarts[s + 1] - a.seqstarts[s]);
+                const int kvlen = (int)(a.kvstarts[s + 1] - a.kvstarts[s]);
+                int prior = a.is_causal ? kvlen - qlen : kvlen;
+                prior = prior > 0 ? prior : 0;
+                lo[k] = (prior + ppw - 1) / ppw;
+                n[k] = qlen > 0 ? (qlen + ppw - 1) / ppw : 0;
+                hi_lane = hi_lane > lo[k] + n[k] ? hi_lane : lo[k] + n[k];
+            }
+        }
+    }
+    // tiles at or above level l
+    auto count_from = [&](int l) {
+        int c = 0;
+#pragma unroll
+        for (int k = 0; k < kPickSlots; ++k)
+            if (k < kmax) {
+                const int from = l > lo[k] ? l : lo[k];
+                const int d = lo[k] + n[k] - from;
+                c += d > 0 ? d : 0;
+            }
+        return wave_sum_small(c);
+    };
+    if (item >= count_from(0)) return false;
+    // the largest level end of the wave, bit by bit
+    int top = 0;
+    for (int bit = 24; bit >= 0; --bit)
+        if (__builtin_amdgcn_ballot_w64(hi_lane >= (top | (1 << bit))) != 0) top |= 1 << bit;
+    int below = 0, above = top; // count_from(below) > item >= count_from(above)
+    while (above - below > 1) {
+        const int mid = (below + above) >> 1;
+        if (count_from(mid) > item) below = mid;
+        else above = mid;
+    }
+    const int level = below;
+    int r = item - count_from(level + 1); // index among the sequences that have a tile at this level
+#pragma unroll
+    for (int k = 0; k < kPickSlots; ++k)
+        if (k < kmax) {
+            const bool has = lo[k] <= level && level < lo[k] + n[k];
+            const uint64_t mask = __builtin_amdgcn_ballot_w64(has);
+            const int cnt = __builtin_popcountll(mask);
+            if (r < cnt) {
+                const int before = __builtin_popcountll(mask & ((1ull << lane) - 1ull));
+                const uint64_t sel = __builtin_amdgcn_ballot_w64(has && before == r);
+                const int src = __builtin_ctzll(sel);
+                b_out = 64 * k + src;
+                tile_out = level - __builtin_amdgcn_readlane(lo[k], src);
+                return true;
+            }
+            r -= cnt;
+        }
+    return false;
+}
+
 } // namespace
 
 // SRC: where K/V come from: 0 = int8 cache in 128-token pages, 1 = int8 cache in contiguous runs,
@@ -82,17 +175,20 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     const int hh = lane >> 5;   // half-wave
     const int l32 = lane & 31;
 
-    // grid: x = (sequence, kv head), y = query tile; workgroups are dispatched x first, so every sequence's
-    // last query tile (the one that walks the most kv tokens) starts before any shorter one
-    const int b = blockIdx.x / (int)a.num_kv_heads;
-    const int kvh = blockIdx.x - b * (int)a.num_kv_heads;
+    // grid: workgroup = (item, kv head), kv head fastest; item i is the i-th query tile of the batch in the order
+    // of falling cost (pick_query_tile), and workgroups start in the order of their numbers
     const int G = (int)(a.num_heads / a.num_kv_heads);
     const int ppw = kCols / G > 0 ? kCols / G : 1; // query positions per workgroup
+    const int item = blockIdx.x / (int)a.num_kv_heads;
+    const int kvh = blockIdx.x - item * (int)a.num_kv_heads;
+    int b_pick = 0, tile_pick = 0;
+    if (!pick_query_tile(a, ppw, item, lane, b_pick, tile_pick)) return;
+    const int b = __builtin_amdgcn_readfirstlane(b_pick);
     const int64_t q_row0 = a.seqstarts[b];
     const int qlen = (int)(a.seqstarts[b + 1] - q_row0);
     const int kvlen = (int)(a.kvstarts[b + 1] - a.kvstarts[b]);
-    const int p0 = (int)(gridDim.y - 1 - blockIdx.y) * ppw;
-    if (p0 >= qlen) return;
+    const int p0 = __builtin_amdgcn_readfirstlane(tile_pick) * ppw;
+    if (p0 < 0 || p0 >= qlen) return;
 
     // ---- this lane's column ----
     const int col = wave * 32 + l32;
@@ -542,7 +638,8 @@ static void launch_prefill_d(const PrefillLaunch& a, hipStream_t stream)
 {
     const int G = (int)(a.num_heads / a.num_kv_heads);
     const int ppw = kCols / G > 0 ? kCols / G : 1;
-    const dim3 grid((unsigned)(a.prefill_batches * a.num_kv_heads), (unsigned)((a.max_seqlen + ppw - 1) / ppw), 1);
+    // one workgroup per (query tile, kv head) that the batch can have at most; the kernel numbers the real ones first
+    const dim3 grid((unsigned)(a.prefill_batches * ((a.max_seqlen + ppw - 1) / ppw) * a.num_kv_heads), 1, 1);
     const bool extra = a.attn_mask != nullptr || a.alibi_slopes != nullptr;
     const int src = a.current_key ? 2 : (a.cache_mode == 1 ? 0 : 1);
     if (extra) {

@@ -64,6 +64,27 @@ def test_prefill_short_chunks_over_long_histories(pkg, oracle, shape):
     assert_attention_close(got, ref, "short chunks %s" % (shape,))
 
 
+@pytest.mark.parametrize("n_seq,is_causal", [(150, True), (150, False), (1100, True)])
+def test_prefill_many_sequences_every_tile_once(pkg, oracle, n_seq, is_causal):
+    """The kernel numbers the batch's query tiles in the order of falling cost and every workgroup looks its own
+    tile up: with more than 64 sequences a lane holds several of them, beyond 1024 the plain order applies.  Every
+    output row must be written exactly once (rows left NaN or wrong show a tile that was skipped or mixed up);
+    sequences with a short prior context and many rows sit next to long ones with one row."""
+    rng0 = np.random.default_rng(n_seq)
+    big = n_seq <= 200
+    q_lens = rng0.integers(1, 150 if big else 4, size=n_seq)
+    prior = rng0.integers(0, 300 if big else 40, size=n_seq)
+    q_lens[::7] = 1
+    prior[::7] = rng0.integers(200 if big else 30, 400 if big else 60, size=len(prior[::7]))
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 360 + n_seq, num_heads=4, num_kv_heads=2, head_dim=64,
+                                         cache_mode=1, dec_kv_lens=[5], prefill_q_lens=q_lens.tolist(),
+                                         prefill_prior=prior.tolist(), is_causal=is_causal)
+    ref = oracle_prefill(oracle, bt, q, cache, scale)
+    got = run_prefill(pkg, dev)
+    assert np.isnan(got[:1]).all() and not np.isnan(got[1:]).any()
+    assert_attention_close(got[1:], ref[1:], "many sequences %d" % n_seq)
+
+
 def test_prefill_non_causal_and_single_row_equals_decode(pkg, oracle):
     bt, dev, q, cache, scale = make_case(pkg, oracle, 320, num_heads=8, num_kv_heads=2, head_dim=128, cache_mode=1,
                                          dec_kv_lens=[], prefill_q_lens=[1, 65], prefill_prior=[300, 10],
