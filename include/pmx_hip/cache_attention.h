@@ -70,6 +70,7 @@ public:
         int64_t workspace_size;
         void* workspace; // the caller assigns this after heuristic_prepare, before forward*()
         bool enable_cache_prefill;
+        int64_t prefill_query_rows; // not in the reference: rows of query beyond the decode rows (sizes the prefill launch)
     } cfg{};
 
     // Validates, derives strides / attn_scale / split plan and fills cfg.  Host only.

@@ -86,6 +86,7 @@ class PrefillParams(ctypes.Structure):
         ("cache_stride_kv", c_i64), ("cachestarts_stride_b", c_i64),
         ("attn_mask", c_vp), ("mask_stride_s", c_i64), ("mask_stride_h", c_i64), ("alibi_slopes", c_vp),
         ("current_key", c_vp), ("current_value", c_vp), ("key_stride_s", c_i64), ("value_stride_s", c_i64),
+        ("prefill_query_rows", c_i64),
     ]
 
 

@@ -358,6 +358,7 @@ int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t str
     a.cache_mode = p->cache_mode;
     a.prefill_batches = prefill_batches;
     a.max_seqlen = p->max_seqlen;
+    a.query_rows = p->prefill_query_rows > 0 ? p->prefill_query_rows : 0;
     a.layer_idx = p->layer_idx;
     a.num_heads = p->num_heads;
     a.num_kv_heads = p->num_kv_heads;

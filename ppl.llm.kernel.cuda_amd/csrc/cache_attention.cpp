@@ -178,6 +178,7 @@ ppl::common::RetCode dynamic_batching_multi_head_cache_attention::heuristic_prep
     cfg.decoding_batches = decoding_batches;
     cfg.max_seqlen = max_seqlen;
     cfg.max_kvlen = max_kvlen;
+    cfg.prefill_query_rows = query_shape->GetDim(0) - decoding_batches; // decode sequences have one row each
     cfg.layer_idx = layer_idx;
     cfg.num_layer = num_layer;
     cfg.num_heads = num_heads;
@@ -322,6 +323,7 @@ ppl::common::RetCode dynamic_batching_multi_head_cache_attention::forward_prefil
     p.mask_stride_s = cfg.mask_stride_s;
     p.mask_stride_h = cfg.mask_stride_h;
     p.alibi_slopes = static_cast<const float*>(cfg.alibi_slopes);
+    p.prefill_query_rows = cfg.prefill_query_rows;
     if (!cfg.enable_cache_prefill) { // kernel.cu:2181-2212: the step's own fp16 K/V only, no cache read
         p.current_key = cfg.current_key;
         p.current_value = cfg.current_value;

@@ -79,6 +79,7 @@ struct PrefillLaunch {
     int32_t cache_mode;
     int64_t prefill_batches;
     int64_t max_seqlen;
+    int64_t query_rows;         // rows of the prefill sequences, 0 = unknown (bounds the launch only)
     int64_t layer_idx;
     int64_t num_heads;
     int64_t num_kv_heads;

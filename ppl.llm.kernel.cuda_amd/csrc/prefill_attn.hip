@@ -638,8 +638,14 @@ static void launch_prefill_d(const PrefillLaunch& a, hipStream_t stream)
 {
     const int G = (int)(a.num_heads / a.num_kv_heads);
     const int ppw = kCols / G > 0 ? kCols / G : 1;
-    // one workgroup per (query tile, kv head) that the batch can have at most; the kernel numbers the real ones first
-    const dim3 grid((unsigned)(a.prefill_batches * ((a.max_seqlen + ppw - 1) / ppw) * a.num_kv_heads), 1, 1);
+    // one workgroup per (query tile, kv head) that the batch can have at most; the kernel numbers the real ones first.
+    // Every sequence has at most the tiles of max_seqlen; all together at most one per ppw rows plus a partial one each.
+    int64_t items = a.prefill_batches * ((a.max_seqlen + ppw - 1) / ppw);
+    if (a.query_rows > 0 && a.prefill_batches <= 64 * kPickSlots) {
+        const int64_t by_rows = a.query_rows / ppw + a.prefill_batches;
+        if (by_rows < items) items = by_rows;
+    }
+    const dim3 grid((unsigned)(items * a.num_kv_heads), 1, 1);
     const bool extra = a.attn_mask != nullptr || a.alibi_slopes != nullptr;
     const int src = a.current_key ? 2 : (a.cache_mode == 1 ? 0 : 1);
     if (extra) {

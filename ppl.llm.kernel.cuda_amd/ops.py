@@ -147,7 +147,8 @@ def prefill_attention(query, output, cache, scale, seqstarts, kvstarts, cachesta
                       batch, decoding_batches, max_seqlen, max_kvlen, layer_idx, num_heads, num_kv_heads,
                       head_dim, cache_mode, page_size, cache_stride_s, cache_stride_l, cache_stride_h,
                       cache_stride_kv, cachestarts_stride_b, attn_mask=None, mask_stride_s=0, mask_stride_h=0,
-                      alibi_slopes=None, current_key=None, current_value=None, stream=None, check=True):
+                      alibi_slopes=None, current_key=None, current_value=None, prefill_query_rows=None, stream=None,
+                      check=True):
     """Multi-query-token attention of the prefill sequences.  Optional: additive half `attn_mask` with its
     strides, float32 `alibi_slopes` [Hq], and `current_key`/`current_value` [rows, KVH, D] to attend over
     the step's own fp16 rows instead of the cache."""
@@ -187,6 +188,8 @@ def prefill_attention(query, output, cache, scale, seqstarts, kvstarts, cachesta
         p.current_value = _ptr(current_value)
         p.key_stride_s = num_kv_heads * head_dim
         p.value_stride_s = num_kv_heads * head_dim
+    # the rows of the prefill sequences follow from the query tensor, as in the reference's call
+    p.prefill_query_rows = (int(query.shape[0]) - decoding_batches) if prefill_query_rows is None else prefill_query_rows
     rc = _lib.lib().pmxhip_prefill_attention(ctypes.byref(p), _stream(stream))
     if check and rc != RC_SUCCESS:
         raise PmxError(rc, "prefill_attention")

@@ -83,6 +83,9 @@ def test_prefill_many_sequences_every_tile_once(pkg, oracle, n_seq, is_causal):
     got = run_prefill(pkg, dev)
     assert np.isnan(got[:1]).all() and not np.isnan(got[1:]).any()
     assert_attention_close(got[1:], ref[1:], "many sequences %d" % n_seq)
+    # the row count only sizes the launch: without it (0 = unknown) the rows are the same bit for bit
+    got0 = run_prefill(pkg, dev, prefill_query_rows=0)
+    assert np.array_equal(got0[1:].view(np.uint32), got[1:].view(np.uint32))
 
 
 def test_prefill_non_causal_and_single_row_equals_decode(pkg, oracle):
