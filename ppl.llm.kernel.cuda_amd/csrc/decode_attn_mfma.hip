@@ -363,6 +363,9 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
 {
     constexpr int D = kMfmaD;
     __shared__ __attribute__((aligned(16))) half_t s_vt[NW][2][D * kMfmaBlock]; // [wave][hi, lo]
+    // a block's raw K rows, on their way from whole-line loads to the lanes that hold them as MFMA operands:
+    // row = token, eight 16-byte chunks per row, chunk index XORed with (token ^ token >> 3) & 7 (no bank conflicts)
+    __shared__ __attribute__((aligned(16))) char s_k[NW][kMfmaBlock * D];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -373,6 +376,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
     const int kvh = blockIdx.y * NW + wave;
     half_t* const sV = s_vt[wave][0];
     half_t* const sVlo = s_vt[wave][1];
+    char* const sK = s_k[wave];
 
     const const_i64_ptr kvstarts = as_constant(a.kvstarts);
     const const_i64_ptr cachestarts = as_constant(a.cachestarts);
@@ -441,15 +445,19 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
 
         // ---- raw bytes of one block: K of tokens r16 and 16 + r16, V as two (token quad, group) units ----
         u32x4 kq[2][2];
+        u32x4 kraw[4];      // K as loaded: token 8 i + lane / 8, channels 16 (lane % 8) .. + 16 (whole lines per instruction)
         uint32_t ksc[2][2]; // two half scales each
         u32x2 vq[2][4];
         half_t vsc[2][4];
         // per-lane offsets inside a block: constant except in a piece's last block, whose tokens beyond the
         // piece re-read its last token (their logits are masked)
         uint32_t k_off[2];
+        uint32_t kl_off[4];
         uint32_t v_off[2][4];
 #pragma unroll
         for (int t = 0; t < 2; ++t) k_off[t] = (uint32_t)(16 * t + r16) * stride_s32 + 16 * qq;
+#pragma unroll
+        for (int i4 = 0; i4 < 4; ++i4) kl_off[i4] = (uint32_t)(8 * i4 + (lane >> 3)) * stride_s32 + 16 * (lane & 7);
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -460,6 +468,11 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
             for (int t = 0; t < 2; ++t) {
                 const int tk = 16 * t + r16;
                 k_off[t] = (uint32_t)(tk < last ? tk : last) * stride_s32 + 16 * qq;
+            }
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                const int tk = 8 * i4 + (lane >> 3);
+                kl_off[i4] = (uint32_t)(tk < last ? tk : last) * stride_s32 + 16 * (lane & 7);
             }
 #pragma unroll
             for (int u = 0; u < 2; ++u)
@@ -474,11 +487,26 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
             const char* bk = cache_k + boff;
             const half_t* sk = scale_k + (boff >> 3);
 #pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) kraw[i4] = __builtin_nontemporal_load((const u32x4*)(bk + kl_off[i4]));
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) ksc[t][j] = *(const uint32_t*)(sk + (k_off[t] >> 3) + 8 * j);
+        };
+        // through the wave's LDS rows to the operand layout: lane (r16, qq) takes channels 64 j + 16 qq .. + 16 of the
+        // tokens r16 and 16 + r16 (the wave's LDS operations execute in order: no barrier)
+        auto stage_k = [&]() {
+#pragma unroll
+            for (int i4 = 0; i4 < 4; ++i4) {
+                const int tk = 8 * i4 + (lane >> 3);
+                *(u32x4*)(sK + tk * D + ((((lane & 7) ^ tk ^ (tk >> 3)) & 7) << 4)) = kraw[i4];
+            }
+#pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
-                    kq[t][j] = *(const u32x4*)(bk + k_off[t] + 64 * j);
-                    ksc[t][j] = *(const uint32_t*)(sk + (k_off[t] >> 3) + 8 * j);
+                    const int tk = 16 * t + r16;
+                    kq[t][j] = *(const u32x4*)(sK + tk * D + ((((4 * j + qq) ^ tk ^ (tk >> 3)) & 7) << 4));
                 }
         };
         auto load_v = [&](int pos) {
@@ -489,7 +517,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
             for (int u = 0; u < 2; ++u)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    vq[u][r] = *(const u32x2*)(bv + v_off[u][r]);
+                    vq[u][r] = __builtin_nontemporal_load((const u32x2*)(bv + v_off[u][r]));
                     vsc[u][r] = sv[v_off[u][r] >> 3];
                 }
         };
@@ -540,6 +568,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
             }
 
             // ---- S^T = K Q^T: the A fragments are built from this lane's raw bytes step by step ----
+            stage_k();
             f32x4 s_acc[2];
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
