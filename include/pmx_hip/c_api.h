@@ -215,8 +215,9 @@ typedef struct pmxhip_prefill_params {
     const void* current_value;
     int64_t key_stride_s;
     int64_t value_stride_s;
-    /* Rows of `query` that belong to the prefill sequences (the reference knows them from the query
-     * tensor's shape, fmha.cu:144-257 total_q); 0 = unknown.  Only the launch size depends on it: the
+    /* Rows of `query` that belong to the prefill sequences; 0 = unknown.  No counterpart in the reference's
+     * call, which sizes its launch from max_seqlen (kernel.cu:2143-2179); the operator class takes it from
+     * the query shape that heuristic_prepare receives.  Only the launch size depends on it: the
      * batch has at most rows / (positions per workgroup) + sequences query tiles, far fewer than
      * sequences * tiles of max_seqlen when one long sequence sits among short ones. */
     int64_t prefill_query_rows;

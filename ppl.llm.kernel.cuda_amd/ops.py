@@ -188,7 +188,7 @@ def prefill_attention(query, output, cache, scale, seqstarts, kvstarts, cachesta
         p.current_value = _ptr(current_value)
         p.key_stride_s = num_kv_heads * head_dim
         p.value_stride_s = num_kv_heads * head_dim
-    # the rows of the prefill sequences follow from the query tensor, as in the reference's call
+    # the rows of the prefill sequences follow from the query tensor (decode sequences have one row each)
     p.prefill_query_rows = (int(query.shape[0]) - decoding_batches) if prefill_query_rows is None else prefill_query_rows
     rc = _lib.lib().pmxhip_prefill_attention(ctypes.byref(p), _stream(stream))
     if check and rc != RC_SUCCESS:
