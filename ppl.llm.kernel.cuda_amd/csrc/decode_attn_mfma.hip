@@ -353,7 +353,9 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
 //   lane = (r = lane % 16, qq = lane / 16)
 //   S^T tile (16 tokens x 16 columns, two per block): A = K rows of token 16 tile + r, B = Q of head r;
 //     k-step s = 2 j + e pairs the lane's channels [64 j + 16 qq + 8 e, + 8) on both sides
-//     (one 16-byte load covers 64 j + 16 qq .. + 16: a load instruction reads whole 64-byte segments);
+//     (those 16-byte pieces reach the lane through LDS: with this layout a load instruction would read 64 of a
+//     row's 128 bytes, so the rows are loaded as whole lines by eight lanes each, with the non-temporal hint,
+//     and the block's 4 KB pass through a wave-private LDS buffer);
 //     the accumulator holds tokens 16 tile + 4 qq + i of column r
 //   O^T tile (16 channels x 16 columns, eight per block): A = row `channel 16 cb + r` of the V^T tile,
 //     16-byte block qq, whose eight positions are the tokens of the lane's two S^T accumulators in order:
