@@ -119,32 +119,59 @@ typedef struct pmxhip_decode_params {
     int64_t num_kv_heads;
     int64_t head_dim;
     int32_t cache_mode;
-    /* split-KV plan: from pmxhip_decode_plan(); workspace >= plan.workspace_size */
+    /* split-KV plan: from pmxhip_decode_plan_make(); workspace >= plan.workspace_size */
     int32_t num_token_ranges;
     void* workspace;
     int64_t workspace_size;
+    /* 0 (PMXHIP_DECODE_KERNEL_AUTO) = the library chooses the token-range kernel by shape.  Any other
+     * pmxhip_decode_kernel_t insists on that kernel (comparison runs, tests of every kernel on one shape); the
+     * call fails with PMXHIP_UNSUPPORTED when that kernel does not serve the shape or the buffers.  The plan
+     * must have been made for the same request (pmxhip_decode_plan_make_kernel). */
+    int32_t kernel_request;
 } pmxhip_decode_params;
+
+/* The token-range kernels of the decode step.  The reference chooses among its three kernels with the
+ * enable_* flags of heuristic_prepare (utils.cu:136-264); here the choice follows from the shape. */
+typedef enum pmxhip_decode_kernel_t {
+    PMXHIP_DECODE_KERNEL_AUTO = 0,
+    PMXHIP_DECODE_KERNEL_GENERAL = 1, /* VALU; every head_dim and head count */
+    PMXHIP_DECODE_KERNEL_QUAD = 2,    /* head_dim 128 (even number of kv heads) or 256, up to 4 query heads per kv
+                                         head (8 at head_dim 128 with kv heads in eights) */
+    PMXHIP_DECODE_KERNEL_MFMA16 = 3,  /* head_dim 128, up to 16 query heads per kv head as MFMA columns */
+    PMXHIP_DECODE_KERNEL_MFMA32 = 4   /* head_dim 128, up to 32 */
+} pmxhip_decode_kernel_t;
 
 typedef struct pmxhip_decode_plan {
     int32_t num_token_ranges;   /* workgroups along the kv-token stream */
-    int32_t kv_heads_per_group; /* kv heads one workgroup serves (the largest power of two up to 8 that divides
-                                   num_kv_heads, fewer for head_dim 256) */
-    int32_t q_heads_per_pass;   /* query heads per kv head served at once: up to 8 from registers, or the 32
-                                   MFMA columns when head_dim is 128 and num_kv_repeats is 5..32 (3..32 when
-                                   the kv heads do not come in eights); kv_heads_per_group is then 4, 2 or 1 */
+    int32_t kv_heads_per_group; /* kv heads one workgroup serves */
+    int32_t q_heads_per_pass;   /* query heads per kv head served at once: 1, 2, 4 or 8 from registers (general
+                                   and quad kernels), or the 16 / 32 MFMA columns */
     int32_t num_passes;         /* ceil(num_kv_repeats / q_heads_per_pass) */
     int64_t partial_out_size;   /* bytes: float32 partial outputs */
     int64_t partial_ml_size;    /* bytes: float32 (running max, exp-sum) pairs */
     int64_t workspace_size;     /* total bytes */
+    int32_t kernel;             /* pmxhip_decode_kernel_t the plan was made for.  The launch falls back to the
+                                   general kernel when the quad kernel's needs of the buffers (16-byte aligned
+                                   output rows) are not met; pmxhip_decode_kernel_name tells what a call runs. */
 } pmxhip_decode_plan;
 
-/* Host-only.  `compute_units` is hipDeviceProp_t::multiProcessorCount.
+/* Host-only.  `compute_units` is hipDeviceProp_t::multiProcessorCount (0 = ask the current device).
  * `num_token_ranges_hint` 0 = choose; > 0 = use exactly this many ranges. */
 PMXHIP_API int pmxhip_decode_plan_make(int64_t decoding_batches, int64_t num_heads, int64_t num_kv_heads,
                                        int64_t head_dim, int64_t max_kvlen, int32_t compute_units,
                                        int32_t num_token_ranges_hint, pmxhip_decode_plan* plan);
+/* The same for a requested kernel (pmxhip_decode_params::kernel_request). */
+PMXHIP_API int pmxhip_decode_plan_make_kernel(int64_t decoding_batches, int64_t num_heads, int64_t num_kv_heads,
+                                              int64_t head_dim, int64_t max_kvlen, int32_t compute_units,
+                                              int32_t num_token_ranges_hint, int32_t kernel_request,
+                                              pmxhip_decode_plan* plan);
 
 PMXHIP_API int pmxhip_decode_attention(const pmxhip_decode_params* p, pmxhip_stream_t stream);
+
+/* Name of the token-range kernel that pmxhip_decode_attention(p) launches ("" if the call would be rejected):
+ * one of decode_attention_kernel, decode_attention_quad_kernel, decode_attention_mfma16_kernel,
+ * decode_attention_mfma_kernel -- the names a profiler's kernel trace shows.  Host only, launches nothing. */
+PMXHIP_API const char* pmxhip_decode_kernel_name(const pmxhip_decode_params* p);
 
 /* The same step split at its kernel boundary, for callers that time or overlap
  * the two kernels: stage 1 = the token-range kernel only (final rows of
@@ -397,6 +424,13 @@ typedef struct pmxhip_rope_params {
 PMXHIP_API int pmxhip_rotary_position_embedding(const pmxhip_rope_params* p, pmxhip_stream_t stream);
 PMXHIP_API int pmxhip_rope_kv_cache_quantize(const pmxhip_rope_params* rope, const pmxhip_kvstore_params* store,
                                              pmxhip_stream_t stream);
+
+/* One-time set-up on the current device, for callers that record their first step under stream capture: the
+ * attribute calls of the kernels with large dynamic LDS (otherwise made at each kernel's first launch, which a
+ * capturing stream refuses with PMXHIP_OTHER_ERROR).  Optional
+ * otherwise; idempotent; host only.  No counterpart in the reference, whose cudaFuncSetAttribute calls sit in
+ * its launch path (kernel.cu:1946). */
+PMXHIP_API int pmxhip_init(void);
 
 /* Library identity / build check (host only). */
 PMXHIP_API const char* pmxhip_version(void);

@@ -22,6 +22,9 @@
  *     holds the range count.
  *   * cfg.workspace_size follows this implementation (float32 partial outputs
  *     and (max, sum) pairs; no arrival counters), not utils.cu:334-343.
+ *   * The prefill stage serves head_dim 64 and 128 (the reference's flash_attn2 also has 96 and 256).
+ *     heuristic_prepare rejects a batch with prefill sequences at any other head_dim with
+ *     RC_UNSUPPORTED, before anything is enqueued; decode-only batches take 64, 96, 128 and 256.
  */
 #ifndef PMX_HIP_CACHE_ATTENTION_H_
 #define PMX_HIP_CACHE_ATTENTION_H_
@@ -70,7 +73,9 @@ public:
         int64_t workspace_size;
         void* workspace; // the caller assigns this after heuristic_prepare, before forward*()
         bool enable_cache_prefill;
-        int64_t prefill_query_rows; // not in the reference: rows of query beyond the decode rows (sizes the prefill launch)
+        int64_t prefill_query_rows; // not in the reference: rows of query beyond the decode rows.  A hint that lets the
+                                    // prefill stage launch fewer workgroups; 0 = unknown.  A wrong value costs time only:
+                                    // the stage's workgroups walk every query tile of the batch whatever the launch size.
     } cfg{};
 
     // Validates, derives strides / attn_scale / split plan and fills cfg.  Host only.
@@ -82,7 +87,7 @@ public:
         const ppl::common::TensorShape* attn_mask_shape, const void* attn_mask, // (Sq, align8(Skv)) or (Hq, Sq, align8(Skv))
         const void* seqstarts, const void* kvstarts, // int64 (B + 1) each
         const void* cachestarts, const void* start_pos, // int64 (B) or (B, MaxP); int64 (B)
-        const void* alibi_slopes, // (Hq); accepted, unused on this path
+        const void* alibi_slopes, // float32 (Hq) or null; applied by the prefill stage only, as in the reference
         const bool is_causal,
         const int64_t batch, const int64_t decoding_batches,
         const int64_t max_seqlen, const int64_t max_kvlen,

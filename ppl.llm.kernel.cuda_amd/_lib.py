@@ -23,7 +23,9 @@ DATATYPE_FLOAT32 = 6
 EXPORTED_SYMBOLS = (
     "pmxhip_version", "pmxhip_last_error",
     "pmxhip_kv_cache_quantize", "pmxhip_key_value_cache",
-    "pmxhip_decode_plan_make", "pmxhip_decode_attention", "pmxhip_decode_attention_stage",
+    "pmxhip_init",
+    "pmxhip_decode_plan_make", "pmxhip_decode_plan_make_kernel", "pmxhip_decode_attention",
+    "pmxhip_decode_attention_stage", "pmxhip_decode_kernel_name",
     "pmxhip_splitkv_combine",
     "pmxhip_prefill_attention",
     "pmxhip_mhca_create", "pmxhip_mhca_destroy", "pmxhip_mhca_heuristic_prepare",
@@ -62,6 +64,7 @@ class DecodeParams(ctypes.Structure):
         ("decoding_batches", c_i64), ("num_heads", c_i64), ("num_kv_heads", c_i64), ("head_dim", c_i64),
         ("cache_mode", c_i32), ("num_token_ranges", c_i32),
         ("workspace", c_vp), ("workspace_size", c_i64),
+        ("kernel_request", c_i32),
     ]
 
 
@@ -70,7 +73,16 @@ class DecodePlan(ctypes.Structure):
         ("num_token_ranges", c_i32), ("kv_heads_per_group", c_i32),
         ("q_heads_per_pass", c_i32), ("num_passes", c_i32),
         ("partial_out_size", c_i64), ("partial_ml_size", c_i64), ("workspace_size", c_i64),
+        ("kernel", c_i32),
     ]
+
+
+# pmxhip_decode_kernel_t
+DECODE_KERNEL_AUTO = 0
+DECODE_KERNEL_GENERAL = 1
+DECODE_KERNEL_QUAD = 2
+DECODE_KERNEL_MFMA16 = 3
+DECODE_KERNEL_MFMA32 = 4
 
 
 class PrefillParams(ctypes.Structure):
@@ -196,6 +208,12 @@ def lib():
     L.pmxhip_key_value_cache.argtypes = [c_vp] * 6 + [c_i64] * 6 + [c_i32] + [c_i64] * 6 + [c_vp] * 2
     L.pmxhip_decode_plan_make.restype = ctypes.c_int
     L.pmxhip_decode_plan_make.argtypes = [c_i64] * 5 + [c_i32, c_i32, ctypes.POINTER(DecodePlan)]
+    L.pmxhip_init.restype = ctypes.c_int
+    L.pmxhip_init.argtypes = []
+    L.pmxhip_decode_plan_make_kernel.restype = ctypes.c_int
+    L.pmxhip_decode_plan_make_kernel.argtypes = [c_i64] * 5 + [c_i32, c_i32, c_i32, ctypes.POINTER(DecodePlan)]
+    L.pmxhip_decode_kernel_name.restype = ctypes.c_char_p
+    L.pmxhip_decode_kernel_name.argtypes = [ctypes.POINTER(DecodeParams)]
     L.pmxhip_decode_attention.restype = ctypes.c_int
     L.pmxhip_decode_attention.argtypes = [ctypes.POINTER(DecodeParams), c_vp]
     L.pmxhip_decode_attention_stage.restype = ctypes.c_int

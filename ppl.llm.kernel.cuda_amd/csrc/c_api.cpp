@@ -3,8 +3,9 @@
 // thread-local message (pmxhip_last_error).
 #include "pmx_hip/c_api.h"
 
-#include <hip/hip_runtime_api.h>
+#include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -49,18 +50,46 @@ int launch_status(const char* who)
     return PMXHIP_SUCCESS;
 }
 
-int largest_pow2_divisor_upto(int64_t n, int cap)
+int launch_result(const char* who, int launch_rc)
 {
-    int r = 1;
-    while (r * 2 <= cap && n % (r * 2) == 0) r *= 2;
-    return r;
+    if (launch_rc == pmxhip::kLaunchNoKernel) return fail(PMXHIP_UNSUPPORTED, "%s: no kernel for this shape", who);
+    if (launch_rc == pmxhip::kLaunchNeedsWarmup)
+        return fail(PMXHIP_OTHER_ERROR,
+                    "%s: the first launch of this kernel in the process came while the stream is being captured; "
+                    "call pmxhip_init() (or run one step outside the capture) first", who);
+    return launch_status(who);
+}
+
+// Compute units of the current device, looked up once per device.
+int current_compute_units()
+{
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> cached[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+    int cus = cached[dev].load(std::memory_order_relaxed);
+    if (cus == 0) {
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        cached[dev].store(cus, std::memory_order_relaxed);
+    }
+    return cus;
 }
 
 } // namespace
 
 extern "C" {
 
-const char* pmxhip_version(void) { return "pmx_hip 0.1 (gfx950)"; }
+const char* pmxhip_version(void) { return "pmx_hip 0.2 (gfx950)"; }
+
+int pmxhip_init(void)
+{
+    if (pmxhip::init_decode_kernels() != 0 || pmxhip::init_prefill_kernels() != 0) {
+        const hipError_t e = hipGetLastError();
+        return fail(PMXHIP_OTHER_ERROR, "init: hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+    }
+    (void)current_compute_units();
+    return PMXHIP_SUCCESS;
+}
 
 const char* pmxhip_last_error(void) { return g_last_error; }
 
@@ -103,8 +132,7 @@ int pmxhip_kv_cache_quantize(const pmxhip_kvstore_params* p, pmxhip_stream_t str
     a.cachestarts_stride_b = p->cachestarts_stride_b;
     a.max_tokens = p->batch * p->max_seqlen;
     a.cache_mode = p->cache_mode;
-    pmxhip::launch_kv_quantize(a, stream);
-    return launch_status("kv_cache_quantize");
+    return launch_result("kv_cache_quantize", pmxhip::launch_kv_quantize(a, current_compute_units(), stream));
 }
 
 int pmxhip_key_value_cache(pmxhip_stream_t stream, const void* current_key, const void* current_value,
@@ -145,6 +173,14 @@ int pmxhip_decode_plan_make(int64_t decoding_batches, int64_t num_heads, int64_t
                             int64_t max_kvlen, int32_t compute_units, int32_t num_token_ranges_hint,
                             pmxhip_decode_plan* plan)
 {
+    return pmxhip_decode_plan_make_kernel(decoding_batches, num_heads, num_kv_heads, head_dim, max_kvlen, compute_units,
+                                          num_token_ranges_hint, PMXHIP_DECODE_KERNEL_AUTO, plan);
+}
+
+int pmxhip_decode_plan_make_kernel(int64_t decoding_batches, int64_t num_heads, int64_t num_kv_heads, int64_t head_dim,
+                                   int64_t max_kvlen, int32_t compute_units, int32_t num_token_ranges_hint,
+                                   int32_t kernel_request, pmxhip_decode_plan* plan)
+{
     if (!plan) return fail(PMXHIP_INVALID_VALUE, "decode_plan: null plan");
     memset(plan, 0, sizeof(*plan));
     if (!head_dim_supported(head_dim))
@@ -152,38 +188,33 @@ int pmxhip_decode_plan_make(int64_t decoding_batches, int64_t num_heads, int64_t
     if (num_kv_heads <= 0 || num_heads <= 0 || num_heads % num_kv_heads != 0)
         return fail(PMXHIP_UNSUPPORTED, "only support num_heads %% num_kv_heads == 0.");
     if (num_token_ranges_hint < 0) return fail(PMXHIP_INVALID_VALUE, "decode_plan: negative range hint");
-    const int64_t repeats = num_heads / num_kv_heads;
-    const int lanes_per_slot = head_dim == 64 ? 4 : (head_dim == 256 ? 16 : 8);
-    const int slots_per_wave = 64 / lanes_per_slot;
-    // many query heads per kv head: the MFMA kernels, a wave per kv head, all query heads in one pass
-    const bool mfma = pmxhip::decode_mfma_shape(head_dim, num_heads, num_kv_heads);
-    const int kvhb = mfma ? pmxhip::decode_mfma_kv_heads(num_kv_heads)
-                          : largest_pow2_divisor_upto(num_kv_heads, slots_per_wave < 8 ? slots_per_wave : 8);
-    int gt = 1;
-    while (gt < repeats && gt < 8) gt *= 2;
-    if (mfma) gt = pmxhip::kDecodeMfmaColumns;
-    const int passes = (int)((repeats + gt - 1) / gt);
-    const int wg_tokens = mfma ? pmxhip::kDecodeMfmaTokens : pmxhip::decode_wg_tokens((int)head_dim, kvhb);
-    const int min_tokens = wg_tokens > 128 ? wg_tokens : 128;
+    if (kernel_request < PMXHIP_DECODE_KERNEL_AUTO || kernel_request > PMXHIP_DECODE_KERNEL_MFMA32)
+        return fail(PMXHIP_INVALID_VALUE, "decode_plan: unknown kernel request %d", kernel_request);
+    pmxhip::DecodeChoice c;
+    if (!pmxhip::decode_choose(head_dim, num_heads, num_kv_heads, kernel_request, &c))
+        return fail(PMXHIP_UNSUPPORTED, "decode_plan: kernel %d (%s) does not serve %lld query / %lld kv heads of %lld channels",
+                    kernel_request, pmxhip::decode_kernel_name(kernel_request), (long long)num_heads, (long long)num_kv_heads,
+                    (long long)head_dim);
+    const int min_tokens = c.wg_tokens > 128 ? c.wg_tokens : 128;
 
     int64_t ranges = num_token_ranges_hint;
     if (ranges == 0) {
-        const int64_t groups = (num_kv_heads / kvhb) * passes;
-        const int cus = compute_units > 0 ? compute_units : 256;
-        // workgroups that a CU holds at once: two of four waves, or as many as eight waves make where a kernel with
-        // smaller workgroups serves the shape (a wave per kv head, or per two)
-        const bool quad = !mfma && pmxhip::decode_quad_shape(head_dim, num_heads, num_kv_heads);
-        const int wgs_per_cu = mfma ? pmxhip::kDecodeMfmaWavesPerCu / kvhb : (quad ? (head_dim == 256 ? 8 : 16) / kvhb : 2);
-        ranges = ((int64_t)cus * wgs_per_cu + groups - 1) / groups;
+        const int64_t groups = (num_kv_heads / c.kv_heads_per_group) * c.num_passes;
+        int cus = compute_units > 0 ? compute_units : current_compute_units();
+        if (cus <= 0) return fail(PMXHIP_INVALID_VALUE, "decode_plan: compute_units not given and no current device");
+        // as many ranges as fill the workgroup slots of the chip: two workgroups of four waves per CU, or as many as
+        // eight waves make where a kernel with smaller workgroups serves the shape (a wave per kv head, or per two)
+        ranges = ((int64_t)cus * c.wgs_per_cu + groups - 1) / groups;
         const int64_t max_tokens = decoding_batches * (max_kvlen > 0 ? max_kvlen : 1);
         const int64_t useful = (max_tokens + min_tokens - 1) / min_tokens;
         if (ranges > useful) ranges = useful;
         if (ranges < 1) ranges = 1;
     }
     plan->num_token_ranges = (int32_t)ranges;
-    plan->kv_heads_per_group = kvhb;
-    plan->q_heads_per_pass = gt;
-    plan->num_passes = passes;
+    plan->kv_heads_per_group = c.kv_heads_per_group;
+    plan->q_heads_per_pass = c.q_heads_per_pass;
+    plan->num_passes = c.num_passes;
+    plan->kernel = c.kernel;
     if (ranges > 1) {
         const int64_t pieces = ranges + decoding_batches;
         plan->partial_out_size = pieces * num_heads * head_dim * (int64_t)sizeof(float);
@@ -193,54 +224,32 @@ int pmxhip_decode_plan_make(int64_t decoding_batches, int64_t num_heads, int64_t
     return PMXHIP_SUCCESS;
 }
 
-int pmxhip_decode_attention(const pmxhip_decode_params* p, pmxhip_stream_t stream)
-{
-    return pmxhip_decode_attention_stage(p, 0, stream);
-}
+namespace {
 
-int pmxhip_decode_attention_stage(const pmxhip_decode_params* p, int32_t stage, pmxhip_stream_t stream)
+// Checks of a decode call and the launch block it becomes.  `workspace` / `workspace_size` are the caller's
+// (pmxhip_decode_attention).
+int decode_prepare(const char* who, const pmxhip_decode_params* p, void* workspace, int64_t workspace_size,
+                   pmxhip::DecodeLaunch* out)
 {
-    if (stage < 0 || stage > 2) return fail(PMXHIP_INVALID_VALUE, "decode_attention: stage must be 0, 1 or 2");
-    if (!p) return fail(PMXHIP_INVALID_VALUE, "decode_attention: null params");
-    if (p->decoding_batches < 0) return fail(PMXHIP_INVALID_VALUE, "decode_attention: negative decoding_batches");
-    if (p->decoding_batches == 0) return PMXHIP_SUCCESS; // kernel.cu:2084
     if (!head_dim_supported(p->head_dim))
         return fail(PMXHIP_UNSUPPORTED, "cache flash decoding attention do not support head dim %lld", (long long)p->head_dim);
     if (p->num_kv_heads <= 0 || p->num_heads % p->num_kv_heads != 0 || p->num_kv_repeats != p->num_heads / p->num_kv_heads)
         return fail(PMXHIP_UNSUPPORTED, "only support num_heads %% num_kv_heads == 0.");
-    if (int rc = check_cache_layout("decode_attention", p->cache_mode, p->page_size, p->cache_stride_s, p->cache_stride_l,
+    if (int rc = check_cache_layout(who, p->cache_mode, p->page_size, p->cache_stride_s, p->cache_stride_l,
                                     p->cache_stride_h, p->cache_stride_kv, 16))
         return rc;
     if (!p->query || !p->output || !p->cache || !p->scale || !p->cachestarts || !p->kvstarts)
-        return fail(PMXHIP_INVALID_VALUE, "decode_attention: null device pointer");
+        return fail(PMXHIP_INVALID_VALUE, "%s: null device pointer", who);
     if (!aligned16(p->query) || !aligned16(p->cache) || (reinterpret_cast<uintptr_t>(p->scale) & 3u) ||
         p->query_stride_s % 8 != 0)
-        return fail(PMXHIP_UNSUPPORTED, "decode_attention: query/cache must be 16-byte aligned, scale 4-byte aligned");
+        return fail(PMXHIP_UNSUPPORTED, "%s: query/cache must be 16-byte aligned, scale 4-byte aligned", who);
     if ((reinterpret_cast<uintptr_t>(p->output) & 7u) || p->output_stride_s % 4 != 0) // 8-byte stores of four halves
-        return fail(PMXHIP_UNSUPPORTED, "decode_attention: output must be 8-byte aligned with a row stride that is a multiple of 4");
+        return fail(PMXHIP_UNSUPPORTED, "%s: output must be 8-byte aligned with a row stride that is a multiple of 4", who);
     if (p->attn_mask && p->mask_stride_s % 8 != 0) // utils.cu:127-130
         return fail(PMXHIP_UNSUPPORTED, "last dimension of attn_mask must be aligned with 8");
-
-    pmxhip_decode_plan plan;
-    if (p->num_token_ranges <= 0) return fail(PMXHIP_INVALID_VALUE, "decode_attention: num_token_ranges must be >= 1");
-    if (int rc = pmxhip_decode_plan_make(p->decoding_batches, p->num_heads, p->num_kv_heads, p->head_dim, 0, 0,
-                                         p->num_token_ranges, &plan))
-        return rc;
-    if (plan.workspace_size > 0) {
-        if (!p->workspace || p->workspace_size < plan.workspace_size)
-            return fail(PMXHIP_INVALID_VALUE, "decode_attention: workspace too small (%lld < %lld)",
-                        (long long)p->workspace_size, (long long)plan.workspace_size);
-        if (!aligned16(p->workspace)) return fail(PMXHIP_INVALID_VALUE, "decode_attention: workspace must be 16-byte aligned");
-    }
-
-    {   // per-lane cache offsets are 32-bit: (tokens of one wave block) * stride_s + (kv heads of a group) * stride_h
-        const int wg_tok = plan.q_heads_per_pass == pmxhip::kDecodeMfmaColumns
-                               ? pmxhip::kDecodeMfmaTokens
-                               : pmxhip::decode_wg_tokens((int)p->head_dim, plan.kv_heads_per_group);
-        const double span = (double)wg_tok * (double)p->cache_stride_s + (double)plan.kv_heads_per_group * (double)p->cache_stride_h;
-        if (p->cache_stride_s < 0 || p->cache_stride_h < 0 || span >= 2147483648.0)
-            return fail(PMXHIP_UNSUPPORTED, "decode_attention: cache_stride_s/cache_stride_h too large for 32-bit lane offsets");
-    }
+    if (p->num_token_ranges <= 0) return fail(PMXHIP_INVALID_VALUE, "%s: num_token_ranges must be >= 1", who);
+    if (p->kernel_request < PMXHIP_DECODE_KERNEL_AUTO || p->kernel_request > PMXHIP_DECODE_KERNEL_MFMA32)
+        return fail(PMXHIP_INVALID_VALUE, "%s: unknown kernel request %d", who, p->kernel_request);
 
     pmxhip::DecodeLaunch a{};
     a.query = p->query;
@@ -250,8 +259,6 @@ int pmxhip_decode_attention_stage(const pmxhip_decode_params* p, int32_t stage, 
     a.scale = p->scale;
     a.cachestarts = p->cachestarts;
     a.kvstarts = p->kvstarts;
-    a.partial_out = static_cast<float*>(p->workspace);
-    a.partial_ml = reinterpret_cast<float*>(static_cast<char*>(p->workspace) + plan.partial_out_size);
     a.attn_scale = p->attn_scale;
     a.cache_mode = p->cache_mode;
     a.layer_idx = p->layer_idx;
@@ -269,19 +276,75 @@ int pmxhip_decode_attention_stage(const pmxhip_decode_params* p, int32_t stage, 
     a.num_heads = p->num_heads;
     a.num_kv_heads = p->num_kv_heads;
     a.head_dim = (int32_t)p->head_dim;
-    a.ranges = plan.num_token_ranges;
-    a.kv_heads_per_group = plan.kv_heads_per_group;
-    a.q_heads_per_pass = plan.q_heads_per_pass;
-    a.num_passes = plan.num_passes;
-    // tokens that a workgroup takes per step, the unit of the range cuts: a property of the kernel that will run
-    if (plan.q_heads_per_pass == pmxhip::kDecodeMfmaColumns) a.wg_tokens = pmxhip::kDecodeMfmaTokens;
-    else if (pmxhip::decode_quad_shape(p->head_dim, p->num_heads, p->num_kv_heads) &&
-             (!p->attn_mask || pmxhip::decode_quad_mask_ok(p->num_heads, p->num_kv_repeats, p->mask_stride_h)))
-        a.wg_tokens = pmxhip::kDecodeQuadTokens;
-    else a.wg_tokens = pmxhip::decode_wg_tokens((int)p->head_dim, plan.kv_heads_per_group);
-    a.min_tokens_per_range = a.wg_tokens > 128 ? a.wg_tokens : 128;
-    if (pmxhip::launch_decode(a, stage, stream) != 0) return fail(PMXHIP_UNSUPPORTED, "decode_attention: no kernel for this shape");
-    return launch_status("decode_attention");
+    a.ranges = p->num_token_ranges;
+
+    // The kernel that will run, decided once and here: by shape (or by request), then by what the quad kernel
+    // needs of the buffers beyond this entry point's own checks.  Everything that depends on the kernel (the unit
+    // of the range cuts above all, which the combine kernel must share) follows from this one choice.
+    pmxhip::DecodeChoice c;
+    if (!pmxhip::decode_choose(p->head_dim, p->num_heads, p->num_kv_heads, p->kernel_request, &c))
+        return fail(PMXHIP_UNSUPPORTED, "%s: kernel %d (%s) does not serve this shape", who, p->kernel_request,
+                    pmxhip::decode_kernel_name(p->kernel_request));
+    if (c.kernel == pmxhip::kDecodeKernelQuad && !pmxhip::decode_quad_launch_ok(a)) {
+        if (p->kernel_request == PMXHIP_DECODE_KERNEL_QUAD)
+            return fail(PMXHIP_UNSUPPORTED, "%s: the quad kernel needs 16-byte aligned output rows and, with attn_mask, at "
+                                            "most four query heads per kv head", who);
+        pmxhip::decode_choose(p->head_dim, p->num_heads, p->num_kv_heads, pmxhip::kDecodeKernelGeneral, &c);
+    }
+    a.kernel = c.kernel;
+    a.kv_heads_per_group = c.kv_heads_per_group;
+    a.q_heads_per_pass = c.q_heads_per_pass;
+    a.num_passes = c.num_passes;
+    a.wg_tokens = c.wg_tokens;
+    a.min_tokens_per_range = c.wg_tokens > 128 ? c.wg_tokens : 128;
+
+    if (a.ranges > 1) {
+        const int64_t pieces = (int64_t)a.ranges + p->decoding_batches;
+        const int64_t out_bytes = pieces * p->num_heads * p->head_dim * (int64_t)sizeof(float);
+        const int64_t ml_bytes = pieces * p->num_heads * 2 * (int64_t)sizeof(float);
+        if (!workspace || workspace_size < out_bytes + ml_bytes)
+            return fail(PMXHIP_INVALID_VALUE, "%s: workspace too small (%lld < %lld)", who, (long long)workspace_size,
+                        (long long)(out_bytes + ml_bytes));
+        if (!aligned16(workspace)) return fail(PMXHIP_INVALID_VALUE, "%s: workspace must be 16-byte aligned", who);
+        a.partial_out = static_cast<float*>(workspace);
+        a.partial_ml = reinterpret_cast<float*>(static_cast<char*>(workspace) + out_bytes);
+    }
+
+    {   // per-lane cache offsets are 32-bit: (tokens of one wave block) * stride_s + (kv heads of a group) * stride_h
+        const double span = (double)c.wg_tokens * (double)p->cache_stride_s + (double)c.kv_heads_per_group * (double)p->cache_stride_h;
+        if (p->cache_stride_s < 0 || p->cache_stride_h < 0 || span >= 2147483648.0)
+            return fail(PMXHIP_UNSUPPORTED, "%s: cache_stride_s/cache_stride_h too large for 32-bit lane offsets", who);
+    }
+    *out = a;
+    return PMXHIP_SUCCESS;
+}
+
+} // namespace
+
+int pmxhip_decode_attention(const pmxhip_decode_params* p, pmxhip_stream_t stream)
+{
+    return pmxhip_decode_attention_stage(p, 0, stream);
+}
+
+int pmxhip_decode_attention_stage(const pmxhip_decode_params* p, int32_t stage, pmxhip_stream_t stream)
+{
+    if (stage < 0 || stage > 2) return fail(PMXHIP_INVALID_VALUE, "decode_attention: stage must be 0, 1 or 2");
+    if (!p) return fail(PMXHIP_INVALID_VALUE, "decode_attention: null params");
+    if (p->decoding_batches < 0) return fail(PMXHIP_INVALID_VALUE, "decode_attention: negative decoding_batches");
+    if (p->decoding_batches == 0) return PMXHIP_SUCCESS; // kernel.cu:2084
+    pmxhip::DecodeLaunch a;
+    if (int rc = decode_prepare("decode_attention", p, p->workspace, p->workspace_size, &a)) return rc;
+    return launch_result("decode_attention", pmxhip::launch_decode(a, stage, stream));
+}
+
+const char* pmxhip_decode_kernel_name(const pmxhip_decode_params* p)
+{
+    if (!p || p->decoding_batches <= 0) return "";
+    pmxhip::DecodeLaunch a;
+    // the workspace plays no part in the choice; a dummy satisfies the size check
+    alignas(16) static char dummy[16];
+    if (decode_prepare("decode_kernel_name", p, p->workspace ? p->workspace : dummy, INT64_MAX, &a) != PMXHIP_SUCCESS) return "";
+    return pmxhip::decode_kernel_name(a.kernel);
 }
 
 int pmxhip_splitkv_combine(const float* partial_out, const float* partial_ml, const int64_t* piece_begin,
@@ -370,8 +433,7 @@ int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t str
     a.cache_stride_h = p->cache_stride_h;
     a.cache_stride_kv = p->cache_stride_kv;
     a.cachestarts_stride_b = p->cachestarts_stride_b;
-    if (pmxhip::launch_prefill(a, stream) != 0) return fail(PMXHIP_UNSUPPORTED, "prefill_attention: no kernel for this shape");
-    return launch_status("prefill_attention");
+    return launch_result("prefill_attention", pmxhip::launch_prefill(a, stream));
 }
 
 static int reorder_common(const char* what, bool invert, pmxhip_stream_t stream, const void* cache, const void* scale,
@@ -507,8 +569,7 @@ static int rope_common(const char* what, const pmxhip_rope_params* p, const pmxh
         a.cachestarts_stride_b = st->cachestarts_stride_b;
         a.cache_mode = st->cache_mode;
     }
-    if (pmxhip::launch_rope(a, stream) != 0) return fail(PMXHIP_UNSUPPORTED, "%s: no kernel for this shape", what);
-    return launch_status(what);
+    return launch_result(what, pmxhip::launch_rope(a, stream));
 }
 
 int pmxhip_rotary_position_embedding(const pmxhip_rope_params* p, pmxhip_stream_t stream)

@@ -655,58 +655,66 @@ __global__ __launch_bounds__(64) void splitkv_combine_rows_kernel(
 // ---- host-side launchers (called from the C ABI) -------------------------------
 
 template <int D, int GT, bool PAGED, bool MASK>
-static void launch_decode_variant(const DecodeLaunch& a, dim3 grid, hipStream_t stream)
+static std::atomic<int>& decode_variant_ready()
+{
+    static std::atomic<int> ready{0};
+    return ready;
+}
+
+template <int D, int GT, bool PAGED, bool MASK>
+static int launch_decode_variant(const DecodeLaunch& a, dim3 grid, hipStream_t stream)
 {
     constexpr size_t lds_bytes = decode_lds_bytes(D, GT);
     // above the default limit of dynamic LDS per workgroup for the wider variants
-    static const hipError_t once = hipFuncSetAttribute((const void*)decode_attention_kernel<D, GT, PAGED, MASK>,
-                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    (void)once;
+    if (int rc = ensure_dynamic_lds((const void*)decode_attention_kernel<D, GT, PAGED, MASK>, (int)lds_bytes, stream,
+                                    decode_variant_ready<D, GT, PAGED, MASK>()))
+        return rc;
     hipLaunchKernelGGL((decode_attention_kernel<D, GT, PAGED, MASK>), grid, dim3(kDecodeThreads), lds_bytes, stream, a);
+    return kLaunchOk;
 }
 
 template <int D, int GT>
-static void launch_decode_dgt(const DecodeLaunch& a, dim3 grid, hipStream_t stream)
+static int launch_decode_dgt(const DecodeLaunch& a, dim3 grid, hipStream_t stream)
 {
     const bool paged = a.cache_mode == 1;
     const bool mask = a.attn_mask != nullptr;
-    if (paged) {
-        if (mask) launch_decode_variant<D, GT, true, true>(a, grid, stream);
-        else launch_decode_variant<D, GT, true, false>(a, grid, stream);
-    } else {
-        if (mask) launch_decode_variant<D, GT, false, true>(a, grid, stream);
-        else launch_decode_variant<D, GT, false, false>(a, grid, stream);
-    }
-}
-
-// PMX_HIP_DECODE_GENERAL=1 keeps every shape on the general kernel (for comparisons)
-bool decode_general_forced()
-{
-    static const bool forced = [] {
-        const char* e = getenv("PMX_HIP_DECODE_GENERAL");
-        return e && e[0] == '1';
-    }();
-    return forced;
+    if (paged) return mask ? launch_decode_variant<D, GT, true, true>(a, grid, stream)
+                           : launch_decode_variant<D, GT, true, false>(a, grid, stream);
+    return mask ? launch_decode_variant<D, GT, false, true>(a, grid, stream)
+                : launch_decode_variant<D, GT, false, false>(a, grid, stream);
 }
 
 template <int D>
 static int launch_decode_d(const DecodeLaunch& a, int stage, hipStream_t stream)
 {
-    const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / a.kv_heads_per_group), (unsigned)a.num_passes);
-    if (stage != 2 && D == 128 && decode_mfma_applicable(a) && !decode_general_forced()) {
-        launch_decode_mfma(a, stream);
-    } else if (stage != 2 && (D == 128 || D == 256) && decode_quad_applicable(a) && !decode_general_forced()) {
-        launch_decode_quad(a, stream);
-    } else if (stage != 2) {
-        switch (a.q_heads_per_pass) {
-            case 1: launch_decode_dgt<D, 1>(a, grid, stream); break;
-            case 2: launch_decode_dgt<D, 2>(a, grid, stream); break;
-            case 4: launch_decode_dgt<D, 4>(a, grid, stream); break;
-            case 8: launch_decode_dgt<D, 8>(a, grid, stream); break;
-            default: return 1;
+    if (stage != 2) {
+        switch (a.kernel) {
+            case kDecodeKernelMfma16:
+            case kDecodeKernelMfma32:
+                if (D != 128) return kLaunchNoKernel;
+                launch_decode_mfma(a, stream);
+                break;
+            case kDecodeKernelQuad:
+                if (D != 128 && D != 256) return kLaunchNoKernel;
+                launch_decode_quad(a, stream);
+                break;
+            case kDecodeKernelGeneral: {
+                const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / a.kv_heads_per_group), (unsigned)a.num_passes);
+                int rc = kLaunchNoKernel;
+                switch (a.q_heads_per_pass) {
+                    case 1: rc = launch_decode_dgt<D, 1>(a, grid, stream); break;
+                    case 2: rc = launch_decode_dgt<D, 2>(a, grid, stream); break;
+                    case 4: rc = launch_decode_dgt<D, 4>(a, grid, stream); break;
+                    case 8: rc = launch_decode_dgt<D, 8>(a, grid, stream); break;
+                    default: break;
+                }
+                if (rc != kLaunchOk) return rc;
+                break;
+            }
+            default: return kLaunchNoKernel;
         }
     }
-    if (stage == 1) return 0;
+    if (stage == 1) return kLaunchOk;
     // always run: it also writes the zero rows of empty sequences
     {
         // waves per (sequence, head) row by the mean number of pieces per sequence: with many rows of a few
@@ -717,7 +725,40 @@ static int launch_decode_d(const DecodeLaunch& a, int stage, hipStream_t stream)
         else if (a.ranges <= 48 * a.decoding_batches) hipLaunchKernelGGL((decode_combine_kernel<D, 2>), cgrid, dim3(128), 0, stream, a);
         else hipLaunchKernelGGL((decode_combine_kernel<D, 4>), cgrid, dim3(256), 0, stream, a);
     }
-    return 0;
+    return kLaunchOk;
+}
+
+// the one-time attribute call of every variant (pmxhip_init)
+template <int D, int GT>
+static int init_decode_dgt()
+{
+    hipError_t e = hipSuccess;
+    auto one = [&](const void* k, std::atomic<int>& ready) {
+        if (e == hipSuccess && ready.load() == 0) {
+            e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)decode_lds_bytes(D, GT));
+            if (e == hipSuccess) ready.store(1);
+        }
+    };
+    one((const void*)decode_attention_kernel<D, GT, true, true>, decode_variant_ready<D, GT, true, true>());
+    one((const void*)decode_attention_kernel<D, GT, true, false>, decode_variant_ready<D, GT, true, false>());
+    one((const void*)decode_attention_kernel<D, GT, false, true>, decode_variant_ready<D, GT, false, true>());
+    one((const void*)decode_attention_kernel<D, GT, false, false>, decode_variant_ready<D, GT, false, false>());
+    return e == hipSuccess ? kLaunchOk : kLaunchNoKernel;
+}
+template <int D>
+static int init_decode_d()
+{
+    if (int rc = init_decode_dgt<D, 1>()) return rc;
+    if (int rc = init_decode_dgt<D, 2>()) return rc;
+    if (int rc = init_decode_dgt<D, 4>()) return rc;
+    return init_decode_dgt<D, 8>();
+}
+int init_decode_kernels()
+{
+    if (int rc = init_decode_d<64>()) return rc;
+    if (int rc = init_decode_d<96>()) return rc;
+    if (int rc = init_decode_d<128>()) return rc;
+    return init_decode_d<256>();
 }
 
 int launch_decode(const DecodeLaunch& a, int stage, hipStream_t stream)
@@ -727,7 +768,7 @@ int launch_decode(const DecodeLaunch& a, int stage, hipStream_t stream)
         case 96: return launch_decode_d<96>(a, stage, stream);
         case 128: return launch_decode_d<128>(a, stage, stream);
         case 256: return launch_decode_d<256>(a, stage, stream);
-        default: return 1;
+        default: return kLaunchNoKernel;
     }
 }
 

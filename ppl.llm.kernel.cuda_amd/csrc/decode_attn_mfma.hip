@@ -31,9 +31,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kMfmaD = 128;
 constexpr int kMfmaBlock = 32;  // tokens per wave iteration (rows of one MFMA block)
-constexpr int kMfmaMaxHeads = 4; // kv heads (= waves) per workgroup: four, or two or one when the kv heads do not come in fours
-constexpr int kMfmaCols = 32;   // columns of the MFMA block: query heads of the kv head, padded
-constexpr int kMfma16Cols = 16; // columns of the narrow variant
 constexpr float kPShift = 14.0f; // p is kept as 2^14 * exp2(logit - max): its half parts stay normal numbers
 
 // position of token offset o (0..15) inside its 16-token group of the transposed V tile:
@@ -200,6 +197,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
             const int pos = pa32 + i * kMfmaBlock;
 
             // ---- V: dequantise (hi + lo halves) and store transposed into the wave's LDS tile ----
+            wave_lds_handoff(); // every lane is past its reads of the previous block's tile
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const half2_t s01 = {vsc[u][0], vsc[u][1]}, s23 = {vsc[u][2], vsc[u][3]};
@@ -223,6 +221,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
                 }
             }
 
+            wave_lds_handoff(); // the tile is complete before any lane reads it
             // the raw registers are free again: the next block's bytes travel while this one is finished
             if (i + 1 < nb) {
                 if (pos + 2 * kMfmaBlock > pe32) clamp_offsets(pos + kMfmaBlock); // the next block is the last and partial
@@ -496,13 +495,16 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
                 for (int j = 0; j < 2; ++j) ksc[t][j] = *(const uint32_t*)(sk + (k_off[t] >> 3) + 8 * j);
         };
         // through the wave's LDS rows to the operand layout: lane (r16, qq) takes channels 64 j + 16 qq .. + 16 of the
-        // tokens r16 and 16 + r16 (the wave's LDS operations execute in order: no barrier)
+        // tokens r16 and 16 + r16 (the wave's LDS operations execute in order: no workgroup barrier, only the
+        // compiler is told about the hand-off)
         auto stage_k = [&]() {
+            wave_lds_handoff(); // every lane is past its reads of the previous block's rows
 #pragma unroll
             for (int i4 = 0; i4 < 4; ++i4) {
                 const int tk = 8 * i4 + (lane >> 3);
                 *(u32x4*)(sK + tk * D + ((((lane & 7) ^ tk ^ (tk >> 3)) & 7) << 4)) = kraw[i4];
             }
+            wave_lds_handoff(); // rows stored by eight lanes each, read back by the lanes that hold them as operands
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -540,6 +542,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
             // ---- V: dequantise (hi + lo halves) and store transposed into the wave's LDS tile ----
             // (8-byte stores of the two tiles pair up into one instruction; 16-byte stores of a channel's eight
             // tokens take the same time)
+            wave_lds_handoff(); // every lane is past its reads of the previous block's tile
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const half2_t s01 = {vsc[u][0], vsc[u][1]}, s23 = {vsc[u][2], vsc[u][3]};
@@ -563,6 +566,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
                 }
             }
 
+            wave_lds_handoff(); // the tile is complete before any lane reads it
             // the raw registers are free again: the next block's bytes travel while this one is finished
             if (i + 1 < nb) {
                 if (pos + 2 * kMfmaBlock > pe32) clamp_offsets(pos + kMfmaBlock); // the next block is the last and partial
@@ -696,56 +700,13 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
     }
 }
 
-// PMX_HIP_DECODE_MFMA=0 keeps these shapes on the VALU kernels (for comparisons)
-static bool mfma_kernel_enabled()
-{
-    static const bool on = [] {
-        const char* e = getenv("PMX_HIP_DECODE_MFMA");
-        return !(e && e[0] == '0');
-    }();
-    return on;
-}
-
-// PMX_HIP_DECODE_MFMA=32 runs every shape on the 32-column kernel (for comparisons)
-static bool wide_columns_forced()
-{
-    static const bool on = [] {
-        const char* e = getenv("PMX_HIP_DECODE_MFMA");
-        return e && e[0] == '3' && e[1] == '2';
-    }();
-    return on;
-}
-
-// kv heads per workgroup for a shape that these kernels serve
-int decode_mfma_kv_heads(int64_t num_kv_heads)
-{
-    return num_kv_heads % 4 == 0 ? 4 : (num_kv_heads % 2 == 0 ? 2 : 1);
-}
-
-// true when the variants above serve the shape (the plan chooses its grouping from the same test): five or more query
-// heads per kv head, and three or four with an odd number of kv heads (the others have decode_attn_quad.hip)
-bool decode_mfma_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads)
-{
-    if (!mfma_kernel_enabled() || decode_general_forced()) return false;
-    if (head_dim != kMfmaD || num_kv_heads <= 0 || num_heads % num_kv_heads != 0) return false;
-    const int64_t g = num_heads / num_kv_heads;
-    return g <= kMfmaCols && (g >= 5 || (g >= 3 && num_kv_heads % 2 != 0));
-}
-
-bool decode_mfma_applicable(const DecodeLaunch& a)
-{
-    return decode_mfma_shape(a.head_dim, a.num_heads, a.num_kv_heads) &&
-           a.kv_heads_per_group == decode_mfma_kv_heads(a.num_kv_heads) && a.num_passes == 1 &&
-           a.wg_tokens == kMfmaBlock && a.output_stride_s % 4 == 0 && (reinterpret_cast<uintptr_t>(a.output) & 7u) == 0;
-}
-
 template <int NW>
 static void launch_decode_mfma_nw(const DecodeLaunch& a, hipStream_t stream)
 {
     const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / NW), 1);
     const dim3 block(NW * kWave);
     const bool paged = a.cache_mode == 1, mask = a.attn_mask != nullptr;
-    if (a.num_kv_repeats <= kMfma16Cols && !wide_columns_forced()) {
+    if (a.kernel == kDecodeKernelMfma16) {
         if (paged) {
             if (mask) hipLaunchKernelGGL((decode_attention_mfma16_kernel<NW, true, true>), grid, block, 0, stream, a);
             else hipLaunchKernelGGL((decode_attention_mfma16_kernel<NW, true, false>), grid, block, 0, stream, a);
@@ -766,7 +727,7 @@ static void launch_decode_mfma_nw(const DecodeLaunch& a, hipStream_t stream)
 
 void launch_decode_mfma(const DecodeLaunch& a, hipStream_t stream)
 {
-    switch (decode_mfma_kv_heads(a.num_kv_heads)) {
+    switch (a.kv_heads_per_group) { // a wave per kv head
     case 4: launch_decode_mfma_nw<4>(a, stream); break;
     case 2: launch_decode_mfma_nw<2>(a, stream); break;
     default: launch_decode_mfma_nw<1>(a, stream); break;

@@ -36,7 +36,6 @@ namespace {
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
-constexpr int kQuadD = 128;
 constexpr int kQuadMaxHeads = 8; // kv heads per workgroup (two per wave): eight, or four or two when the kv heads do not come in eights
 constexpr int kQuadBlock = 16;  // tokens per block
 constexpr int kDppRor8 = 0x128; // row_ror:8 = lane ^ 8 inside a row of 16
@@ -502,46 +501,9 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
     }
 }
 
-// kv heads per workgroup for a shape that this kernel serves (a wave holds two kv heads of 128 channels, one of 256)
-int decode_quad_kv_heads(int64_t head_dim, int64_t num_kv_heads)
-{
-    const int per_wave = head_dim == 256 ? 1 : 2;
-    const int64_t pairs = num_kv_heads / per_wave;
-    return per_wave * (pairs % 4 == 0 ? 4 : (pairs % 2 == 0 ? 2 : 1));
-}
-
-// true when the variant above serves the shape: head_dim 128 with an even number of kv heads or head_dim 256, up to
-// four query heads per kv head (head_dim 128: up to eight with kv heads in eights; decode_attn_mfma.hip takes five and
-// more first).
 // One or two query heads per kv head leave rows of the 4x4x4 products and three quarters or half of the PV
 // arithmetic unused, but this kernel's row loads take the non-temporal hint, which the general kernel's cannot.
-bool decode_quad_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads)
-{
-    if (decode_general_forced()) return false;
-    if (num_kv_heads <= 0 || num_heads % num_kv_heads != 0) return false;
-    const int64_t g = num_heads / num_kv_heads;
-    if (head_dim == 256) return g <= 4;
-    if (head_dim != kQuadD || num_kv_heads % 2 != 0) return false;
-    return g <= 4 || (g <= 8 && num_kv_heads % 8 == 0);
-}
-
-// attn_mask: one set of waves only, and the mask's byte offsets inside a sequence's rows (heads x mask_stride_h, plus
-// a block) fit 32 bits
-bool decode_quad_mask_ok(int64_t num_heads, int64_t num_kv_repeats, int64_t mask_stride_h)
-{
-    if (num_kv_repeats > 4 || mask_stride_h < 0) return false;
-    return ((double)num_heads * (double)mask_stride_h + 64.0) * 2.0 < 4294967296.0;
-}
-
-// true when it serves the launch; the caller falls back to the general kernel otherwise
-bool decode_quad_applicable(const DecodeLaunch& a)
-{
-    if (!decode_quad_shape(a.head_dim, a.num_heads, a.num_kv_heads)) return false;
-    if (a.attn_mask != nullptr && !decode_quad_mask_ok(a.num_heads, a.num_kv_repeats, a.mask_stride_h)) return false;
-    return a.kv_heads_per_group == decode_quad_kv_heads(a.head_dim, a.num_kv_heads) && a.num_passes == 1 &&
-           a.wg_tokens == kQuadBlock && a.output_stride_s % 8 == 0 && (reinterpret_cast<uintptr_t>(a.output) & 15u) == 0;
-}
-
+// Which shapes come here is decided in decode_select.cpp.
 template <int WP, int HD>
 static void launch_decode_quad_wp(const DecodeLaunch& a, hipStream_t stream)
 {
@@ -565,7 +527,7 @@ void launch_decode_quad(const DecodeLaunch& a, hipStream_t stream)
         else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 2, 4, false, 128>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
         return;
     }
-    const int waves = decode_quad_kv_heads(a.head_dim, a.num_kv_heads) / (a.head_dim == 256 ? 1 : 2);
+    const int waves = a.kv_heads_per_group / (a.head_dim == 256 ? 1 : 2);
     if (a.head_dim == 256) {
         switch (waves) {
         case 4: launch_decode_quad_wp<4, 256>(a, stream); break;

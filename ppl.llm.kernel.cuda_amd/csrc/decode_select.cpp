@@ -1,0 +1,112 @@
+// Which kernel runs the token ranges of a decode step, and the grouping of heads and tokens it implies.
+// Host only.  The plan (pmxhip_decode_plan_make*) and the launch (pmxhip_decode_attention*) both come here, so
+// the unit of the range cuts that the token-range kernel uses is by construction the one the combine kernel uses.
+#include "launch_params.h"
+
+namespace pmxhip {
+
+namespace {
+
+int largest_pow2_divisor_upto(int64_t n, int cap)
+{
+    int r = 1;
+    while (r * 2 <= cap && n % (r * 2) == 0) r *= 2;
+    return r;
+}
+
+// head_dim 128 with an even number of kv heads, or head_dim 256: up to four query heads per kv head on one set of
+// waves; head_dim 128 with kv heads in eights: up to eight on two sets
+bool quad_serves(int64_t head_dim, int64_t g, int64_t num_kv_heads)
+{
+    if (head_dim == 256) return g <= 4;
+    if (head_dim != 128 || num_kv_heads % 2 != 0) return false;
+    return g <= 4 || (g <= 8 && num_kv_heads % 8 == 0);
+}
+
+} // namespace
+
+const char* decode_kernel_name(int32_t kernel)
+{
+    switch (kernel) {
+        case kDecodeKernelGeneral: return "decode_attention_kernel";
+        case kDecodeKernelQuad: return "decode_attention_quad_kernel";
+        case kDecodeKernelMfma16: return "decode_attention_mfma16_kernel";
+        case kDecodeKernelMfma32: return "decode_attention_mfma_kernel";
+        default: return "";
+    }
+}
+
+bool decode_choose(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, int32_t requested, DecodeChoice* out)
+{
+    if (head_dim != 64 && head_dim != 96 && head_dim != 128 && head_dim != 256) return false;
+    if (num_kv_heads <= 0 || num_heads <= 0 || num_heads % num_kv_heads != 0) return false;
+    const int64_t g = num_heads / num_kv_heads;
+    int32_t kernel = requested;
+    if (kernel == kDecodeKernelAuto) {
+        // Many query heads per kv head: their VALU arithmetic outweighs the cache stream, so they become MFMA
+        // columns (five and more; three and four as well where the kv heads do not come in pairs, which the quad
+        // kernel needs).  Up to four: the quad kernel, whose row loads stream whole lines.  Everything else
+        // (head_dim 64 and 96, odd kv-head counts with one or two query heads each, more than 32 query heads per
+        // kv head) stays on the general kernel.
+        if (head_dim == 128 && g <= kDecodeMfmaColumns && (g >= 5 || (g >= 3 && num_kv_heads % 2 != 0)))
+            kernel = g <= kDecodeMfma16Columns ? kDecodeKernelMfma16 : kDecodeKernelMfma32;
+        else if (quad_serves(head_dim, g, num_kv_heads) && g <= 4)
+            kernel = kDecodeKernelQuad;
+        else
+            kernel = kDecodeKernelGeneral;
+    }
+    DecodeChoice c{};
+    c.kernel = kernel;
+    switch (kernel) {
+        case kDecodeKernelGeneral: {
+            const int lanes_per_slot = head_dim == 64 ? 4 : (head_dim == 256 ? 16 : 8);
+            const int slots_per_wave = 64 / lanes_per_slot;
+            c.kv_heads_per_group = largest_pow2_divisor_upto(num_kv_heads, slots_per_wave < 8 ? slots_per_wave : 8);
+            int gt = 1;
+            while (gt < g && gt < 8) gt *= 2;
+            c.q_heads_per_pass = gt;
+            c.num_passes = (int32_t)((g + gt - 1) / gt);
+            c.wg_tokens = decode_wg_tokens((int)head_dim, c.kv_heads_per_group);
+            c.wgs_per_cu = 2;
+            break;
+        }
+        case kDecodeKernelQuad: {
+            if (!quad_serves(head_dim, g, num_kv_heads)) return false;
+            // a wave holds two kv heads of 128 channels or one of 256; four, two or one waves per set
+            const int per_wave = head_dim == 256 ? 1 : 2;
+            const int64_t pairs = num_kv_heads / per_wave;
+            c.kv_heads_per_group = per_wave * (pairs % 4 == 0 ? 4 : (pairs % 2 == 0 ? 2 : 1));
+            c.q_heads_per_pass = g <= 1 ? 1 : (g <= 2 ? 2 : (g <= 4 ? 4 : 8)); // rows of the 4x4x4 products in use
+            c.num_passes = 1;
+            c.wg_tokens = kDecodeQuadTokens;
+            c.wgs_per_cu = (head_dim == 256 ? 8 : 16) / c.kv_heads_per_group;
+            break;
+        }
+        case kDecodeKernelMfma16:
+        case kDecodeKernelMfma32: {
+            const int cols = kernel == kDecodeKernelMfma16 ? kDecodeMfma16Columns : kDecodeMfmaColumns;
+            if (head_dim != 128 || g > cols) return false;
+            c.kv_heads_per_group = num_kv_heads % 4 == 0 ? 4 : (num_kv_heads % 2 == 0 ? 2 : 1); // a wave per kv head
+            c.q_heads_per_pass = cols;
+            c.num_passes = 1;
+            c.wg_tokens = kDecodeMfmaTokens;
+            c.wgs_per_cu = kDecodeMfmaWavesPerCu / c.kv_heads_per_group;
+            break;
+        }
+        default: return false;
+    }
+    *out = c;
+    return true;
+}
+
+bool decode_quad_launch_ok(const DecodeLaunch& a)
+{
+    if (a.output_stride_s % 8 != 0 || (reinterpret_cast<uintptr_t>(a.output) & 15u) != 0) return false;
+    if (a.attn_mask != nullptr) {
+        if (a.num_kv_repeats > 4 || a.mask_stride_h < 0) return false;
+        if (((double)a.num_heads * (double)a.mask_stride_h + 64.0) * 2.0 >= 4294967296.0) return false;
+    }
+    return true;
+}
+
+} // namespace pmxhip

@@ -126,6 +126,16 @@ __device__ __forceinline__ float sub_half_hi(float p, half2_t h)
     return r;
 }
 
+// Hand-off of wave-private LDS data between the lanes of one wave: stores by some lanes, then loads of the same
+// bytes by others (or the reverse, before a tile is overwritten).  The wave's LDS operations execute in program
+// order, so the hardware needs nothing; the wavefront-scope fence keeps the compiler from moving the accesses
+// across this point (it emits no instruction), and the wave barrier keeps it from rescheduling around it.
+__device__ __forceinline__ void wave_lds_handoff()
+{
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
 // Index arrays (kvstarts, cachestarts) are read-only for the whole launch and are read at
 // wave-uniform addresses: viewing them through the constant address space lets the compiler use
 // scalar loads (scalar cache, no vector registers, no vector wait count) for them.

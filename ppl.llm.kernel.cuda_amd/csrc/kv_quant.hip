@@ -253,17 +253,17 @@ int launch_rope(const RopeLaunch& a, hipStream_t stream)
     return 0;
 }
 
-int launch_kv_quantize(const QuantLaunch& a, hipStream_t stream)
+int launch_kv_quantize(const QuantLaunch& a, int compute_units, hipStream_t stream)
 {
     const int64_t groups_per_token = (int64_t)a.num_kv_heads * (a.head_dim >> 3);
     const int64_t max_units = a.max_tokens * groups_per_token;
     if (max_units <= 0) return 0;
     int64_t blocks = (max_units + kQuantThreads - 1) / kQuantThreads;
-    // grid-stride beyond this: eight workgroups per CU of a 256-CU part hold every wave slot at once, and a lane then
-    // takes two or three units in turn (11 104 new tokens of 8 heads x 128 channels: 23.4 us against 28 us with four
+    // grid-stride beyond this: eight workgroups per CU hold every wave slot at once, and a lane then takes two or
+    // three units in turn (11 104 new tokens of 8 heads x 128 channels on 256 CUs: 23.4 us against 28 us with four
     // times as many workgroups and one unit per lane, 36 us with 32 times as many, most of them without a unit;
     // 25 us with half as many)
-    const int64_t cap = 256 * 8;
+    const int64_t cap = (int64_t)(compute_units > 0 ? compute_units : 256) * 8;
     if (blocks > cap) blocks = cap;
     if (a.cache_mode == 1)
         hipLaunchKernelGGL(kv_quantize_kernel<true>, dim3((unsigned)blocks), dim3(kQuantThreads), 0, stream, a);

@@ -6,6 +6,8 @@
 #include <hip/hip_runtime_api.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace pmxhip {
 
 struct QuantLaunch {
@@ -62,8 +64,10 @@ struct DecodeLaunch {
     int32_t kv_heads_per_group;   // kv heads per workgroup (power of two)
     int32_t q_heads_per_pass;     // GT
     int32_t num_passes;           // ceil(num_kv_repeats / GT)
-    int32_t wg_tokens;            // tokens one workgroup iteration covers
+    int32_t wg_tokens;            // tokens one workgroup iteration covers: the unit of the range cuts, a property
+                                  // of the kernel named by `kernel` (the combine kernel derives the same cuts from it)
     int32_t min_tokens_per_range;
+    int32_t kernel;               // DecodeKernel that runs the token ranges; never kDecodeKernelAuto at launch
 };
 
 struct PrefillLaunch {
@@ -142,26 +146,67 @@ struct RopeLaunch {
     int32_t cache_mode;
 };
 
-int launch_kv_quantize(const QuantLaunch& a, hipStream_t stream);
+// Return codes of the launchers below.
+constexpr int kLaunchOk = 0;
+constexpr int kLaunchNoKernel = 1;      // no kernel serves the shape
+constexpr int kLaunchNeedsWarmup = 2;   // the kernel's one-time attribute call is due, but the stream is being captured
+
+// The one-time hipFuncSetAttribute of a kernel whose dynamic LDS exceeds the default limit.  It runs before the
+// kernel's first launch in the process (one GPU per process) and never while `stream` is being captured into a
+// graph: a caller that captures first gets kLaunchNeedsWarmup and calls pmxhip_init() or one eager step before.
+inline int ensure_dynamic_lds(const void* kernel, int bytes, hipStream_t stream, std::atomic<int>& ready)
+{
+    if (ready.load(std::memory_order_acquire) != 0) return kLaunchOk;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &st) != hipSuccess || st != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return kLaunchNeedsWarmup;
+    }
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return kLaunchNoKernel;
+    ready.store(1, std::memory_order_release);
+    return kLaunchOk;
+}
+
+int launch_kv_quantize(const QuantLaunch& a, int compute_units, hipStream_t stream);
 int launch_rope(const RopeLaunch& a, hipStream_t stream);
 void launch_page_copy(const PageCopyLaunch& a, hipStream_t stream);
 int launch_decode(const DecodeLaunch& a, int stage, hipStream_t stream); // stage: 0 both, 1 ranges, 2 combine
-int decode_wg_tokens(int head_dim, int kv_heads_per_group);
-bool decode_general_forced(); // PMX_HIP_DECODE_GENERAL=1 in the environment: every shape on the general kernel
-bool decode_quad_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads); // head_dim 128 (even number of kv heads) or 256, <= 4 query heads each
-int decode_quad_kv_heads(int64_t head_dim, int64_t num_kv_heads);                  // kv heads per workgroup: 8, 4 or 2 (head_dim 256: 4, 2 or 1)
-bool decode_quad_mask_ok(int64_t num_heads, int64_t num_kv_repeats, int64_t mask_stride_h); // attn_mask within its reach
-bool decode_quad_applicable(const DecodeLaunch& a);
+
+// ---- which kernel runs the token ranges of a decode step (decode_select.cpp; host only) ----
+// The values are those of pmxhip_decode_kernel_t in the C header.
+enum DecodeKernel : int32_t {
+    kDecodeKernelAuto = 0,    // as a request: by shape
+    kDecodeKernelGeneral = 1, // decode_attn.hip: VALU, every head_dim and head count, up to 8 query heads per pass
+    kDecodeKernelQuad = 2,    // decode_attn_quad.hip: 4x4x4 MFMA per quad; head_dim 128 (even number of kv heads) or 256
+    kDecodeKernelMfma16 = 3,  // decode_attn_mfma.hip: 16 query-head columns, head_dim 128
+    kDecodeKernelMfma32 = 4,  // decode_attn_mfma.hip: 32 query-head columns, head_dim 128
+};
+struct DecodeChoice {
+    int32_t kernel;             // never kDecodeKernelAuto
+    int32_t kv_heads_per_group; // kv heads one workgroup serves
+    int32_t q_heads_per_pass;   // query heads per kv head served by one pass (general kernel: 1, 2, 4 or 8)
+    int32_t num_passes;
+    int32_t wg_tokens;          // tokens per workgroup iteration = unit of the range cuts
+    int32_t wgs_per_cu;         // workgroups that a CU holds at once (sizes the number of ranges)
+};
+// The kernel that serves a shape, and the grouping it implies.  `requested` kDecodeKernelAuto picks by shape;
+// any other value insists on that kernel and the call fails (false) when it cannot serve the shape.
+bool decode_choose(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, int32_t requested, DecodeChoice* out);
+// What the quad kernel needs of a launch beyond the C ABI's own checks: 16-byte aligned output rows and,
+// with attn_mask, one set of waves and mask offsets within 32 bits.
+bool decode_quad_launch_ok(const DecodeLaunch& a);
+const char* decode_kernel_name(int32_t kernel);
+int decode_wg_tokens(int head_dim, int kv_heads_per_group); // of the general kernel
 constexpr int kDecodeQuadTokens = 16;
-void launch_decode_quad(const DecodeLaunch& a, hipStream_t stream);
-// head_dim 128, 5 to 32 query heads per kv head, kv heads in fours: MFMA kernel, groups of four kv heads, 32-token blocks
-bool decode_mfma_shape(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads);
-bool decode_mfma_applicable(const DecodeLaunch& a);
-void launch_decode_mfma(const DecodeLaunch& a, hipStream_t stream);
-int decode_mfma_kv_heads(int64_t num_kv_heads); // kv heads (= waves) per workgroup: 4, 2 or 1
-constexpr int kDecodeMfmaWavesPerCu = 8;         // 16 KB of LDS per wave
+constexpr int kDecodeMfmaWavesPerCu = 8; // 20 KB of LDS per wave
 constexpr int kDecodeMfmaTokens = 32;
+constexpr int kDecodeMfma16Columns = 16;
 constexpr int kDecodeMfmaColumns = 32;
+void launch_decode_quad(const DecodeLaunch& a, hipStream_t stream);
+void launch_decode_mfma(const DecodeLaunch& a, hipStream_t stream);
+// One-time attribute calls of the kernels whose dynamic LDS exceeds the default limit, all variants at once.
+int init_decode_kernels();
+int init_prefill_kernels();
 void launch_splitkv_combine_rows(const float* partial_out, const float* partial_ml, const int64_t* piece_begin,
                                  const int64_t* piece_end, int64_t rows, int64_t head_dim, void* output,
                                  hipStream_t stream);

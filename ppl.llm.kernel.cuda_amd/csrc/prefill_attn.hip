@@ -621,20 +621,34 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     }
 }
 
-template <int D, int SRC, bool EXTRA>
-static void launch_prefill_variant(const PrefillLaunch& a, dim3 grid, hipStream_t stream)
+template <int D, int SRC>
+constexpr size_t prefill_lds_bytes()
 {
     // int8 source: K hi/lo tiles + transposed V hi/lo tiles (above the 64 KB static limit for D = 128, hence
     // dynamic); fp16 source: one K tile and one transposed V tile; two buffers of each
-    constexpr size_t lds_bytes = 2 * (SRC == 2 ? 1 : 2) * (kBN * (D + 8) + D * (kBN + 8)) * sizeof(half_t); // two tile buffers
-    static const hipError_t once = hipFuncSetAttribute((const void*)prefill_attention_kernel<D, SRC, EXTRA>,
-                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    (void)once;
+    return 2 * (SRC == 2 ? 1 : 2) * (kBN * (D + 8) + D * (kBN + 8)) * sizeof(half_t);
+}
+
+template <int D, int SRC, bool EXTRA>
+static std::atomic<int>& prefill_variant_ready()
+{
+    static std::atomic<int> ready{0};
+    return ready;
+}
+
+template <int D, int SRC, bool EXTRA>
+static int launch_prefill_variant(const PrefillLaunch& a, dim3 grid, hipStream_t stream)
+{
+    constexpr size_t lds_bytes = prefill_lds_bytes<D, SRC>();
+    if (int rc = ensure_dynamic_lds((const void*)prefill_attention_kernel<D, SRC, EXTRA>, (int)lds_bytes, stream,
+                                    prefill_variant_ready<D, SRC, EXTRA>()))
+        return rc;
     hipLaunchKernelGGL((prefill_attention_kernel<D, SRC, EXTRA>), grid, dim3(kPrefillThreads), lds_bytes, stream, a);
+    return kLaunchOk;
 }
 
 template <int D>
-static void launch_prefill_d(const PrefillLaunch& a, hipStream_t stream)
+static int launch_prefill_d(const PrefillLaunch& a, hipStream_t stream)
 {
     const int G = (int)(a.num_heads / a.num_kv_heads);
     const int ppw = kCols / G > 0 ? kCols / G : 1;
@@ -649,24 +663,50 @@ static void launch_prefill_d(const PrefillLaunch& a, hipStream_t stream)
     const bool extra = a.attn_mask != nullptr || a.alibi_slopes != nullptr;
     const int src = a.current_key ? 2 : (a.cache_mode == 1 ? 0 : 1);
     if (extra) {
-        if (src == 0) launch_prefill_variant<D, 0, true>(a, grid, stream);
-        else if (src == 1) launch_prefill_variant<D, 1, true>(a, grid, stream);
-        else launch_prefill_variant<D, 2, true>(a, grid, stream);
-    } else {
-        if (src == 0) launch_prefill_variant<D, 0, false>(a, grid, stream);
-        else if (src == 1) launch_prefill_variant<D, 1, false>(a, grid, stream);
-        else launch_prefill_variant<D, 2, false>(a, grid, stream);
+        if (src == 0) return launch_prefill_variant<D, 0, true>(a, grid, stream);
+        if (src == 1) return launch_prefill_variant<D, 1, true>(a, grid, stream);
+        return launch_prefill_variant<D, 2, true>(a, grid, stream);
     }
+    if (src == 0) return launch_prefill_variant<D, 0, false>(a, grid, stream);
+    if (src == 1) return launch_prefill_variant<D, 1, false>(a, grid, stream);
+    return launch_prefill_variant<D, 2, false>(a, grid, stream);
 }
 
 int launch_prefill(const PrefillLaunch& a, hipStream_t stream)
 {
-    if (a.num_heads / a.num_kv_heads > kCols) return 1;
+    if (a.num_heads / a.num_kv_heads > kCols) return kLaunchNoKernel;
     switch (a.head_dim) {
-        case 64: launch_prefill_d<64>(a, stream); return 0;
-        case 128: launch_prefill_d<128>(a, stream); return 0;
-        default: return 1;
+        case 64: return launch_prefill_d<64>(a, stream);
+        case 128: return launch_prefill_d<128>(a, stream);
+        default: return kLaunchNoKernel;
     }
+}
+
+template <int D, int SRC, bool EXTRA>
+static int init_prefill_variant()
+{
+    std::atomic<int>& ready = prefill_variant_ready<D, SRC, EXTRA>();
+    if (ready.load() != 0) return kLaunchOk;
+    if (hipFuncSetAttribute((const void*)prefill_attention_kernel<D, SRC, EXTRA>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)prefill_lds_bytes<D, SRC>()) != hipSuccess)
+        return kLaunchNoKernel;
+    ready.store(1);
+    return kLaunchOk;
+}
+template <int D>
+static int init_prefill_d()
+{
+    if (int rc = init_prefill_variant<D, 0, false>()) return rc;
+    if (int rc = init_prefill_variant<D, 0, true>()) return rc;
+    if (int rc = init_prefill_variant<D, 1, false>()) return rc;
+    if (int rc = init_prefill_variant<D, 1, true>()) return rc;
+    if (int rc = init_prefill_variant<D, 2, false>()) return rc;
+    return init_prefill_variant<D, 2, true>();
+}
+int init_prefill_kernels()
+{
+    if (int rc = init_prefill_d<64>()) return rc;
+    return init_prefill_d<128>();
 }
 
 } // namespace pmxhip

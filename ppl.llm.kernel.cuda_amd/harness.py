@@ -108,19 +108,25 @@ class DeviceBatch:
         return op
 
     def decode_only(self, num_token_ranges=0, workspace=None, attn_mask=None, mask_stride_s=0, mask_stride_h=0,
-                    output=None, stage=0):
-        """Decode attention through the flat C entry point (no operator object)."""
+                    output=None, stage=0, kernel=0, output_stride_s=None, name_only=False,
+                    stream=None):
+        """Decode attention through the flat C entry point (no operator object).  `kernel` requests a
+        token-range kernel; `name_only`
+        launches nothing and returns the name of the kernel the call would run."""
         bt = self.bt
         plan = ops.decode_plan(bt.decoding_batches, bt.num_heads, bt.num_kv_heads, bt.head_dim, bt.max_kvlen,
-                               ranges_hint=num_token_ranges)
-        if workspace is None and plan.workspace_size > 0:
+                               ranges_hint=num_token_ranges, kernel=kernel)
+        if workspace is None and plan.workspace_size > 0 and not name_only:
             workspace = torch.empty(int(plan.workspace_size), dtype=torch.uint8, device=self.device)
         out = self.output if output is None else output
-        ops.decode_attention(self.query, out, self.cache, self.scale, self.cachestarts, self.kvstarts,
-                             attn_scale=bt.attn_scale, layer_idx=bt.layer_idx,
-                             decoding_batches=bt.decoding_batches, num_heads=bt.num_heads,
-                             num_kv_heads=bt.num_kv_heads, head_dim=bt.head_dim,
-                             num_token_ranges=plan.num_token_ranges, workspace=workspace,
-                             attn_mask=attn_mask, mask_stride_s=mask_stride_s, mask_stride_h=mask_stride_h, stage=stage,
-                             **self.layout_kwargs())
+        r = ops.decode_attention(self.query, out, self.cache, self.scale, self.cachestarts, self.kvstarts,
+                                 attn_scale=bt.attn_scale, layer_idx=bt.layer_idx,
+                                 decoding_batches=bt.decoding_batches, num_heads=bt.num_heads,
+                                 num_kv_heads=bt.num_kv_heads, head_dim=bt.head_dim,
+                                 num_token_ranges=plan.num_token_ranges, workspace=workspace,
+                                 attn_mask=attn_mask, mask_stride_s=mask_stride_s, mask_stride_h=mask_stride_h, stage=stage,
+                                 kernel=kernel, output_stride_s=output_stride_s,
+                                 name_only=name_only, stream=stream, **self.layout_kwargs())
+        if name_only:
+            return r
         return plan, workspace

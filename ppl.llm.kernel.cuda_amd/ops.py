@@ -84,10 +84,20 @@ def key_value_cache(current_key, current_value, seqstarts, cachestarts, start_po
     return rc
 
 
-def decode_plan(decoding_batches, num_heads, num_kv_heads, head_dim, max_kvlen, cus=None, ranges_hint=0):
+def init():
+    """The library's one-time set-up on the current device (needed only before a first step under stream capture)."""
+    rc = _lib.lib().pmxhip_init()
+    if rc != RC_SUCCESS:
+        raise PmxError(rc, "init")
+    return rc
+
+
+def decode_plan(decoding_batches, num_heads, num_kv_heads, head_dim, max_kvlen, cus=None, ranges_hint=0, kernel=0):
+    """The split plan of a decode step; `kernel` requests a token-range kernel (0 = chosen by shape)."""
     plan = DecodePlan()
-    rc = _lib.lib().pmxhip_decode_plan_make(decoding_batches, num_heads, num_kv_heads, head_dim, max_kvlen,
-                                            compute_units() if cus is None else cus, ranges_hint, ctypes.byref(plan))
+    rc = _lib.lib().pmxhip_decode_plan_make_kernel(decoding_batches, num_heads, num_kv_heads, head_dim, max_kvlen,
+                                                   compute_units() if cus is None else cus, ranges_hint, kernel,
+                                                   ctypes.byref(plan))
     if rc != RC_SUCCESS:
         raise PmxError(rc, "decode_plan")
     return plan
@@ -97,8 +107,10 @@ def decode_attention(query, output, cache, scale, cachestarts, kvstarts, *, attn
                      decoding_batches, num_heads, num_kv_heads, head_dim, cache_mode, page_size,
                      cache_stride_s, cache_stride_l, cache_stride_h, cache_stride_kv, cachestarts_stride_b,
                      num_token_ranges, workspace=None, attn_mask=None, mask_stride_s=0, mask_stride_h=0,
-                     stage=0, stream=None, check=True):
-    """Decode attention of sequences [0, decoding_batches); output fp16 [B_dec, Hq, D]."""
+                     stage=0, stream=None, check=True, kernel=0, output_stride_s=None,
+                     name_only=False):
+    """Decode attention of sequences [0, decoding_batches); output fp16 [B_dec, Hq, D].
+    `kernel` requests a token-range kernel; `name_only` launches nothing and returns the kernel's name."""
     p = DecodeParams()
     p.query = _ptr(query)
     p.attn_mask = _ptr(attn_mask)
@@ -112,7 +124,7 @@ def decode_attention(query, output, cache, scale, cachestarts, kvstarts, *, attn
     p.num_kv_repeats = num_heads // num_kv_heads if num_kv_heads else 0
     p.page_size = page_size
     p.query_stride_s = num_heads * head_dim
-    p.output_stride_s = num_heads * head_dim
+    p.output_stride_s = num_heads * head_dim if output_stride_s is None else output_stride_s
     p.mask_stride_s = mask_stride_s
     p.mask_stride_h = mask_stride_h
     p.cache_stride_s = cache_stride_s
@@ -128,6 +140,9 @@ def decode_attention(query, output, cache, scale, cachestarts, kvstarts, *, attn
     p.num_token_ranges = num_token_ranges
     p.workspace = _ptr(workspace)
     p.workspace_size = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    p.kernel_request = kernel
+    if name_only:
+        return _lib.lib().pmxhip_decode_kernel_name(ctypes.byref(p)).decode()
     rc = _lib.lib().pmxhip_decode_attention_stage(ctypes.byref(p), stage, _stream(stream))
     if check and rc != RC_SUCCESS:
         raise PmxError(rc, "decode_attention")

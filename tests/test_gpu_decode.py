@@ -60,6 +60,60 @@ def test_decode_matches_oracle(pkg, oracle, shape, cache_mode):
         assert_attention_close(got, ref, "shape %s mode %d ranges %d" % (shape, cache_mode, plan.num_token_ranges))
 
 
+KERNEL_NAMES = {1: "decode_attention_kernel", 2: "decode_attention_quad_kernel",
+                3: "decode_attention_mfma16_kernel", 4: "decode_attention_mfma_kernel"}
+
+
+@pytest.mark.parametrize("shape,kernels", [
+    ((32, 8, 128), (1, 2, 3, 4)),   # Llama-3-8B: every kernel serves it
+    ((64, 8, 128), (1, 2, 3, 4)),   # 8 query heads per kv head: the quad kernel runs two sets of waves
+    ((8, 8, 128), (1, 2, 3)),
+    ((12, 2, 128), (1, 3, 4)),
+    ((96, 4, 128), (1, 4)),         # 24 per kv head: three passes of the general kernel, or 32 columns
+    ((16, 8, 256), (1, 2)),
+    ((6, 3, 128), (1, 3)),
+])
+def test_decode_requested_kernel(pkg, oracle, shape, kernels):
+    """Every token-range kernel that serves a shape, requested through the C ABI: the library reports that it
+    runs, and the result is the oracle's whatever the split."""
+    hq, hkv, d = shape
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 400 + hq + d, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                         cache_mode=1, dec_kv_lens=[1, 300, 17, 129, 640, 2, 128], outliers=True)
+    ref = oracle_decode(oracle, bt, q, cache, scale)
+    for k in kernels:
+        assert dev.decode_only(kernel=k, name_only=True) == KERNEL_NAMES[k]
+        for ranges in (1, 0, 5):
+            got, plan = run_decode(dev, ranges, kernel=k)
+            assert plan.kernel == k
+            assert_attention_close(got, ref, "shape %s kernel %d ranges %d" % (shape, k, plan.num_token_ranges))
+
+
+@pytest.mark.parametrize("shape", [(16, 4, 128), (8, 2, 128), (12, 6, 128), (8, 4, 256)])
+def test_decode_output_rows_aligned_to_8_bytes_only(pkg, oracle, shape):
+    """The C ABI admits output rows that are 8-byte aligned; the quad kernel needs 16.  Such a call runs on the
+    general kernel, and the token-range kernel and the combine kernel must then cut the ranges by the same unit
+    (several ranges, so that sequences are split into pieces)."""
+    hq, hkv, d = shape
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 450 + hq + d, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                         cache_mode=1, dec_kv_lens=[900, 300, 17, 129, 640, 2, 128], outliers=True)
+    ref = oracle_decode(oracle, bt, q, cache, scale)
+    assert dev.decode_only(name_only=True) == "decode_attention_quad_kernel"
+    n = bt.decoding_batches * hq * d
+    buf = torch.full((n + 8,), float("nan"), dtype=torch.float16, device="cuda")
+    out = buf[4:4 + n].view(bt.decoding_batches, hq, d)
+    assert out.data_ptr() % 16 == 8
+    assert dev.decode_only(output=out, name_only=True) == "decode_attention_kernel"
+    for ranges in (1, 0, 3, 11, 40):
+        out.fill_(float("nan"))
+        plan, _ = dev.decode_only(num_token_ranges=ranges, output=out)
+        torch.cuda.synchronize()
+        assert_attention_close(out.float().cpu().numpy(), ref, "shape %s ranges %d" % (shape, plan.num_token_ranges))
+    assert torch.isnan(buf[:4]).all() and torch.isnan(buf[4 + n:]).all()
+    # insisting on the quad kernel for these rows is refused, not silently served by another kernel
+    with pytest.raises(pkg.ops.PmxError):
+        dev.decode_only(output=out, kernel=2)
+
+
 def test_decode_c1_golden_shape(pkg, oracle):
     bt, rng = pkg.workloads.make_batch("C1")
     cache, scale = host_cache(bt)

@@ -106,6 +106,17 @@ def test_forward_in_a_hip_graph(pkg, oracle):
     assert_attention_close(eager.float().cpu().numpy(), ref, "eager rows")
 
 
+def test_first_step_under_capture():
+    """In a fresh process: a first forward() under stream capture is refused with a message that names
+    pmxhip_init(), and after that call the capture succeeds (tests/capture_first_child.py)."""
+    import os
+    import subprocess
+    import sys
+    child = os.path.join(os.path.dirname(os.path.abspath(__file__)), "capture_first_child.py")
+    r = subprocess.run([sys.executable, "-u", child], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.strip().endswith("OK"), r.stdout[-2000:] + r.stderr[-2000:]
+
+
 def test_contiguous_mode_and_stagewise_calls(pkg, oracle):
     bt, rng = pkg.workloads.custom_batch(402, num_heads=8, num_kv_heads=8, head_dim=64, cache_mode=0,
                                          dec_kv_lens=[200, 31], prefill_q_lens=[40], prefill_prior=[9])

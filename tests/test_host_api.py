@@ -74,6 +74,11 @@ def test_prepare_derives_the_reference_values(pkg, hip_lib):
     (dict(specify_decoding_multi_block=-1), 4),
     (dict(specify_decoding_tpb=128), 4),
     (dict(enable_sharemem_mhca=False, enable_infinity_mhca=False, enable_infinity_gqca=False), 1),  # no algorithm
+    # prefill sequences at a head_dim the prefill stage does not have: refused before anything is enqueued
+    (dict(batch=9, decoding_batches=6, max_seqlen=40, head_dim=256, query_shape=(90, 32, 256),
+          current_key_shape=(90, 8, 256), current_value_shape=(90, 8, 256), output_shape=(90, 32, 256)), 2),
+    (dict(batch=9, decoding_batches=6, max_seqlen=40, head_dim=96, query_shape=(90, 32, 96),
+          current_key_shape=(90, 8, 96), current_value_shape=(90, 8, 96), output_shape=(90, 32, 96)), 2),
 ])
 def test_prepare_error_branches(pkg, hip_lib, over, code):
     _, rc = prepare(pkg, **over)
@@ -83,7 +88,12 @@ def test_prepare_error_branches(pkg, hip_lib, over, code):
 def test_prepare_accepts_what_the_reference_accepts(pkg, hip_lib):
     for over in (dict(specify_decoding_tpb=256), dict(specify_decoding_tpb=512), dict(cache_mode=0, page_size=0),
                  dict(enable_infinity_gqca=False), dict(enable_sharemem_mhca=False),
-                 dict(specify_decoding_multi_block=0), dict(specify_decoding_multi_block=2)):
+                 dict(specify_decoding_multi_block=0), dict(specify_decoding_multi_block=2),
+                 # decode-only batches take every head_dim of the decode kernels
+                 dict(head_dim=256, query_shape=(6, 32, 256), current_key_shape=(6, 8, 256),
+                      current_value_shape=(6, 8, 256), output_shape=(6, 32, 256)),
+                 dict(head_dim=96, query_shape=(6, 32, 96), current_key_shape=(6, 8, 96),
+                      current_value_shape=(6, 8, 96), output_shape=(6, 32, 96))):
         op, rc = prepare(pkg, **over)
         assert rc == 0, over
     op, _ = prepare(pkg, specify_decoding_multi_block=0)
@@ -113,13 +123,13 @@ def test_decode_plan(pkg, hip_lib):
     assert plan.partial_out_size == pieces * 32 * 128 * 4 and plan.partial_ml_size == pieces * 32 * 2 * 4
     plan = pkg.ops.decode_plan(64, 32, 32, 128, 4096, cus=256)  # MHA: 4 groups of 8 kv heads
     assert plan.kv_heads_per_group == 8 and plan.q_heads_per_pass == 1 and plan.num_token_ranges == 128
-    plan = pkg.ops.decode_plan(32, 64, 8, 128, 32768, cus=256)  # G = 8: MFMA kernel, 4 kv heads per workgroup, 32 columns
-    assert plan.q_heads_per_pass == 32 and plan.num_passes == 1 and plan.kv_heads_per_group == 4
+    plan = pkg.ops.decode_plan(32, 64, 8, 128, 32768, cus=256)  # G = 8: MFMA kernel, 4 kv heads per workgroup, 16 columns
+    assert plan.q_heads_per_pass == 16 and plan.num_passes == 1 and plan.kv_heads_per_group == 4
     assert plan.num_token_ranges == 256
     plan = pkg.ops.decode_plan(64, 8, 1, 128, 8192, cus=256)  # one kv head: one wave per workgroup, eight workgroups per CU
-    assert plan.q_heads_per_pass == 32 and plan.kv_heads_per_group == 1 and plan.num_token_ranges == 2048
+    assert plan.q_heads_per_pass == 16 and plan.kv_heads_per_group == 1 and plan.num_token_ranges == 2048
     plan = pkg.ops.decode_plan(64, 16, 2, 128, 8192, cus=256)
-    assert plan.q_heads_per_pass == 32 and plan.kv_heads_per_group == 2 and plan.num_token_ranges == 1024
+    assert plan.q_heads_per_pass == 16 and plan.kv_heads_per_group == 2 and plan.num_token_ranges == 1024
     plan = pkg.ops.decode_plan(64, 16, 4, 128, 8192, cus=256)  # four kv heads: two waves per workgroup, four workgroups per CU
     assert plan.q_heads_per_pass == 4 and plan.kv_heads_per_group == 4 and plan.num_token_ranges == 1024
     plan = pkg.ops.decode_plan(4, 48, 3, 64, 512, cus=256)  # G = 16 -> two passes of 8; 3 kv heads -> 1 per group
@@ -132,6 +142,27 @@ def test_decode_plan(pkg, hip_lib):
         pkg.ops.decode_plan(4, 8, 8, 80, 512, cus=256)  # head_dim 80
     with pytest.raises(pkg.ops.PmxError):
         pkg.ops.decode_plan(4, 9, 8, 64, 512, cus=256)
+
+
+def test_decode_plan_names_its_kernel(pkg, hip_lib):
+    """The plan reports the token-range kernel it was made for, and a requested kernel is honoured or refused."""
+    L = pkg._lib
+    auto = {(32, 8, 128): L.DECODE_KERNEL_QUAD, (32, 32, 128): L.DECODE_KERNEL_QUAD, (64, 8, 128): L.DECODE_KERNEL_MFMA16,
+            (96, 4, 128): L.DECODE_KERNEL_MFMA32, (9, 3, 128): L.DECODE_KERNEL_MFMA16, (6, 3, 128): L.DECODE_KERNEL_GENERAL,
+            (8, 8, 64): L.DECODE_KERNEL_GENERAL, (12, 4, 96): L.DECODE_KERNEL_GENERAL, (16, 16, 256): L.DECODE_KERNEL_QUAD,
+            (40, 8, 256): L.DECODE_KERNEL_GENERAL, (66, 2, 128): L.DECODE_KERNEL_GENERAL}
+    for (hq, hkv, d), want in auto.items():
+        assert pkg.ops.decode_plan(16, hq, hkv, d, 4096, cus=256).kernel == want, (hq, hkv, d)
+    # requests: every kernel on the Llama-3-70B shape (8 query heads per kv head, kv heads in eights)
+    for k, (kvhb, gt, ranges) in {L.DECODE_KERNEL_GENERAL: (8, 8, 512), L.DECODE_KERNEL_QUAD: (8, 8, 512),
+                                  L.DECODE_KERNEL_MFMA16: (4, 16, 256), L.DECODE_KERNEL_MFMA32: (4, 32, 256)}.items():
+        plan = pkg.ops.decode_plan(32, 64, 8, 128, 32768, cus=256, kernel=k)
+        assert (plan.kernel, plan.kv_heads_per_group, plan.q_heads_per_pass, plan.num_token_ranges) == (k, kvhb, gt, ranges)
+    for hq, hkv, d, k in [(32, 8, 64, L.DECODE_KERNEL_QUAD), (32, 8, 64, L.DECODE_KERNEL_MFMA16),
+                          (40, 2, 128, L.DECODE_KERNEL_MFMA16), (66, 2, 128, L.DECODE_KERNEL_MFMA32),
+                          (10, 2, 128, L.DECODE_KERNEL_QUAD), (3, 3, 128, L.DECODE_KERNEL_QUAD), (32, 8, 128, 5), (32, 8, 128, -1)]:
+        with pytest.raises(pkg.ops.PmxError):
+            pkg.ops.decode_plan(16, hq, hkv, d, 4096, cus=256, kernel=k)
 
 
 def test_c_entry_points_reject_bad_arguments_without_launching(pkg, hip_lib):
