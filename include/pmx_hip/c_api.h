@@ -173,6 +173,20 @@ PMXHIP_API int pmxhip_decode_attention(const pmxhip_decode_params* p, pmxhip_str
  * decode_attention_mfma_kernel -- the names a profiler's kernel trace shows.  Host only, launches nothing. */
 PMXHIP_API const char* pmxhip_decode_kernel_name(const pmxhip_decode_params* p);
 
+/* pmxhip_decode_attention for callers that cannot allocate: it has no counterpart in the reference, whose caller
+ * always sizes and passes cfg.workspace (multi_head_cache_attention.h:104-106).  It is for code that must not
+ * call hipMalloc -- a step recorded under HIP graph capture, a serving loop or harness that forbids allocation:
+ * p->workspace and p->workspace_size are ignored and the split-KV pieces go to a static array of
+ * PMXHIP_STATIC_WORKSPACE_BYTES inside the library (one per GPU, held until the process ends).  The call
+ * allocates and frees nothing.  A step whose pieces need more -- (num_token_ranges + decoding_batches) *
+ * num_heads * (head_dim + 2) * 4 bytes -- is rejected with PMXHIP_INVALID_VALUE.  All calls on one GPU share the
+ * array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream are safe.  Nothing in
+ * the array needs clearing between calls: a piece is read back only by the step that wrote it.  The first call
+ * on a device resolves the array's address (hipGetSymbolAddress); under stream capture do that beforehand with
+ * pmxhip_init(). */
+#define PMXHIP_STATIC_WORKSPACE_BYTES (32 * 1024 * 1024)
+PMXHIP_API int pmxhip_decode_attention_static(const pmxhip_decode_params* p, pmxhip_stream_t stream);
+
 /* The same step split at its kernel boundary, for callers that time or overlap
  * the two kernels: stage 1 = the token-range kernel only (final rows of
  * sequences that fit one range, float32 pieces of the others), stage 2 = the
@@ -427,7 +441,7 @@ PMXHIP_API int pmxhip_rope_kv_cache_quantize(const pmxhip_rope_params* rope, con
 
 /* One-time set-up on the current device, for callers that record their first step under stream capture: the
  * attribute calls of the kernels with large dynamic LDS (otherwise made at each kernel's first launch, which a
- * capturing stream refuses with PMXHIP_OTHER_ERROR).  Optional
+ * capturing stream refuses with PMXHIP_OTHER_ERROR) and the address of the static workspace.  Optional
  * otherwise; idempotent; host only.  No counterpart in the reference, whose cudaFuncSetAttribute calls sit in
  * its launch path (kernel.cu:1946). */
 PMXHIP_API int pmxhip_init(void);

@@ -25,7 +25,7 @@ EXPORTED_SYMBOLS = (
     "pmxhip_kv_cache_quantize", "pmxhip_key_value_cache",
     "pmxhip_init",
     "pmxhip_decode_plan_make", "pmxhip_decode_plan_make_kernel", "pmxhip_decode_attention",
-    "pmxhip_decode_attention_stage", "pmxhip_decode_kernel_name",
+    "pmxhip_decode_attention_stage", "pmxhip_decode_attention_static", "pmxhip_decode_kernel_name",
     "pmxhip_splitkv_combine",
     "pmxhip_prefill_attention",
     "pmxhip_mhca_create", "pmxhip_mhca_destroy", "pmxhip_mhca_heuristic_prepare",
@@ -83,6 +83,7 @@ DECODE_KERNEL_GENERAL = 1
 DECODE_KERNEL_QUAD = 2
 DECODE_KERNEL_MFMA16 = 3
 DECODE_KERNEL_MFMA32 = 4
+STATIC_WORKSPACE_BYTES = 32 * 1024 * 1024
 
 
 class PrefillParams(ctypes.Structure):
@@ -212,6 +213,8 @@ def lib():
     L.pmxhip_init.argtypes = []
     L.pmxhip_decode_plan_make_kernel.restype = ctypes.c_int
     L.pmxhip_decode_plan_make_kernel.argtypes = [c_i64] * 5 + [c_i32, c_i32, c_i32, ctypes.POINTER(DecodePlan)]
+    L.pmxhip_decode_attention_static.restype = ctypes.c_int
+    L.pmxhip_decode_attention_static.argtypes = [ctypes.POINTER(DecodeParams), c_vp]
     L.pmxhip_decode_kernel_name.restype = ctypes.c_char_p
     L.pmxhip_decode_kernel_name.argtypes = [ctypes.POINTER(DecodeParams)]
     L.pmxhip_decode_attention.restype = ctypes.c_int

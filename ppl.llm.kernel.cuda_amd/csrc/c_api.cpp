@@ -12,6 +12,14 @@
 
 #include "launch_params.h"
 
+// ---- scratch of the entry point that allocates nothing (pmxhip_decode_attention_static) ----
+// Split-KV pieces of one decode step: float32 partial outputs and (max, exp-sum) pairs, the same layout the
+// caller's workspace has in pmxhip_decode_attention.  One array per GPU, resident until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress; every use of the memory goes through
+// the per-device pointer resolved below.
+constexpr int64_t kStaticScratchBytes = PMXHIP_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace {
 
 thread_local char g_last_error[512] = "";
@@ -75,6 +83,31 @@ int current_compute_units()
     return cus;
 }
 
+constexpr int kScratchDevices = 64;
+std::atomic<void*> g_scratch_ptr[kScratchDevices];
+
+// The device address of `scratch` on the current device; resolved on first use per device (never under capture).
+int static_scratch(const char* who, pmxhip_stream_t stream, void** out)
+{
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kScratchDevices)
+        return fail(PMXHIP_OTHER_ERROR, "%s: no current device", who);
+    void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &st) != hipSuccess || st != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return fail(PMXHIP_OTHER_ERROR, "%s: first call on this device under stream capture; call pmxhip_init() first", who);
+        }
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            return fail(PMXHIP_OTHER_ERROR, "%s: hipGetSymbolAddress failed: %s", who, hipGetErrorString(e));
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return PMXHIP_SUCCESS;
+}
+
 } // namespace
 
 extern "C" {
@@ -87,6 +120,8 @@ int pmxhip_init(void)
         const hipError_t e = hipGetLastError();
         return fail(PMXHIP_OTHER_ERROR, "init: hipFuncSetAttribute failed: %s", hipGetErrorString(e));
     }
+    void* ptr = nullptr;
+    if (int rc = static_scratch("init", nullptr, &ptr)) return rc;
     (void)current_compute_units();
     return PMXHIP_SUCCESS;
 }
@@ -227,7 +262,7 @@ int pmxhip_decode_plan_make_kernel(int64_t decoding_batches, int64_t num_heads, 
 namespace {
 
 // Checks of a decode call and the launch block it becomes.  `workspace` / `workspace_size` are the caller's
-// (pmxhip_decode_attention).
+// (pmxhip_decode_attention) or the library's static array (pmxhip_decode_attention_static).
 int decode_prepare(const char* who, const pmxhip_decode_params* p, void* workspace, int64_t workspace_size,
                    pmxhip::DecodeLaunch* out)
 {
@@ -335,6 +370,27 @@ int pmxhip_decode_attention_stage(const pmxhip_decode_params* p, int32_t stage, 
     pmxhip::DecodeLaunch a;
     if (int rc = decode_prepare("decode_attention", p, p->workspace, p->workspace_size, &a)) return rc;
     return launch_result("decode_attention", pmxhip::launch_decode(a, stage, stream));
+}
+
+int pmxhip_decode_attention_static(const pmxhip_decode_params* p, pmxhip_stream_t stream)
+{
+    if (!p) return fail(PMXHIP_INVALID_VALUE, "decode_attention_static: null params");
+    if (p->decoding_batches < 0) return fail(PMXHIP_INVALID_VALUE, "decode_attention_static: negative decoding_batches");
+    if (p->decoding_batches == 0) return PMXHIP_SUCCESS;
+    if (p->num_token_ranges > 1) {
+        const double need = ((double)p->num_token_ranges + (double)p->decoding_batches) * (double)p->num_heads *
+                            ((double)p->head_dim + 2.0) * sizeof(float);
+        if (need > (double)kStaticScratchBytes)
+            return fail(PMXHIP_INVALID_VALUE,
+                        "decode_attention_static: the split-KV pieces of this call need %.0f bytes, the static workspace "
+                        "holds %lld; use fewer token ranges or pmxhip_decode_attention with a workspace of your own",
+                        need, (long long)kStaticScratchBytes);
+    }
+    void* ws = nullptr;
+    if (int rc = static_scratch("decode_attention_static", stream, &ws)) return rc;
+    pmxhip::DecodeLaunch a;
+    if (int rc = decode_prepare("decode_attention_static", p, ws, kStaticScratchBytes, &a)) return rc;
+    return launch_result("decode_attention_static", pmxhip::launch_decode(a, 0, stream));
 }
 
 const char* pmxhip_decode_kernel_name(const pmxhip_decode_params* p)

@@ -108,15 +108,15 @@ class DeviceBatch:
         return op
 
     def decode_only(self, num_token_ranges=0, workspace=None, attn_mask=None, mask_stride_s=0, mask_stride_h=0,
-                    output=None, stage=0, kernel=0, output_stride_s=None, name_only=False,
+                    output=None, stage=0, kernel=0, static_workspace=False, output_stride_s=None, name_only=False,
                     stream=None):
         """Decode attention through the flat C entry point (no operator object).  `kernel` requests a
-        token-range kernel; `name_only`
+        token-range kernel; `static_workspace` uses the entry point that allocates nothing; `name_only`
         launches nothing and returns the name of the kernel the call would run."""
         bt = self.bt
         plan = ops.decode_plan(bt.decoding_batches, bt.num_heads, bt.num_kv_heads, bt.head_dim, bt.max_kvlen,
                                ranges_hint=num_token_ranges, kernel=kernel)
-        if workspace is None and plan.workspace_size > 0 and not name_only:
+        if workspace is None and plan.workspace_size > 0 and not static_workspace and not name_only:
             workspace = torch.empty(int(plan.workspace_size), dtype=torch.uint8, device=self.device)
         out = self.output if output is None else output
         r = ops.decode_attention(self.query, out, self.cache, self.scale, self.cachestarts, self.kvstarts,
@@ -125,7 +125,7 @@ class DeviceBatch:
                                  num_kv_heads=bt.num_kv_heads, head_dim=bt.head_dim,
                                  num_token_ranges=plan.num_token_ranges, workspace=workspace,
                                  attn_mask=attn_mask, mask_stride_s=mask_stride_s, mask_stride_h=mask_stride_h, stage=stage,
-                                 kernel=kernel, output_stride_s=output_stride_s,
+                                 kernel=kernel, static_workspace=static_workspace, output_stride_s=output_stride_s,
                                  name_only=name_only, stream=stream, **self.layout_kwargs())
         if name_only:
             return r

@@ -107,10 +107,11 @@ def decode_attention(query, output, cache, scale, cachestarts, kvstarts, *, attn
                      decoding_batches, num_heads, num_kv_heads, head_dim, cache_mode, page_size,
                      cache_stride_s, cache_stride_l, cache_stride_h, cache_stride_kv, cachestarts_stride_b,
                      num_token_ranges, workspace=None, attn_mask=None, mask_stride_s=0, mask_stride_h=0,
-                     stage=0, stream=None, check=True, kernel=0, output_stride_s=None,
+                     stage=0, stream=None, check=True, kernel=0, static_workspace=False, output_stride_s=None,
                      name_only=False):
     """Decode attention of sequences [0, decoding_batches); output fp16 [B_dec, Hq, D].
-    `kernel` requests a token-range kernel; `name_only` launches nothing and returns the kernel's name."""
+    `kernel` requests a token-range kernel; `static_workspace` goes through the entry point that allocates
+    nothing (the library's own workspace); `name_only` launches nothing and returns the kernel's name."""
     p = DecodeParams()
     p.query = _ptr(query)
     p.attn_mask = _ptr(attn_mask)
@@ -143,7 +144,12 @@ def decode_attention(query, output, cache, scale, cachestarts, kvstarts, *, attn
     p.kernel_request = kernel
     if name_only:
         return _lib.lib().pmxhip_decode_kernel_name(ctypes.byref(p)).decode()
-    rc = _lib.lib().pmxhip_decode_attention_stage(ctypes.byref(p), stage, _stream(stream))
+    if static_workspace:
+        if stage != 0:
+            raise ValueError("the static-workspace entry point runs both stages")
+        rc = _lib.lib().pmxhip_decode_attention_static(ctypes.byref(p), _stream(stream))
+    else:
+        rc = _lib.lib().pmxhip_decode_attention_stage(ctypes.byref(p), stage, _stream(stream))
     if check and rc != RC_SUCCESS:
         raise PmxError(rc, "decode_attention")
     return rc
