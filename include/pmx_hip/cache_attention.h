@@ -37,7 +37,7 @@
 
 namespace ppl { namespace kernel { namespace llm { namespace cuda { namespace pmx {
 
-class dynamic_batching_multi_head_cache_attention {
+class PMXHIP_CXX_API dynamic_batching_multi_head_cache_attention {
 public:
     typedef int32_t decoding_algo_t;
     struct decoding_algo {

@@ -18,7 +18,7 @@
 
 namespace ppl { namespace kernel { namespace llm { namespace cuda { namespace pmx {
 
-ppl::common::RetCode dynamic_batching_key_value_cache(
+PMXHIP_CXX_API ppl::common::RetCode dynamic_batching_key_value_cache(
     const hipStream_t stream,
     const ppl::common::TensorShape* current_key_shape,
     const void* current_key, // half (S, KVH, D)

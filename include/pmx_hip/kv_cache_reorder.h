@@ -34,7 +34,7 @@ struct Stride {
     int d_stride_scale;
 };
 
-ppl::common::RetCode kv_cache_reorder(
+PMXHIP_CXX_API ppl::common::RetCode kv_cache_reorder(
     hipStream_t stream,
     const void* kv_cache,
     const void* kv_scale,
@@ -51,7 +51,7 @@ ppl::common::RetCode kv_cache_reorder(
     int64_t tp_size,
     void* outer_mem);
 
-ppl::common::RetCode kv_cache_invert_reorder(
+PMXHIP_CXX_API ppl::common::RetCode kv_cache_invert_reorder(
     hipStream_t stream,
     const void* outer_mem,
     const void* page_ids,

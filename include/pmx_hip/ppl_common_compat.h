@@ -12,6 +12,14 @@
 #ifndef PMX_HIP_PPL_COMMON_COMPAT_H_
 #define PMX_HIP_PPL_COMMON_COMPAT_H_
 
+/* libpmx_hip.so is built with hidden visibility; the operator class and the free functions of the C++ interface
+ * are exported explicitly so that a call site links against the library as it links against the reference's. */
+#if defined(__GNUC__)
+#define PMXHIP_CXX_API __attribute__((visibility("default")))
+#else
+#define PMXHIP_CXX_API
+#endif
+
 #ifdef PMX_HIP_USE_PPL_COMMON
 #include "ppl/common/retcode.h"
 #include "ppl/common/tensor_shape.h"

@@ -30,7 +30,7 @@ struct rope_scaling {
     static const rope_scaling_t DYNAMIC = 2;
 };
 
-ppl::common::RetCode dynamic_batching_rotary_position_embedding(
+PMXHIP_CXX_API ppl::common::RetCode dynamic_batching_rotary_position_embedding(
     hipStream_t stream,
     const ppl::common::TensorShape* query_shape,
     const void* query, // (seqstarts[-1], ..., head_dim), dim[1] is the leading dim of heads
@@ -55,7 +55,7 @@ ppl::common::RetCode dynamic_batching_rotary_position_embedding(
 
 // The same, then the quantise/append of the rotated key and of current_value into the int8 cache;
 // rotated_key may be nullptr.  The trailing arguments are forward_kvstore's.
-ppl::common::RetCode dynamic_batching_rotary_position_embedding_kv_cache(
+PMXHIP_CXX_API ppl::common::RetCode dynamic_batching_rotary_position_embedding_kv_cache(
     hipStream_t stream,
     const ppl::common::TensorShape* query_shape, const void* query,
     const ppl::common::TensorShape* key_shape, const void* key,

@@ -283,9 +283,10 @@ ppl::common::RetCode dynamic_batching_multi_head_cache_attention::forward_decode
     p.workspace_size = cfg.workspace_size;
     const int rc = pmxhip_decode_attention(&p, stream);
     if (rc != PMXHIP_SUCCESS) {
-        // the reference folds every decode dispatch failure into RC_UNSUPPORTED (kernel.cu:2118-2121)
+        // the reference folds every decode dispatch failure into RC_UNSUPPORTED (kernel.cu:2118-2121); what is not a
+        // matter of the configuration keeps its own code (a bad argument, a first launch under stream capture)
         PMX_LOG_ERROR("decode stage rejected the configuration");
-        return rc == PMXHIP_INVALID_VALUE ? ppl::common::RC_INVALID_VALUE : ppl::common::RC_UNSUPPORTED;
+        return rc == PMXHIP_UNSUPPORTED ? ppl::common::RC_UNSUPPORTED : to_retcode(rc);
     }
     return ppl::common::RC_SUCCESS;
 }

@@ -115,18 +115,30 @@ def test_decode_output_rows_aligned_to_8_bytes_only(pkg, oracle, shape):
 
 
 def test_decode_c1_golden_shape(pkg, oracle):
+    """C1 against the frozen fixture (tests/golden/c1_decode_golden.npz), not against a live oracle: the append
+    kernel's cache bytes and scales by digest and by the stored rows, the decode output within tolerance."""
+    import hashlib
+    import os
+    want = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "c1_decode_golden.npz"),
+                   allow_pickle=False)
     bt, rng = pkg.workloads.make_batch("C1")
-    cache, scale = host_cache(bt)
-    oracle_fill_history(oracle, pkg, bt, rng, cache, scale)
-    q, k, v = pkg.workloads.step_inputs(bt, rng)
-    oracle_append_step(oracle, bt, k, v, cache, scale)
+    assert np.array_equal(bt.kv_lens, want["kv_lens"]) and np.array_equal(bt.cachestarts, want["cachestarts"])
     dev = pkg.harness.DeviceBatch(bt)
-    dev.cache.copy_(torch.from_numpy(cache))
-    dev.scale.copy_(torch.from_numpy(scale))
+    dev.fill_history(rng)  # the history goes through the HIP append kernel
+    q, k, v = pkg.workloads.step_inputs(bt, rng)
     dev.set_step_inputs(q, k, v)
-    ref = oracle_decode(oracle, bt, q, cache, scale)
+    op = dev.make_operator()
+    assert op.forward() == 0
+    torch.cuda.synchronize()
+    cache, scale = dev.cache.cpu().numpy(), dev.scale.cpu().numpy()
+    rows = (bt.cachestarts + bt.start_pos).astype(np.int64)
+    assert np.array_equal(cache[0, 0, rows], want["appended_k"]) and np.array_equal(cache[0, 1, rows], want["appended_v"])
+    assert np.array_equal(scale[0, 0, rows].view(np.uint16), want["appended_k_scale"])
+    assert hashlib.sha256(np.ascontiguousarray(cache).tobytes()).hexdigest() == str(want["sha_cache"])
+    assert hashlib.sha256(np.ascontiguousarray(scale.view(np.uint16)).tobytes()).hexdigest() == str(want["sha_scale"])
+    assert_attention_close(dev.output.float().cpu().numpy(), want["output"], "C1 through the operator")
     got, _ = run_decode(dev)
-    assert_attention_close(got, ref, "C1")
+    assert_attention_close(got, want["output"], "C1")
 
 
 def test_decode_empty_sequence_and_closed_forms(pkg, oracle):
