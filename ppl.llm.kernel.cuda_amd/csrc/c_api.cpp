@@ -625,7 +625,7 @@ static int rope_common(const char* what, const pmxhip_rope_params* p, const pmxh
         a.cachestarts_stride_b = st->cachestarts_stride_b;
         a.cache_mode = st->cache_mode;
     }
-    return launch_result(what, pmxhip::launch_rope(a, stream));
+    return launch_result(what, pmxhip::launch_rope(a, current_compute_units(), stream));
 }
 
 int pmxhip_rotary_position_embedding(const pmxhip_rope_params* p, pmxhip_stream_t stream)

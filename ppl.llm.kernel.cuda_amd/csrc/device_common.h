@@ -110,6 +110,16 @@ __device__ __forceinline__ float dot2_init(half2_t a, half2_t b, float c)
     return r;
 }
 
+// max of three in one instruction.  Written as assembly because the compiler's fmaxf first passes every operand of
+// unknown origin through a quieting v_max_f32 x, x (one more instruction per accumulator element); the operands
+// here are products and sums of finite numbers or -inf, never a signalling NaN.
+__device__ __forceinline__ float max3(float a, float b, float c)
+{
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 // p - float(h.x) and p - float(h.y) in one instruction each: the mixed-precision fused multiply-add reads the
 // half operand in place (exact: the conversion and the subtraction round once, and the result is representable
 // whenever h is p rounded to half)

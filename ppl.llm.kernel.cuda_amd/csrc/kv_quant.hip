@@ -9,14 +9,16 @@
 // The half quotient is the correctly rounded binary32 quotient rounded once more to
 // binary16, which equals the correctly rounded half quotient (24 >= 2*11 + 2); the
 // binary32 quotient comes from one division per group (the reciprocal of the scale) and
-// a residual correction per element, see quantise_group.  The integer rounding is
-// v_rndne -- HIP's __half2short_rn truncates, so it is not used.
+// a residual correction per element, see quantise_group.  The integer rounding is an
+// addition in half (1536 + h, ulp one) -- HIP's __half2short_rn truncates, so it is not used.
 //
 // Decomposition (this file's own): a flat grid over (new token, group of 8
 // channels); one lane owns one group of K and the same group of V: two 128-bit
 // loads, two 64-bit int8 stores, two 16-bit scale stores.  The sequence of a
 // token is found by bisection over seqstarts, so no workgroup is launched per
 // (position, sequence) pair that does not exist.
+#include <cmath>
+
 #include "device_common.h"
 #include "launch_params.h"
 
@@ -31,41 +33,76 @@ struct Quantised {
     half_t scale;
 };
 
+// float(h.x) * b + c and float(h.y) * b + c with the half operand read in place (one instruction, one rounding)
+__device__ __forceinline__ float fma_half_lo(half2_t h, float b, float c)
+{
+    float r;
+    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(h), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ float fma_half_hi(half2_t h, float b, float c)
+{
+    float r;
+    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(h), "v"(b), "v"(c));
+    return r;
+}
+// float(h.x) - a * b and float(h.y) - a * b (the negation is a source modifier)
+__device__ __forceinline__ float half_lo_minus_product(half2_t h, float a, float b)
+{
+    float r;
+    asm("v_fma_mix_f32 %0, -%1, %2, %3 op_sel_hi:[0,0,1]" : "=v"(r) : "v"(a), "v"(b), "v"(h));
+    return r;
+}
+__device__ __forceinline__ float half_hi_minus_product(half2_t h, float a, float b)
+{
+    float r;
+    asm("v_fma_mix_f32 %0, -%1, %2, %3 op_sel:[0,0,1] op_sel_hi:[0,0,1]" : "=v"(r) : "v"(a), "v"(b), "v"(h));
+    return r;
+}
+
 __device__ __forceinline__ Quantised quantise_group(const u32x4 raw)
 {
-    half_t x[8];
+    half2_t x[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const half2_t h = bitcast<half2_t>(raw[i]);
-        x[2 * i] = h.x;
-        x[2 * i + 1] = h.y;
-    }
-    half_t amax = (half_t)0.0f;
+    for (int i = 0; i < 4; ++i) x[i] = bitcast<half2_t>(raw[i]);
+    // absmax in half, two channels at a time (sign bits cleared, packed maximum), then the two halves of the result
+    half2_t m2 = bitcast<half2_t>(raw[0] & 0x7fff7fffu);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const half_t ax = __builtin_fabsf16(x[i]);
-        amax = amax > ax ? amax : ax;
-    }
+    for (int i = 1; i < 4; ++i) m2 = __builtin_elementwise_max(m2, bitcast<half2_t>(raw[i] & 0x7fff7fffu));
+    const half_t amax = m2.x > m2.y ? m2.x : m2.y;
     const half_t eps = (half_t)1e-5f;
-    half_t s = (half_t)((float)amax / 127.0f);
+    // float(amax) / 127.0f, correctly rounded, without the division sequence: with r = fl(1 / 127), q0 = a * r,
+    // e = fma(-q0, 127, a), q = fma(e, r, q0).  Equal to the correctly rounded quotient for every positive finite
+    // half a (all 31 743 compared in exact arithmetic on the CPU).
+    const float af = (float)amax;
+    const float r127 = 1.0f / 127.0f;
+    const float s0 = af * r127;
+    half_t s = (half_t)__builtin_fmaf(__builtin_fmaf(-s0, 127.0f, af), r127, s0);
     s = s > eps ? s : eps;
     const float sf = (float)s;
     // One correctly rounded reciprocal per group, then a residual step per element:
     //   q0 = x * rcp, e = fma(-q0, sf, x), quotient = fma(e, rcp, q0).
     // Rounded to half this equals the correctly rounded quotient for every pair of a finite half x and a half
     // scale >= eps (all 2.0e9 pairs compared on the CPU; the one difference, -0 / s -> +0, yields the same int8 0).
+    // The half channels enter the mixed-precision multiply-adds in place, two quotients are rounded to half by one
+    // packed conversion, and the integer rounding is an addition: 1536 + h in half has an ulp of one, so the sum
+    // is h rounded to the nearest integer with ties to even, and its low byte is that integer in two's
+    // complement (|h| <= 127.4, the sum stays inside [1024, 2048)).
     const float rcp = 1.0f / sf;
-    uint32_t packed[2] = {0u, 0u};
+    const half2_t magic = {(half_t)1536.0f, (half_t)1536.0f};
+    uint32_t biased[4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const float xf = (float)x[i];
-        const float q0 = xf * rcp;
-        const half_t quo = (half_t)__builtin_fmaf(__builtin_fmaf(-q0, sf, xf), rcp, q0);
-        const int qi = (int)__builtin_rintf((float)quo);
-        packed[i >> 2] |= ((uint32_t)qi & 0xffu) << (8 * (i & 3));
+    for (int i = 0; i < 4; ++i) {
+        const float a0 = fma_half_lo(x[i], rcp, 0.0f), a1 = fma_half_hi(x[i], rcp, 0.0f);
+        const float e0 = half_lo_minus_product(x[i], a0, sf), e1 = half_hi_minus_product(x[i], a1, sf);
+        const float q0 = __builtin_fmaf(e0, rcp, a0), q1 = __builtin_fmaf(e1, rcp, a1);
+        typedef float float2_t __attribute__((ext_vector_type(2)));
+        const half2_t h = __builtin_convertvector(float2_t{q0, q1}, half2_t); // round to nearest even, both at once
+        biased[i] = bitcast<uint32_t>(h + magic);
     }
     Quantised r;
-    r.q = u32x2{packed[0], packed[1]};
+    // bytes 0 and 2 of each word are the integers of its two channels
+    r.q = u32x2{__builtin_amdgcn_perm(biased[1], biased[0], 0x06040200u), __builtin_amdgcn_perm(biased[3], biased[2], 0x06040200u)};
     r.scale = s;
     return r;
 }
@@ -85,23 +122,26 @@ __device__ __forceinline__ int sequence_of(const int64_t* __restrict__ starts, i
 
 } // namespace
 
+// stride_tokens: tokens between a thread's units, (workgroups * threads) / groups_per_token; the host sizes the launch
+// so that this division is exact whenever a thread takes more than one unit, which keeps a thread on one
+// (head, channel group) for all its units: the two integer divisions below then happen once, not once per unit.
 template <bool PAGED>
-__global__ __launch_bounds__(kQuantThreads) void kv_quantize_kernel(const QuantLaunch a)
+__global__ __launch_bounds__(kQuantThreads) void kv_quantize_kernel(const QuantLaunch a, const uint32_t stride_tokens)
 {
-    const int groups_per_head = a.head_dim >> 3;
-    const int groups_per_token = a.num_kv_heads * groups_per_head;
+    const uint32_t groups_per_head = (uint32_t)a.head_dim >> 3;
+    const uint32_t groups_per_token = (uint32_t)a.num_kv_heads * groups_per_head;
     const int64_t first = a.seqstarts[0];
     const int64_t n_tokens = a.seqstarts[a.batch] - first;
-    const int64_t n_units = n_tokens * groups_per_token;
-    const int64_t stride = (int64_t)gridDim.x * kQuantThreads;
-    for (int64_t u = (int64_t)blockIdx.x * kQuantThreads + threadIdx.x; u < n_units; u += stride) {
-        const int64_t tok = u / groups_per_token;
-        const int gi = (int)(u - tok * groups_per_token);
-        const int h = gi / groups_per_head;
-        const int d0 = (gi - h * groups_per_head) << 3;
+    const uint32_t u0 = blockIdx.x * kQuantThreads + threadIdx.x; // the host keeps workgroups * threads below 2^31
+    const uint32_t tok0 = u0 / groups_per_token;
+    const uint32_t gi = u0 - tok0 * groups_per_token;
+    const uint32_t h = gi / groups_per_head;
+    const uint32_t d0 = (gi - h * groups_per_head) << 3;
+    const int64_t in_idx = (int64_t)h * a.head_dim + d0;
+    const int64_t out_idx = a.layer_idx * a.cache_stride_l + (int64_t)h * a.cache_stride_h + d0;
+    for (int64_t tok = tok0; tok < n_tokens; tok += stride_tokens) {
         const int64_t in_tok = first + tok;
         // the rows to quantise do not depend on the sequence: requested first, they travel during the index lookups
-        const int64_t in_idx = (int64_t)h * a.head_dim + d0;
         const u32x4 kraw = *(const u32x4*)((const half_t*)a.current_key + in_tok * a.current_key_stride_s + in_idx);
         const u32x4 vraw = *(const u32x4*)((const half_t*)a.current_value + in_tok * a.current_value_stride_s + in_idx);
         // decode steps have one new token per sequence: token i then belongs to sequence i, which two independent
@@ -124,7 +164,7 @@ __global__ __launch_bounds__(kQuantThreads) void kv_quantize_kernel(const QuantL
         const Quantised kq = quantise_group(kraw);
         const Quantised vq = quantise_group(vraw);
 
-        const int64_t k_out = row * a.cache_stride_s + a.layer_idx * a.cache_stride_l + (int64_t)h * a.cache_stride_h + d0;
+        const int64_t k_out = row * a.cache_stride_s + out_idx;
         const int64_t v_out = k_out + a.cache_stride_kv;
         *(u32x2*)(a.cache + k_out) = kq.q;
         *(u32x2*)(a.cache + v_out) = vq.q;
@@ -150,7 +190,7 @@ __global__ __launch_bounds__(kQuantThreads) void rope_append_kernel(const RopeLa
     __shared__ float s_cos[kQuantThreads], s_sin[kQuantThreads];
     __shared__ int64_t s_row[kQuantThreads / 4];
     const int pairs = a.head_dim >> 1, rd2 = a.rotary_dim >> 1;
-    const int tokens_per_wg = kQuantThreads / pairs; // pairs <= 128
+    const int tokens_per_wg = a.tokens_per_wg; // at most kQuantThreads / pairs; pairs <= 128
     const int64_t first = a.seqstarts[0];
     const int64_t n_tokens = a.seqstarts[a.batch] - first;
     const int64_t tok0 = (int64_t)blockIdx.x * tokens_per_wg;
@@ -175,11 +215,15 @@ __global__ __launch_bounds__(kQuantThreads) void rope_append_kernel(const RopeLa
                         th = a.theta * (float)pow((double)base, (double)expn);
                     }
                 }
-                const float inv = 1.0f / (float)pow((double)th, (double)((float)i / (float)rd2));
+                // theta^(i / rd2) is the same for every token unless the dynamic scaling applies: then it comes in the
+                // launch arguments and the binary64 pow leaves the kernel
+                const float inv = a.has_inv_freq ? a.inv_freq[i] : 1.0f / (float)pow((double)th, (double)((float)i / (float)rd2));
                 const float p = a.scaling_type == 1 ? (float)pos / a.scaling_factor : (float)pos;
                 const float angle = inv * p;
-                c = (float)cos((double)angle);
-                s = (float)sin((double)angle);
+                double sd, cd;
+                sincos((double)angle, &sd, &cd); // one argument reduction for both
+                c = (float)cd;
+                s = (float)sd;
             }
             s_cos[threadIdx.x] = c;
             s_sin[threadIdx.x] = s;
@@ -242,34 +286,63 @@ __global__ __launch_bounds__(kQuantThreads) void rope_append_kernel(const RopeLa
     }
 }
 
-int launch_rope(const RopeLaunch& a, hipStream_t stream)
+int launch_rope(const RopeLaunch& a_in, int compute_units, hipStream_t stream)
 {
-    if (a.max_tokens <= 0) return 0;
-    if (a.head_dim > 256 || a.head_dim < 8) return 1;
-    const int tokens_per_wg = kQuantThreads / (a.head_dim / 2);
+    if (a_in.max_tokens <= 0) return kLaunchOk;
+    if (a_in.head_dim > 256 || a_in.head_dim < 8) return kLaunchNoKernel;
+    RopeLaunch a = a_in;
+    const int pairs = a.head_dim / 2, rd2 = a.rotary_dim / 2;
+    a.has_inv_freq = 0;
+    if (a.scaling_type != 2 && rd2 <= 128) {
+        for (int i = 0; i < rd2; ++i) a.inv_freq[i] = 1.0f / (float)pow((double)a.theta, (double)((float)i / (float)rd2));
+        a.has_inv_freq = 1;
+    }
+    // A workgroup computes the coefficients of its tokens once and shares them through LDS: as many tokens as its
+    // threads have pairs for, but no more than leaves two workgroups per CU (a decode step has a token per sequence,
+    // and a workgroup works through its tokens' rows one after the other)
+    int tokens_per_wg = kQuantThreads / pairs;
+    const int64_t spread = a.max_tokens / (2 * (int64_t)(compute_units > 0 ? compute_units : 256));
+    if (tokens_per_wg > spread) tokens_per_wg = spread > 1 ? (int)spread : 1;
+    a.tokens_per_wg = tokens_per_wg;
     const unsigned blocks = (unsigned)((a.max_tokens + tokens_per_wg - 1) / tokens_per_wg);
     if (a.cache_mode == 1) hipLaunchKernelGGL(rope_append_kernel<true>, dim3(blocks), dim3(kQuantThreads), 0, stream, a);
     else hipLaunchKernelGGL(rope_append_kernel<false>, dim3(blocks), dim3(kQuantThreads), 0, stream, a);
-    return 0;
+    return kLaunchOk;
 }
 
 int launch_kv_quantize(const QuantLaunch& a, int compute_units, hipStream_t stream)
 {
     const int64_t groups_per_token = (int64_t)a.num_kv_heads * (a.head_dim >> 3);
     const int64_t max_units = a.max_tokens * groups_per_token;
-    if (max_units <= 0) return 0;
+    if (max_units <= 0) return kLaunchOk;
     int64_t blocks = (max_units + kQuantThreads - 1) / kQuantThreads;
     // grid-stride beyond this: eight workgroups per CU hold every wave slot at once, and a lane then takes two or
     // three units in turn (11 104 new tokens of 8 heads x 128 channels on 256 CUs: 23.4 us against 28 us with four
     // times as many workgroups and one unit per lane, 36 us with 32 times as many, most of them without a unit;
     // 25 us with half as many)
     const int64_t cap = (int64_t)(compute_units > 0 ? compute_units : 256) * 8;
-    if (blocks > cap) blocks = cap;
+    if (blocks > cap) {
+        // a whole number of token rows per sweep of the grid, so that a thread keeps its (head, channel group):
+        // the workgroup count is a multiple of groups_per_token / gcd(groups_per_token, threads per workgroup)
+        int64_t g = groups_per_token, t = kQuantThreads;
+        while (t != 0) {
+            const int64_t r = g % t;
+            g = t;
+            t = r;
+        }
+        const int64_t unit = groups_per_token / g;
+        blocks = cap / unit * unit;
+        if (blocks == 0) blocks = unit;
+    }
+    if (blocks * kQuantThreads >= (int64_t)1 << 31) return kLaunchNoKernel;
+    // exact when blocks was rounded above; otherwise no thread takes a second unit and the value only has to carry
+    // a thread beyond the last token
+    const uint32_t stride_tokens = (uint32_t)((blocks * kQuantThreads + groups_per_token - 1) / groups_per_token);
     if (a.cache_mode == 1)
-        hipLaunchKernelGGL(kv_quantize_kernel<true>, dim3((unsigned)blocks), dim3(kQuantThreads), 0, stream, a);
+        hipLaunchKernelGGL(kv_quantize_kernel<true>, dim3((unsigned)blocks), dim3(kQuantThreads), 0, stream, a, stride_tokens);
     else
-        hipLaunchKernelGGL(kv_quantize_kernel<false>, dim3((unsigned)blocks), dim3(kQuantThreads), 0, stream, a);
-    return 0;
+        hipLaunchKernelGGL(kv_quantize_kernel<false>, dim3((unsigned)blocks), dim3(kQuantThreads), 0, stream, a, stride_tokens);
+    return kLaunchOk;
 }
 
 } // namespace pmxhip

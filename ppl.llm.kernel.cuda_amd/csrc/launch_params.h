@@ -137,6 +137,11 @@ struct RopeLaunch {
     int64_t max_position_embeddings;
     int32_t scaling_type;       // 0 none, 1 linear, 2 dynamic
     int32_t bypass_key;
+    // 1 / theta^(i / (rotary_dim / 2)) for pair i, computed by the host launcher (in double, rounded to float) when
+    // theta does not depend on the sequence (scaling types 0 and 1); has_inv_freq = 0: the kernel computes it
+    float inv_freq[128];
+    int32_t has_inv_freq;
+    int32_t tokens_per_wg;      // consecutive tokens one workgroup takes, at most 256 / (head_dim / 2)
     // append part (same meaning as QuantLaunch)
     int8_t* cache;
     void* scale;
@@ -168,7 +173,7 @@ inline int ensure_dynamic_lds(const void* kernel, int bytes, hipStream_t stream,
 }
 
 int launch_kv_quantize(const QuantLaunch& a, int compute_units, hipStream_t stream);
-int launch_rope(const RopeLaunch& a, hipStream_t stream);
+int launch_rope(const RopeLaunch& a, int compute_units, hipStream_t stream);
 void launch_page_copy(const PageCopyLaunch& a, hipStream_t stream);
 int launch_decode(const DecodeLaunch& a, int stage, hipStream_t stream); // stage: 0 both, 1 ranges, 2 combine
 

@@ -42,9 +42,15 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kNegBig = -1.0e30f;
 constexpr float kPShift = 14.0f;
 
-// position of token offset o (0..15) inside its 16-token group of the transposed V tile:
-// token bits (a, h, r1, r0) -> position bits (h, a, r1, r0)
-__device__ __forceinline__ int vt_pos16(int o) { return ((o & 4) << 1) | ((o & 8) >> 1) | (o & 3); }
+// LDS tile geometry.  K rows carry 16 bytes of padding: the 16-byte fragment reads of 32 rows then cover all banks.
+// V rows are read with transposing 8-byte loads that take 64 bytes of each of four consecutive rows per
+// half-wave: a row stride of 64 bytes modulo 256 puts those four segments on different banks.
+template <int D>
+struct PrefillTile {
+    static constexpr int K_STRIDE = D + 8;
+    static constexpr int V_STRIDE = D + 32;
+};
+static_assert((PrefillTile<128>::V_STRIDE * 2) % 256 == 64 && (PrefillTile<64>::V_STRIDE * 2) % 256 == 192, "V row stride");
 
 // sum over the wave of small non-negative integers, one ballot per bit (every lane of the wave must be here)
 __device__ __forceinline__ int wave_sum_small(int v)
@@ -143,6 +149,25 @@ __device__ __forceinline__ bool pick_query_tile(const PrefillLaunch& a, int ppw,
 
 // SRC: where K/V come from: 0 = int8 cache in 128-token pages, 1 = int8 cache in contiguous runs,
 // 2 = the step's fp16 current_key/current_value rows.  EXTRA: additive attn_mask and/or alibi slopes.
+//
+// Schedule of one 64-token tile in one wave (the two 32-token blocks b0, b1 of the tile are independent until the
+// output accumulators).  Every phase pairs matrix work of one block with vector work of the other, in one
+// instruction stream whose order is fixed by scheduling barriers:
+//     phase 1   S^T(b0) products        with   dequantisation of the next tile into the other LDS buffer
+//     phase 2   S^T(b1) products        with   softmax of b0 (and the global requests for the tile after next)
+//     phase 3   O^T += V^T P^T of b0    with   softmax of b1
+//     phase 4   O^T += V^T P^T of b1
+// The running maximum is updated per block.  A maximum that moves rescales the accumulators (wave-uniform,
+// rare after the first tiles): for b0 before its products start, for b1 after the products of b0 have been
+// issued (the rescale then waits for them, being a reader of their accumulators).
+//
+// Measured on the mixed workload (16 sequences of 256-1024 query rows over up to 2048 prior tokens, 32 query / 8 kv
+// heads of 128): the kernel takes 655 us; built without its products 442 us, without the LDS fragment reads 543 us,
+// without dequantisation and global loads 531 us, without exp and the split of p 673 us, without the tile barrier
+// 662 us, with none of these 131 us: the parts add up to the whole, so little of them runs concurrently.  The
+// fragment reads alone take what the LDS port allows (512 KB per tile and CU at 256 bytes per clock).  A form with
+// four waves of 64 columns (half the fragment reads per product, fragments requested two steps ahead, the whole
+// register file per wave) took 1094 us: one wave per SIMD exposes every wait that a second wave covers.
 template <int D, int SRC, bool EXTRA>
 __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(const PrefillLaunch a)
 {
@@ -151,10 +176,10 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     constexpr int KSTEPS = D / 16;          // MFMA k-steps over channels for S
     constexpr int CB = D / 32;              // 32-channel blocks of O^T
     constexpr int GPT = D / 8;              // quantisation groups per token row
-    constexpr int K_STRIDE = D + 8;         // halves per K row in LDS (+16 B: conflict-free b128 reads)
-    constexpr int V_STRIDE = kBN + 8;       // halves per V^T row in LDS
-    constexpr int K_UNITS = kBN * GPT / kPrefillThreads;  // (token, group) units per thread
-    constexpr int V_THREADS = (kBN / 4) * GPT;            // threads with a (token quad, group) unit
+    constexpr int K_STRIDE = PrefillTile<D>::K_STRIDE; // halves per K row in LDS
+    constexpr int V_STRIDE = PrefillTile<D>::V_STRIDE; // halves per V row in LDS (row-major, like K)
+    constexpr int UNITS = kBN * GPT / kPrefillThreads; // (token, group) units per thread, of K and of V each
+    constexpr int K_TSTEP = kPrefillThreads / GPT;     // tokens between a thread's units
 
     // K is kept as an unevaluated sum hi + lo of two halves: hi = fp16(int8 * scale) and
     // lo = the rounding error of that product (exact, from one fused multiply-add), so that
@@ -164,9 +189,10 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     // trick, p = hi + lo), and O accumulates hi*hi + lo*hi + hi*lo: at |v| ~ 40 a single fp16
     // rounding of either factor already costs ~1e-2 absolute where contributions cancel.
     extern __shared__ __attribute__((aligned(16))) char smem_raw[];
-    // two tile buffers; a buffer holds K (hi, lo) row-major and V (hi, lo) transposed
+    // two tile buffers; a buffer holds K (hi, lo) and V (hi, lo), all row-major [token][channel]
     // (fp16 K/V need no low parts: the tiles are the values themselves)
-    constexpr int TILE_HALVES = (KV16 ? 1 : 2) * (kBN * K_STRIDE + D * V_STRIDE);
+    constexpr int K_HALVES = kBN * K_STRIDE, V_HALVES = kBN * V_STRIDE;
+    constexpr int TILE_HALVES = (KV16 ? 1 : 2) * (K_HALVES + V_HALVES);
     half_t* const smem = (half_t*)smem_raw;
 
     const int tid = threadIdx.x;
@@ -175,12 +201,41 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     const int hh = lane >> 5;   // half-wave
     const int l32 = lane & 31;
 
-    // grid: workgroup = (item, kv head), kv head fastest; item i is the i-th query tile of the batch in the order
-    // of falling cost (pick_query_tile), and workgroups start in the order of their numbers
+    // per-lane parts of the LDS addresses (halves)
+    const int k_frag_off = l32 * K_STRIDE + 8 * hh; // + (32 mb) rows + 16 s: the A fragment of S^T
+    // A fragment of O^T = rows (channels) of V^T, read from the row-major tile with transposing loads: in a group
+    // of 16 lanes, lane i sends the address of 4 channels (4 (i % 4) ..) of token (i / 4) and receives channel i
+    // of the group's 4 tokens.  The group (lane / 16) = (channel half g % 2, token half hh).
+    const int v_frag_off = (4 * hh + ((lane & 15) >> 2)) * V_STRIDE + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+
     const int G = (int)(a.num_heads / a.num_kv_heads);
     const int ppw = kCols / G > 0 ? kCols / G : 1; // query positions per workgroup
-    const int item = blockIdx.x / (int)a.num_kv_heads;
-    const int kvh = blockIdx.x - item * (int)a.num_kv_heads;
+    const int kvh = blockIdx.x % (int)a.num_kv_heads;
+    const int item_stride = gridDim.x / (int)a.num_kv_heads;
+
+    const int8_t* __restrict__ cache = (const int8_t*)a.cache;
+    const half_t* __restrict__ scale = (const half_t*)a.scale;
+    const int64_t head_off = a.layer_idx * a.cache_stride_l + (int64_t)kvh * a.cache_stride_h;
+    const int8_t* const cache_k = cache + head_off;
+    const int8_t* const cache_v = cache_k + a.cache_stride_kv;
+    const half_t* const scale_k = scale + (head_off >> 3);
+    const half_t* const scale_v = scale_k + (a.cache_stride_kv >> 3);
+    const const_i64_ptr cachestarts = as_constant(a.cachestarts);
+    const float sm_scale = a.attn_scale * kLog2e;
+
+    // this thread's (token, group) units of a tile: token u_t0 + u * K_TSTEP, group u_g, for K and for V alike
+    const int u_g = tid % GPT;
+    const int u_t0 = tid / GPT;
+    const uint32_t stride_s32 = (uint32_t)a.cache_stride_s; // the host checks that a tile's span fits 32 bits
+    const uint32_t kstride16 = (uint32_t)a.key_stride_s, vstride16 = (uint32_t)a.value_stride_s;
+    uint32_t u_off[UNITS];
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) u_off[u] = (uint32_t)(u_t0 + u * K_TSTEP) * stride_s32 + 8 * u_g;
+
+    // The workgroups of the launch share the batch's query tiles: workgroup (item, kv head) takes the items
+    // item, item + item_stride, ... in the order of falling cost, so that a launch that was sized from a hint that
+    // understates the batch still covers every tile (it only takes longer).
+    for (int item = blockIdx.x / (int)a.num_kv_heads;; item += item_stride) {
     int b_pick = 0, tile_pick = 0;
     if (!pick_query_tile(a, ppw, item, lane, b_pick, tile_pick)) return;
     const int b = __builtin_amdgcn_readfirstlane(b_pick);
@@ -188,7 +243,7 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     const int qlen = (int)(a.seqstarts[b + 1] - q_row0);
     const int kvlen = (int)(a.kvstarts[b + 1] - a.kvstarts[b]);
     const int p0 = __builtin_amdgcn_readfirstlane(tile_pick) * ppw;
-    if (p0 < 0 || p0 >= qlen) return;
+    if (p0 < 0 || p0 >= qlen) continue;
 
     // ---- this lane's column ----
     const int col = wave * 32 + l32;
@@ -227,7 +282,6 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
 #pragma unroll
         for (int i = 0; i < 16; ++i) o_acc[cb][i] = 0.f;
     float m_run = kNegBig, l_run = 0.f;
-    const float sm_scale = a.attn_scale * kLog2e;
     // element (head, absolute query row, absolute kv column) of the additive mask; kvstarts holds absolute columns
     const half_t* mask_row = nullptr;
     float slope = 0.f;
@@ -238,28 +292,14 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     }
 
     // ---- global -> register staging of one tile's raw bytes ----
-    const int8_t* __restrict__ cache = (const int8_t*)a.cache;
-    const half_t* __restrict__ scale = (const half_t*)a.scale;
-    const int64_t head_off = a.layer_idx * a.cache_stride_l + (int64_t)kvh * a.cache_stride_h;
     const int64_t table_base = PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b;
-
-    const int k_g = tid % GPT;           // channel group of this thread's K units
-    const int k_t0 = tid / GPT;          // first token; further units are kPrefillThreads / GPT tokens apart
-    const int v_g = tid % GPT;
-    const int v_q = (tid / GPT) % (kBN / 4); // token quad (tokens 4 v_q .. 4 v_q + 3)
-    const int v_half = tid / V_THREADS;      // which four of the group's eight channels this thread transposes
-    const bool v_on = (2 * V_THREADS == kPrefillThreads) || v_half < 2; // compile-time true when every thread has a unit
-
-    u32x2 k_raw[K_UNITS];
-    half_t k_sc[K_UNITS];
-    u32x2 v_raw[4];
-    half_t v_sc[4];
-    u32x4 k16[K_UNITS], v16[4]; // fp16 source: 8 halves per unit
+    u32x2 k_raw[UNITS], v_raw[UNITS];
+    half_t k_sc[UNITS], v_sc[UNITS];
+    u32x4 k16[UNITS], v16[UNITS]; // fp16 source: 8 halves per unit
 
     // Addressing: a tile of 64 tokens starts at a multiple of 64, so it lies inside one page.  Its row
     // base is wave-uniform (scalar loads of the page table, read one tile ahead); the per-lane part
     // (token in tile, channel group) never changes and is computed once.
-    const const_i64_ptr cachestarts = as_constant(a.cachestarts);
     auto tile_row = [&](int tile) -> int64_t {
         int t_base = tile * kBN;
         if (t_base > kvlen - 1) t_base = kvlen > 0 ? kvlen - 1 : 0;
@@ -267,37 +307,17 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         if (PAGED) return cachestarts[table_base + (t_base >> 7)] + (t_base & (kPage - 1));
         return cachestarts[table_base] + t_base;
     };
-    const uint32_t stride_s32 = (uint32_t)a.cache_stride_s; // the host checks that a tile's span fits 32 bits
-    constexpr int K_TSTEP = kPrefillThreads / GPT;           // tokens between a thread's K units
-    uint32_t k_off[K_UNITS], v_off[4];
-#pragma unroll
-    for (int u = 0; u < K_UNITS; ++u) k_off[u] = (uint32_t)(k_t0 + u * K_TSTEP) * stride_s32 + 8 * k_g;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) v_off[r] = (uint32_t)(4 * v_q + r) * stride_s32 + 8 * v_g;
-    const int8_t* const cache_k = cache + head_off;
-    const int8_t* const cache_v = cache_k + a.cache_stride_kv;
-    const half_t* const scale_k = scale + (head_off >> 3);
-    const half_t* const scale_v = scale_k + (a.cache_stride_kv >> 3);
-
-    const uint32_t kstride16 = (uint32_t)a.key_stride_s, vstride16 = (uint32_t)a.value_stride_s;
     auto load_tile = [&](int tile, int64_t row) {
+        const int left = kvlen - 1 - tile * kBN; // offset of the sequence's last token inside this tile
         if (KV16) {
             const half_t* bk = (const half_t*)a.current_key + row * a.key_stride_s + (int64_t)kvh * D;
             const half_t* bv = (const half_t*)a.current_value + row * a.value_stride_s + (int64_t)kvh * D;
-            const int left = kvlen - 1 - tile * kBN;
 #pragma unroll
-            for (int u = 0; u < K_UNITS; ++u) {
-                int t = k_t0 + u * K_TSTEP;
+            for (int u = 0; u < UNITS; ++u) {
+                int t = u_t0 + u * K_TSTEP;
                 t = t < left ? t : (left > 0 ? left : 0);
-                k16[u] = *(const u32x4*)(bk + (uint32_t)t * kstride16 + 8 * k_g);
-            }
-            if (v_on) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    int t = 4 * v_q + r;
-                    t = t < left ? t : (left > 0 ? left : 0);
-                    v16[r] = *(const u32x4*)(bv + (uint32_t)t * vstride16 + 8 * v_g);
-                }
+                k16[u] = *(const u32x4*)(bk + (uint32_t)t * kstride16 + 8 * u_g);
+                v16[u] = *(const u32x4*)(bv + (uint32_t)t * vstride16 + 8 * u_g);
             }
             return;
         }
@@ -306,299 +326,303 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         const int8_t* bv = cache_v + boff;
         const half_t* sk = scale_k + (boff >> 3);
         const half_t* sv = scale_v + (boff >> 3);
-        const int left = kvlen - 1 - tile * kBN; // offset of the sequence's last token inside this tile
         if (left >= kBN - 1) {
 #pragma unroll
-            for (int u = 0; u < K_UNITS; ++u) {
-                k_raw[u] = *(const u32x2*)(bk + k_off[u]);
-                k_sc[u] = sk[k_off[u] >> 3];
-            }
-            if (v_on) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    v_raw[r] = *(const u32x2*)(bv + v_off[r]);
-                    v_sc[r] = sv[v_off[r] >> 3];
-                }
+            for (int u = 0; u < UNITS; ++u) {
+                k_raw[u] = *(const u32x2*)(bk + u_off[u]);
+                k_sc[u] = sk[u_off[u] >> 3];
+                v_raw[u] = *(const u32x2*)(bv + u_off[u]);
+                v_sc[u] = sv[u_off[u] >> 3];
             }
         } else { // last tile of the sequence: tokens beyond it re-read its last token (masked later)
 #pragma unroll
-            for (int u = 0; u < K_UNITS; ++u) {
-                const int t = k_t0 + u * K_TSTEP;
-                const uint32_t off = (uint32_t)(t < left ? t : (left > 0 ? left : 0)) * stride_s32 + 8 * k_g;
+            for (int u = 0; u < UNITS; ++u) {
+                const int t = u_t0 + u * K_TSTEP;
+                const uint32_t off = (uint32_t)(t < left ? t : (left > 0 ? left : 0)) * stride_s32 + 8 * u_g;
                 k_raw[u] = *(const u32x2*)(bk + off);
                 k_sc[u] = sk[off >> 3];
-            }
-            if (v_on) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int t = 4 * v_q + r;
-                    const uint32_t off = (uint32_t)(t < left ? t : (left > 0 ? left : 0)) * stride_s32 + 8 * v_g;
-                    v_raw[r] = *(const u32x2*)(bv + off);
-                    v_sc[r] = sv[off >> 3];
-                }
+                v_raw[u] = *(const u32x2*)(bv + off);
+                v_sc[u] = sv[off >> 3];
             }
         }
     };
-    // One slice of the dequantise-and-store of a tile: slices [0, K_UNITS) are this thread's K units, slices
-    // K_UNITS + [0, 4) its four V channels.  Sliced so that the work can be spread between the MFMAs of the
-    // previous tile's products.
-    constexpr int N_SLICES = K_UNITS + 4;
+    // One slice of the dequantise-and-store of a tile: slices [0, UNITS) are this thread's K units, slices
+    // UNITS + [0, UNITS) its V units.  Sliced so that the work can be spread between the MFMAs of phase 1.
+    constexpr int N_SLICES = 2 * UNITS;
     auto store_slice = [&](int buf, int slice) {
         half_t* const sK = smem + buf * TILE_HALVES;
-        half_t* const sKlo = sK + kBN * K_STRIDE;
-        half_t* const sV = KV16 ? sKlo : sKlo + kBN * K_STRIDE;
-        half_t* const sVlo = sV + D * V_STRIDE;
+        half_t* const sKlo = sK + K_HALVES;
+        half_t* const sV = KV16 ? sKlo : sKlo + K_HALVES;
+        half_t* const sVlo = sV + V_HALVES;
+        const bool is_v = slice >= UNITS;
+        const int u = is_v ? slice - UNITS : slice;
+        const int t = u_t0 + u * K_TSTEP;
+        half_t* const dst = is_v ? &sV[t * V_STRIDE + 8 * u_g] : &sK[t * K_STRIDE + 8 * u_g];
         if (KV16) {
-#pragma unroll
-            for (int u = 0; u < K_UNITS; ++u)
-                if (slice == u) *(u32x4*)&sK[(k_t0 + u * K_TSTEP) * K_STRIDE + 8 * k_g] = k16[u];
-            if (v_on) {
-                const int grp = v_q >> 2;
-                const int posv = 16 * grp + vt_pos16(4 * (v_q & 3));
-#pragma unroll
-                for (int e4 = 0; e4 < 4; ++e4) {
-                    if (slice != K_UNITS + e4) continue;
-                    const int e = 4 * v_half + ((e4 + v_g) & 3); // rotated channel order, as below
-                    const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u; // half (e & 1) of two words
-                    const int w = e >> 1;
-                    const uint32_t w0 = w == 0 ? v16[0][0] : (w == 1 ? v16[0][1] : (w == 2 ? v16[0][2] : v16[0][3]));
-                    const uint32_t w1 = w == 0 ? v16[1][0] : (w == 1 ? v16[1][1] : (w == 2 ? v16[1][2] : v16[1][3]));
-                    const uint32_t w2 = w == 0 ? v16[2][0] : (w == 1 ? v16[2][1] : (w == 2 ? v16[2][2] : v16[2][3]));
-                    const uint32_t w3 = w == 0 ? v16[3][0] : (w == 1 ? v16[3][1] : (w == 2 ? v16[3][2] : v16[3][3]));
-                    u32x2 out;
-                    out[0] = __builtin_amdgcn_perm(w1, w0, sel);
-                    out[1] = __builtin_amdgcn_perm(w3, w2, sel);
-                    *(u32x2*)&sV[(8 * v_g + e) * V_STRIDE + posv] = out;
-                }
-            }
+            *(u32x4*)dst = is_v ? v16[u] : k16[u];
             return;
         }
-        // K: 8 halves of one (token, group) -> one 128-bit LDS store
-#pragma unroll
-        for (int u = 0; u < K_UNITS; ++u) {
-            if (slice != u) continue;
-            const half2_t sc = {k_sc[u], k_sc[u]};
-            const uint32_t f0 = k_raw[u][0] ^ kFlipSigns, f1 = k_raw[u][1] ^ kFlipSigns;
-            const half2_t x0 = cvt_bytes01(f0), x1 = cvt_bytes23(f0), x2 = cvt_bytes01(f1), x3 = cvt_bytes23(f1);
-            const half2_t h0 = x0 * sc, h1 = x1 * sc, h2 = x2 * sc, h3 = x3 * sc;
-            u32x4 w, wl;
-            w[0] = bitcast<uint32_t>(h0);
-            w[1] = bitcast<uint32_t>(h1);
-            w[2] = bitcast<uint32_t>(h2);
-            w[3] = bitcast<uint32_t>(h3);
-            wl[0] = bitcast<uint32_t>(__builtin_elementwise_fma(x0, sc, -h0));
-            wl[1] = bitcast<uint32_t>(__builtin_elementwise_fma(x1, sc, -h1));
-            wl[2] = bitcast<uint32_t>(__builtin_elementwise_fma(x2, sc, -h2));
-            wl[3] = bitcast<uint32_t>(__builtin_elementwise_fma(x3, sc, -h3));
-            const int t = k_t0 + u * (kPrefillThreads / GPT);
-            *(u32x4*)&sK[t * K_STRIDE + 8 * k_g] = w;
-            *(u32x4*)&sKlo[t * K_STRIDE + 8 * k_g] = wl;
-        }
-        // V: four tokens of one channel -> one 64-bit LDS store into the transposed tile
-        if (v_on) {
-            const half2_t s01 = {v_sc[0], v_sc[1]}, s23 = {v_sc[2], v_sc[3]};
-            const int grp = v_q >> 2;
-            const int posv = 16 * grp + vt_pos16(4 * (v_q & 3));
-#pragma unroll
-            for (int e4 = 0; e4 < 4; ++e4) {
-                if (slice != K_UNITS + e4) continue;
-                const int e = 4 * v_half + ((e4 + v_g) & 3); // rotate the channel order per lane: spreads LDS banks
-                // byte e of each of the four tokens; the byte index is a run-time value, so the
-                // v_perm selector is built instead of templated
-                const uint32_t sel = 0x0c000c00u | (uint32_t)(e & 3) | ((uint32_t)(4 + (e & 3)) << 16);
-                const bool upper = e >= 4;
-                const uint32_t w0 = upper ? v_raw[0][1] : v_raw[0][0], w1 = upper ? v_raw[1][1] : v_raw[1][0];
-                const uint32_t w2 = upper ? v_raw[2][1] : v_raw[2][0], w3 = upper ? v_raw[3][1] : v_raw[3][0];
-                const half2_t lo = pk_sub_1152(__builtin_amdgcn_perm(w1, w0, sel) ^ 0x64806480u);
-                const half2_t hi = pk_sub_1152(__builtin_amdgcn_perm(w3, w2, sel) ^ 0x64806480u);
-                const half2_t h01 = lo * s01, h23 = hi * s23;
-                u32x2 out, outl;
-                out[0] = bitcast<uint32_t>(h01);
-                out[1] = bitcast<uint32_t>(h23);
-                outl[0] = bitcast<uint32_t>(__builtin_elementwise_fma(lo, s01, -h01));
-                outl[1] = bitcast<uint32_t>(__builtin_elementwise_fma(hi, s23, -h23));
-                *(u32x2*)&sV[(8 * v_g + e) * V_STRIDE + posv] = out;
-                *(u32x2*)&sVlo[(8 * v_g + e) * V_STRIDE + posv] = outl;
-            }
-        }
-    };
-
-    auto store_tile = [&](int buf) {
-#pragma unroll
-        for (int k = 0; k < N_SLICES; ++k) store_slice(buf, k);
+        half_t* const dst_lo = is_v ? &sVlo[t * V_STRIDE + 8 * u_g] : &sKlo[t * K_STRIDE + 8 * u_g];
+        const u32x2 raw = is_v ? v_raw[u] : k_raw[u];
+        const half_t scl = is_v ? v_sc[u] : k_sc[u];
+        const half2_t sc = {scl, scl};
+        const uint32_t f0 = raw[0] ^ kFlipSigns, f1 = raw[1] ^ kFlipSigns;
+        const half2_t x0 = cvt_bytes01(f0), x1 = cvt_bytes23(f0), x2 = cvt_bytes01(f1), x3 = cvt_bytes23(f1);
+        const half2_t h0 = x0 * sc, h1 = x1 * sc, h2 = x2 * sc, h3 = x3 * sc;
+        u32x4 w, wl;
+        w[0] = bitcast<uint32_t>(h0);
+        w[1] = bitcast<uint32_t>(h1);
+        w[2] = bitcast<uint32_t>(h2);
+        w[3] = bitcast<uint32_t>(h3);
+        wl[0] = bitcast<uint32_t>(__builtin_elementwise_fma(x0, sc, -h0));
+        wl[1] = bitcast<uint32_t>(__builtin_elementwise_fma(x1, sc, -h1));
+        wl[2] = bitcast<uint32_t>(__builtin_elementwise_fma(x2, sc, -h2));
+        wl[3] = bitcast<uint32_t>(__builtin_elementwise_fma(x3, sc, -h3));
+        *(u32x4*)dst = w;
+        *(u32x4*)dst_lo = wl;
     };
 
     // Prologue: tile 0 dequantised into buffer 0, raw bytes of tile 1 in registers.
     int64_t row_next = 0;
     if (n_tiles > 0) {
         load_tile(0, tile_row(0));
-        store_tile(0);
+#pragma unroll
+        for (int k = 0; k < N_SLICES; ++k) store_slice(0, k);
         if (n_tiles > 1) load_tile(1, tile_row(1));
         row_next = tile_row(2);
         __syncthreads();
     }
-    // tokens this wave's columns attend to: beyond them (a tile past its columns' limits, or a wave whose columns lie
-    // beyond the query rows: short chunks leave most waves without any) the wave only helps to stage the tiles
-    int wave_lim = lim;
+    // tokens this wave's columns attend to: beyond the largest limit (a tile past its columns' limits, or a wave
+    // whose columns lie beyond the query rows: short chunks leave most waves without any) the wave only helps to
+    // stage the tiles; up to the smallest limit of its live columns no element needs the limit test
+    int wave_lim = lim, wave_lim_min = col_on ? lim : 0x7fffffff;
 #pragma unroll
     for (int sh = 32; sh >= 1; sh >>= 1) {
-        const int o = __shfl_xor(wave_lim, sh);
+        const int o = __shfl_xor(wave_lim, sh), o2 = __shfl_xor(wave_lim_min, sh);
         wave_lim = o > wave_lim ? o : wave_lim;
+        wave_lim_min = o2 < wave_lim_min ? o2 : wave_lim_min;
     }
     wave_lim = __builtin_amdgcn_readfirstlane(wave_lim);
-    for (int tile = 0; tile < n_tiles; ++tile) {
-        const bool work = tile * kBN < wave_lim;
-        const half_t* const sK = smem + (tile & 1) * TILE_HALVES;
-        const half_t* const sKlo = sK + kBN * K_STRIDE;
-        const half_t* const sV = KV16 ? sKlo : sKlo + kBN * K_STRIDE;
-        const half_t* const sVlo = sV + D * V_STRIDE;
+    wave_lim_min = __builtin_amdgcn_readfirstlane(wave_lim_min);
 
-        // ---- S^T = K Q^T : two 32-token blocks.  The A fragments come from LDS in batches of QB k-steps, the
-        // next batch requested before the current one is multiplied, so that an MFMA never waits for the
-        // read issued just before it ----
-        f32x16 s_acc[2];
+    // ---- one tile, for a wave that has columns in it.  limit: some element may lie beyond its column's limit ----
+    auto tile_body = [&](int tile, const bool limit) {
+        const int buf = tile & 1;
+        const half_t* const sK = smem + buf * TILE_HALVES;
+        const half_t* const sKlo = sK + K_HALVES;
+        const half_t* const sV = KV16 ? sKlo : sKlo + K_HALVES;
+        const half_t* const sVlo = sV + V_HALVES;
+        const int t_base = tile * kBN;
+
+        // K fragments of block mb, k-steps s0, s0 + 1 (hi and lo)
+        constexpr int QB = 1;                  // k-steps per batch
+        constexpr int NQB = KSTEPS / QB;       // batches per block
+        auto read_k = [&](int mb, int qb, f16x8* fh, f16x8* fl) {
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) s_acc[mb][i] = 0.f;
-        if (work) {
-            constexpr int QB = 4;
-            constexpr int PER_MB = KSTEPS / QB;
-            constexpr int NBATCH = 2 * PER_MB;
-            f16x8 fh[2][QB], fl[2][QB];
-            auto read_batch = [&](int bi, f16x8* ph, f16x8* pl) {
-                const int mb = bi / PER_MB, s0 = (bi % PER_MB) * QB;
-#pragma unroll
-                for (int j = 0; j < QB; ++j) {
-                    ph[j] = *(const f16x8*)&sK[(32 * mb + l32) * K_STRIDE + 16 * (s0 + j) + 8 * hh];
-                    if (!KV16) pl[j] = *(const f16x8*)&sKlo[(32 * mb + l32) * K_STRIDE + 16 * (s0 + j) + 8 * hh];
-                }
-            };
-            read_batch(0, fh[0], fl[0]);
-#pragma unroll
-            for (int bi = 0; bi < NBATCH; ++bi) {
-                if (bi + 1 < NBATCH) read_batch(bi + 1, fh[(bi + 1) & 1], fl[(bi + 1) & 1]);
-                __builtin_amdgcn_sched_barrier(0); // keep the requests ahead of the products (the scheduler would sink them)
-                const int mb = bi / PER_MB, s0 = (bi % PER_MB) * QB;
-#pragma unroll
-                for (int j = 0; j < QB; ++j) {
-                    if (!KV16) s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl[bi & 1][j], qf[s0 + j], s_acc[mb], 0, 0, 0);
-                    s_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fh[bi & 1][j], qf[s0 + j], s_acc[mb], 0, 0, 0);
-                }
-                // between the batches: slices of tile + 1 into the other buffer (every wave is past its reads of
-                // that buffer since the barrier that ended the previous iteration; after the last tile the slices
-                // rewrite stale bytes into the idle buffer, which keeps this code free of branches)
-#pragma unroll
-                for (int k = 0; k < N_SLICES; ++k)
-                    if (bi == k * NBATCH / N_SLICES) store_slice((tile & 1) ^ 1, k);
+            for (int j = 0; j < QB; ++j) {
+                fh[j] = *(const f16x8*)&sK[k_frag_off + 32 * mb * K_STRIDE + 16 * (qb * QB + j)];
+                if (!KV16) fl[j] = *(const f16x8*)&sKlo[k_frag_off + 32 * mb * K_STRIDE + 16 * (qb * QB + j)];
             }
-        } else {
+        };
+        auto mul_k = [&](f32x16& acc, int qb, const f16x8* fh, const f16x8* fl) {
 #pragma unroll
-            for (int k = 0; k < N_SLICES; ++k) store_slice((tile & 1) ^ 1, k);
-        }
+            for (int j = 0; j < QB; ++j) {
+                if (!KV16) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl[j], qf[qb * QB + j], acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fh[j], qf[qb * QB + j], acc, 0, 0, 0);
+            }
+        };
+        // V^T fragments of block mb, 16-token step t, channel blocks cb0, cb0 + 1: element j of a fragment is token
+        // 32 mb + 16 t + 8 (j / 4) + 4 hh + j % 4, the token of element 8 t + j of the lane's S^T accumulator
+        constexpr int VB = 1;                  // channel blocks per batch
+        constexpr int NVB = 2 * CB / VB;       // batches per block: (t, pair of channel blocks)
+        auto read_vt = [&](const half_t* base, int mb, int t, int cb) -> f16x8 {
+            typedef short s16x4 __attribute__((ext_vector_type(4)));
+            typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
+            const half_t* p = base + v_frag_off + (32 * mb + 16 * t) * V_STRIDE + 32 * cb;
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 8 * V_STRIDE));
+            return bitcast<f16x8>(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        };
+        auto read_v = [&](int mb, int vb, f16x8* fh, f16x8* fl) {
+            const int t = vb / (CB / VB), cb0 = (vb % (CB / VB)) * VB;
+#pragma unroll
+            for (int j = 0; j < VB; ++j) {
+                fh[j] = read_vt(sV, mb, t, cb0 + j);
+                if (!KV16) fl[j] = read_vt(sVlo, mb, t, cb0 + j);
+            }
+        };
+        auto mul_v = [&](int vb, const f16x8* fh, const f16x8* fl, const f16x8* ph, const f16x8* pl) {
+            const int t = vb / (CB / VB), cb0 = (vb % (CB / VB)) * VB;
+#pragma unroll
+            for (int j = 0; j < VB; ++j) {
+                if (!KV16) o_acc[cb0 + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fl[j], ph[t], o_acc[cb0 + j], 0, 0, 0);
+                o_acc[cb0 + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fh[j], pl[t], o_acc[cb0 + j], 0, 0, 0);
+                o_acc[cb0 + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fh[j], ph[t], o_acc[cb0 + j], 0, 0, 0);
+            }
+        };
 
-        // ---- then the raw bytes of tile + 2 ----
-        if (tile + 2 < n_tiles) {
-            load_tile(tile + 2, row_next);
-            row_next = tile_row(tile + 3);
-        }
-
-        if (work) {
-            // ---- online softmax per column (element i <-> token 32 mb + 8 (i/4) + 4 hh + i%4) ----
-            const int t_base = tile * kBN;
-            // only the tiles that reach beyond a column's limit need the per-element test (wave-uniform branch)
-            const bool need_mask = __builtin_amdgcn_ballot_w64(t_base + kBN > lim) != 0;
+        // ---- softmax of one block, in three parts so that products can be issued between them ----
+        // part A: the block's logits in log2 units where extra terms or limits apply, and the new running maximum
+        auto softmax_max = [&](f32x16& sacc, int mb) -> float {
             float mx = kNegBig;
             if (EXTRA) {
-                // additive terms per element (log2 units): mask value and alibi distance of (query row, token)
 #pragma unroll
-                for (int mb = 0; mb < 2; ++mb)
+                for (int i = 0; i < 16; ++i) {
+                    const int t = t_base + 32 * mb + 8 * (i >> 2) + 4 * hh + (i & 3);
+                    float v = -INFINITY;
+                    if (t < lim) {
+                        float add = 0.f;
+                        if (mask_row) add = (float)mask_row[t];
+                        if (a.alibi_slopes) add += a.is_causal ? slope * (float)t : -slope * fabsf((float)(pos_c + kvlen - qlen - t));
+                        v = __builtin_fmaf(sacc[i], sm_scale, add * kLog2e);
+                    }
+                    sacc[i] = v;
+                    mx = fmaxf(mx, v);
+                }
+            } else {
+                if (limit) { // wave-uniform: only the tiles that reach beyond a column's limit
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
                         const int t = t_base + 32 * mb + 8 * (i >> 2) + 4 * hh + (i & 3);
-                        float v = -INFINITY;
-                        if (t < lim) {
-                            float add = 0.f;
-                            if (mask_row) add = (float)mask_row[t];
-                            if (a.alibi_slopes) add += a.is_causal ? slope * (float)t : -slope * fabsf((float)(pos_c + kvlen - qlen - t));
-                            v = __builtin_fmaf(s_acc[mb][i], sm_scale, add * kLog2e);
-                        }
-                        s_acc[mb][i] = v;
-                        mx = fmaxf(mx, v);
+                        if (t >= lim) sacc[i] = -INFINITY;
                     }
-            } else {
-                // maximum of the raw dot products; the (positive) logit scale is applied to it afterwards
-                if (need_mask) {
-#pragma unroll
-                    for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-                        for (int i = 0; i < 16; ++i) {
-                            const int t = t_base + 32 * mb + 8 * (i >> 2) + 4 * hh + (i & 3);
-                            if (t >= lim) s_acc[mb][i] = -INFINITY;
-                        }
                 }
+                // maximum of the raw dot products; the (positive) logit scale is applied to it afterwards
 #pragma unroll
-                for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[mb][i]);
+                for (int i = 0; i < 16; i += 2) mx = max3(mx, sacc[i], sacc[i + 1]);
                 mx *= sm_scale;
             }
             mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float m_new = fmaxf(m_run, mx);
-            // the running max moves rarely once a few tiles have been seen: rescale only then (wave-uniform)
-            if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
-                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-                l_run *= alpha;
+            return fmaxf(m_run, mx);
+        };
+        // part B: p = 2^(logit - max) as hi + lo halves (hi = p rounded toward zero, two at a time; lo = the exact
+        // remainder), elements [i0, i1) of the block
+        auto softmax_exp = [&](const f32x16& sacc, float bias, int i0, int i1, f16x8* ph, f16x8* pl, float& lsum) {
 #pragma unroll
-                for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) o_acc[cb][i] *= alpha;
-                m_run = m_new;
+            for (int i = 0; i < 16; i += 2) {
+                if (i < i0 || i >= i1) continue;
+                const float p0 = __builtin_amdgcn_exp2f(EXTRA ? sacc[i] + bias : __builtin_fmaf(sacc[i], sm_scale, bias));
+                const float p1 = __builtin_amdgcn_exp2f(EXTRA ? sacc[i + 1] + bias : __builtin_fmaf(sacc[i + 1], sm_scale, bias));
+                lsum += p0 + p1;
+                const half2_t h2 = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(p0, p1));
+                const half2_t l2 = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(sub_half_lo(p0, h2), sub_half_hi(p1, h2)));
+                ph[i >> 3][i & 7] = h2.x;
+                ph[i >> 3][(i & 7) + 1] = h2.y;
+                pl[i >> 3][i & 7] = l2.x;
+                pl[i >> 3][(i & 7) + 1] = l2.y;
             }
-            const float bias = kPShift - m_run;
-            // p = hi + lo in halves: hi = p rounded toward zero (two at a time), lo = the exact remainder
-            f16x8 pf[2][2], pfl[2][2];
-            float lsum = 0.f;
+        };
+        auto rescale = [&](float m_new) {
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            l_run *= alpha;
 #pragma unroll
-            for (int mb = 0; mb < 2; ++mb)
+            for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
-                for (int i = 0; i < 16; i += 2) {
-                    const float p0 = __builtin_amdgcn_exp2f(EXTRA ? s_acc[mb][i] + bias : __builtin_fmaf(s_acc[mb][i], sm_scale, bias));
-                    const float p1 = __builtin_amdgcn_exp2f(EXTRA ? s_acc[mb][i + 1] + bias : __builtin_fmaf(s_acc[mb][i + 1], sm_scale, bias));
-                    lsum += p0 + p1;
-                    const half2_t ph = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(p0, p1));
-                    const half2_t pl = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(sub_half_lo(p0, ph), sub_half_hi(p1, ph)));
-                    pf[mb][i >> 3][i & 7] = ph.x;
-                    pf[mb][i >> 3][(i & 7) + 1] = ph.y;
-                    pfl[mb][i >> 3][i & 7] = pl.x;
-                    pfl[mb][i >> 3][(i & 7) + 1] = pl.y;
-                }
-            l_run += lsum;
+                for (int i = 0; i < 16; ++i) o_acc[cb][i] *= alpha;
+            m_run = m_new;
+        };
+#define PMX_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-            // ---- O^T += V^T P^T : fragment batches of one (32-token block, 16-token step) each, read one ahead ----
-            {
-                f16x8 vh[2][CB], vl[2][CB];
-                auto read_batch = [&](int bi, f16x8* ph, f16x8* pl) {
-                    const int mb = bi >> 1, t = bi & 1;
+        f32x16 s0, s1;
 #pragma unroll
-                    for (int cb = 0; cb < CB; ++cb) {
-                        ph[cb] = *(const f16x8*)&sV[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
-                        if (!KV16) pl[cb] = *(const f16x8*)&sVlo[(32 * cb + l32) * V_STRIDE + 32 * mb + 16 * t + 8 * hh];
-                    }
-                };
-                read_batch(0, vh[0], vl[0]);
+        for (int i = 0; i < 16; ++i) {
+            s0[i] = 0.f;
+            s1[i] = 0.f;
+        }
+        f16x8 fh[2][QB > VB ? QB : VB], fl[2][QB > VB ? QB : VB];
+        f16x8 p0h[2], p0l[2], p1h[2], p1l[2];
+
+        // ---- phase 1: S^T(b0) with the dequantisation of tile + 1 into the other buffer (every wave is past its
+        // reads of that buffer since the barrier that ended the previous iteration; after the last tile the slices
+        // rewrite stale bytes into the idle buffer, which keeps this code free of branches) ----
+        read_k(0, 0, fh[0], fl[0]);
 #pragma unroll
-                for (int bi = 0; bi < 4; ++bi) {
-                    if (bi + 1 < 4) read_batch(bi + 1, vh[(bi + 1) & 1], vl[(bi + 1) & 1]);
-                    __builtin_amdgcn_sched_barrier(0);
-                    const int mb = bi >> 1, t = bi & 1;
+        for (int qb = 0; qb < NQB; ++qb) {
+            if (qb + 1 < NQB) read_k(0, qb + 1, fh[(qb + 1) & 1], fl[(qb + 1) & 1]);
+            else read_k(1, 0, fh[(qb + 1) & 1], fl[(qb + 1) & 1]);
+            PMX_FENCE();
+            mul_k(s0, qb, fh[qb & 1], fl[qb & 1]);
+            PMX_FENCE();
 #pragma unroll
-                    for (int cb = 0; cb < CB; ++cb) {
-                        if (!KV16) o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vl[bi & 1][cb], pf[mb][t], o_acc[cb], 0, 0, 0);
-                        o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vh[bi & 1][cb], pfl[mb][t], o_acc[cb], 0, 0, 0);
-                        o_acc[cb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vh[bi & 1][cb], pf[mb][t], o_acc[cb], 0, 0, 0);
-                    }
+            for (int k = 0; k < N_SLICES; ++k)
+                if (qb == k * NQB / N_SLICES) store_slice(buf ^ 1, k);
+            PMX_FENCE();
+        }
+
+        // ---- phase 2: S^T(b1) with the softmax of b0 ----
+        float lsum = 0.f;
+        float m_new = 0.f, bias = 0.f;
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb) {
+            if (qb + 1 < NQB) read_k(1, qb + 1, fh[(NQB + qb + 1) & 1], fl[(NQB + qb + 1) & 1]);
+            PMX_FENCE();
+            mul_k(s1, qb, fh[(NQB + qb) & 1], fl[(NQB + qb) & 1]);
+            PMX_FENCE();
+            if (qb == 0) {
+                // the raw bytes of tile + 2: their registers were freed by phase 1, and the requests have the rest of
+                // this tile and phase 1 of the next to complete
+                if (tile + 2 < n_tiles) {
+                    load_tile(tile + 2, row_next);
+                    row_next = tile_row(tile + 3);
                 }
+                m_new = softmax_max(s0, 0);
+                // the running max moves rarely once a few tiles have been seen: rescale only then (wave-uniform)
+                if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) rescale(m_new);
+                bias = kPShift - m_run;
+            }
+            if (NQB == 1) softmax_exp(s0, bias, 0, 16, p0h, p0l, lsum);
+            else if (qb >= 1 || NQB == 2) {
+                // the 16 elements over the remaining batches
+                const int parts = NQB == 2 ? 2 : NQB - 1, part = NQB == 2 ? qb : qb - 1;
+                softmax_exp(s0, bias, 16 * part / parts & ~1, 16 * (part + 1) / parts & ~1, p0h, p0l, lsum);
+            }
+            PMX_FENCE();
+        }
+        l_run += lsum;
+
+        // ---- phase 3: O^T += V^T P^T of b0 with the softmax of b1 ----
+        lsum = 0.f;
+        float m_b1 = 0.f;
+        read_v(0, 0, fh[0], fl[0]);
+#pragma unroll
+        for (int vb = 0; vb < NVB; ++vb) {
+            if (vb + 1 < NVB) read_v(0, vb + 1, fh[(vb + 1) & 1], fl[(vb + 1) & 1]);
+            else read_v(1, 0, fh[(vb + 1) & 1], fl[(vb + 1) & 1]);
+            PMX_FENCE();
+            mul_v(vb, fh[vb & 1], fl[vb & 1], p0h, p0l);
+            PMX_FENCE();
+            if (vb == 0) {
+                m_b1 = softmax_max(s1, 1);
+                bias = kPShift - m_b1; // b1's probabilities are taken against the maximum that includes b1
+            }
+            softmax_exp(s1, bias, 16 * vb / NVB & ~1, 16 * (vb + 1) / NVB & ~1, p1h, p1l, lsum);
+            PMX_FENCE();
+        }
+        // b1 raised the maximum: what has been accumulated so far, the products of b0 included, is rescaled
+        if (__builtin_amdgcn_ballot_w64(m_b1 > m_run) != 0) rescale(m_b1);
+        l_run += lsum;
+
+        // ---- phase 4: O^T += V^T P^T of b1; the raw bytes of tile + 2 are requested after the first batch ----
+#pragma unroll
+        for (int vb = 0; vb < NVB; ++vb) {
+            if (vb + 1 < NVB) read_v(1, vb + 1, fh[(NVB + vb + 1) & 1], fl[(NVB + vb + 1) & 1]);
+            PMX_FENCE();
+            mul_v(vb, fh[(NVB + vb) & 1], fl[(NVB + vb) & 1], p1h, p1l);
+            PMX_FENCE();
+            PMX_FENCE();
+        }
+#undef PMX_FENCE
+    };
+
+    for (int tile = 0; tile < n_tiles; ++tile) {
+        if (tile * kBN < wave_lim) {
+            tile_body(tile, (tile + 1) * kBN > wave_lim_min);
+        } else {
+#pragma unroll
+            for (int k = 0; k < N_SLICES; ++k) store_slice((tile & 1) ^ 1, k);
+            if (tile + 2 < n_tiles) {
+                load_tile(tile + 2, row_next);
+                row_next = tile_row(tile + 3);
             }
         }
         __syncthreads(); // tile + 1 is complete in its buffer; this tile's buffer may be overwritten
@@ -619,14 +643,15 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
                 *(f16x4*)(op + 32 * cb + 8 * r + 4 * hh) = w;
             }
     }
+    } // items
 }
 
 template <int D, int SRC>
 constexpr size_t prefill_lds_bytes()
 {
-    // int8 source: K hi/lo tiles + transposed V hi/lo tiles (above the 64 KB static limit for D = 128, hence
-    // dynamic); fp16 source: one K tile and one transposed V tile; two buffers of each
-    return 2 * (SRC == 2 ? 1 : 2) * (kBN * (D + 8) + D * (kBN + 8)) * sizeof(half_t);
+    // int8 source: K hi/lo tiles + V hi/lo tiles (above the 64 KB static limit for D = 128, hence dynamic);
+    // fp16 source: one K tile and one V tile; two buffers of each
+    return 2 * (SRC == 2 ? 1 : 2) * kBN * (PrefillTile<D>::K_STRIDE + PrefillTile<D>::V_STRIDE) * sizeof(half_t);
 }
 
 template <int D, int SRC, bool EXTRA>
