@@ -216,6 +216,22 @@ def main():
     if bt.batch > bt.decoding_batches:
         stages["prefill"] = time_stage(lambda: op.forward_prefill(stream), n_ev)
 
+    # the projection behind the attention (single-rank row_parallel_linear) on this step's decode rows: a square
+    # weight of (heads * head_dim)^2 halves, streamed once per call
+    hidden = bt.num_heads * bt.head_dim
+    w_proj = (torch.randn((hidden, hidden), device="cuda") * hidden ** -0.5).to(torch.float16)
+    proj_in = dev.output[:bt.decoding_batches]
+    proj_out = torch.empty((bt.decoding_batches, hidden), dtype=torch.float16, device="cuda")
+    proj_ws_bytes = ops.row_parallel_linear_workspace_size(bt.decoding_batches, hidden, hidden)
+    proj_ws = torch.empty(proj_ws_bytes, dtype=torch.uint8, device="cuda") if proj_ws_bytes else None
+    stages["o_proj"] = time_stage(lambda: ops.row_parallel_linear(proj_in, w_proj, None, proj_out, workspace=proj_ws), n_ev)
+    proj_replays = None
+    if not args.eager:
+        try:
+            proj_replays = replay_times(lambda st: ops.row_parallel_linear(proj_in, w_proj, None, proj_out, workspace=proj_ws, stream=st))
+        except Exception:
+            torch.cuda.synchronize()
+
     if args.calibration_copy_mib:
         src = torch.ones(args.calibration_copy_mib << 20, dtype=torch.int8, device="cuda")
         dst = torch.empty_like(src)
@@ -276,6 +292,14 @@ def main():
             "frac_launch_loop": dec_bytes / (t_ranges["avg_us"] * 1e-6) / 1e9 / HBM_PEAK_GBS,
         },
     }
+    proj_us = float(np.mean(proj_replays)) if proj_replays else stages["o_proj"]["avg_us"]
+    proj_bytes = hidden * hidden * 2
+    out["o_proj"] = {"kernel": "split_linear_kernel + linear_reduce_kernel" if proj_ws_bytes else "split_linear_kernel", "rows": int(bt.decoding_batches), "in_features": hidden,
+                     "out_features": hidden, "bound": "hbm", "weight_bytes": proj_bytes, "kernel_us": proj_us,
+                     "achieved": proj_bytes / (proj_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": proj_bytes / (proj_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                     "kernel_us_launch_loop": stages["o_proj"]["avg_us"],
+                     "note": "not part of `value`: the step after the layer call, timed on its own"}
     if "prefill" in stages:
         fl = bt.prefill_flops()
         pf_us = float(np.mean(prefill_replays)) if prefill_replays else stages["prefill"]["avg_us"]

@@ -439,6 +439,28 @@ PMXHIP_API int pmxhip_rotary_position_embedding(const pmxhip_rope_params* p, pmx
 PMXHIP_API int pmxhip_rope_kv_cache_quantize(const pmxhip_rope_params* rope, const pmxhip_kvstore_params* store,
                                              pmxhip_stream_t stream);
 
+/* ---- output projection behind the attention ---------------------------------------
+ * Replaces the single-rank case of ppl::kernel::llm::cuda::pmx::row_parallel_linear
+ * (include/ppl/kernel/llm/cuda/pmx/row_parallel_linear.h:28-46,
+ * src/ppl/kernel/llm/cuda/pmx/row_parallel_linear.cu:25-110): output(M, N) = input(M, K) * weight(N, K)^T + bias
+ * with half tensors and float32 accumulation, where the reference calls one cublasLt GEMM and, with more than
+ * one rank, an all-reduce (one GPU here, so none).  The attention output (B, Hq * D) is this call's input in
+ * place.  bias may be NULL.  Strides are in halves per row.  Needs N % 16 == 0, K % 32 == 0, 16-byte aligned
+ * rows of input and weight and 8-byte aligned rows of output and bias; anything else returns
+ * PMXHIP_UNSUPPORTED.  Written for the decode step (M up to a few hundred rows: bound by streaming the
+ * K * N * 2 weight bytes); larger M is served 128 rows at a time.
+ * workspace: at decode sizes there are fewer blocks of 64 output columns than CUs, so the k range is split over
+ * several workgroups whose float32 partial tiles pass through `workspace` (the role of the reference's
+ * cublas_workspace argument) and are added in a fixed order by a second kernel.
+ * pmxhip_row_parallel_linear_workspace_size gives the bytes that serve (M, in_features, out_features) on the
+ * current device (0 = none needed); with a NULL or smaller workspace the call still computes the same function,
+ * one k range per column block (slower at decode sizes).  The workspace needs 16-byte alignment and no clearing. */
+PMXHIP_API int64_t pmxhip_row_parallel_linear_workspace_size(int64_t m, int64_t in_features, int64_t out_features);
+PMXHIP_API int pmxhip_row_parallel_linear(pmxhip_stream_t stream, const void* input, const void* weight, const void* bias,
+                                          int64_t m, int64_t in_features, int64_t out_features, int64_t input_stride,
+                                          int64_t weight_stride, int64_t output_stride, int64_t workspace_size,
+                                          void* workspace, void* output);
+
 /* One-time set-up on the current device, for callers that record their first step under stream capture: the
  * attribute calls of the kernels with large dynamic LDS (otherwise made at each kernel's first launch, which a
  * capturing stream refuses with PMXHIP_OTHER_ERROR) and the address of the static workspace.  Optional

@@ -69,6 +69,8 @@ def lib():
             [_vp] * 4 + [_f32, _i32] + [_i64] * 6 + [_i32, _f32] + [_i64] * 4 + [_vp] * 2)
         _lib.pmx_oracle_kv_cache_reorder.restype = ctypes.c_int
         _lib.pmx_oracle_kv_cache_reorder.argtypes = [_i32] + [_vp] * 6 + [_i64] * 8
+        _lib.pmx_oracle_row_parallel_linear.restype = ctypes.c_int
+        _lib.pmx_oracle_row_parallel_linear.argtypes = [_vp] * 3 + [_i64] * 6 + [_vp]
     return _lib
 
 
@@ -300,3 +302,18 @@ def rotary_position_embedding(query, key, start_pos, seqstarts, theta, rotary_di
     if rc != 0:
         raise ValueError("oracle rope rejected the arguments (rc=%d)" % rc)
     return rq, rk
+
+
+def row_parallel_linear(input, weight, bias=None):
+    """input [M, K], weight [N, K], bias [N] or None, all float16 -> output [M, N] float16 (float32 accumulate)."""
+    input = _c(input, np.float16)
+    weight = _c(weight, np.float16)
+    m, k = input.shape
+    n = weight.shape[0]
+    assert weight.shape[1] == k
+    b = _c(bias, np.float16) if bias is not None else None
+    out = np.zeros((m, n), dtype=np.float16)
+    rc = lib().pmx_oracle_row_parallel_linear(_p(input), _p(weight), _p(b) if b is not None else None, m, n, k, k, k, n, _p(out))
+    if rc != 0:
+        raise ValueError("oracle row_parallel_linear rejected the arguments (rc=%d)" % rc)
+    return out

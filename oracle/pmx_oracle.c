@@ -33,6 +33,11 @@
  *                                  parity unpinned.
  *   pmx_oracle_splitkv_combine     pinned: any split of the kv range equals the
  *                                  single pass (log-sum-exp associativity).
+ *   pmx_oracle_row_parallel_linear pinned: numpy matmul in binary64 of the same half inputs; exact
+ *                                  small-integer products; identity weight = copy; bias alone for a
+ *                                  zero input; linearity in the input.  The reference's own bits come
+ *                                  from cublasLt (row_parallel_linear.cu:61-84, algorithm chosen at run
+ *                                  time): parity unpinned at the bit level, inside the stated tolerance.
  *   The reference itself cannot be compiled here (CUDA, inline PTX, CUTLASS, and
  *   dependencies fetched at configure time), so bit patterns of its fp16
  *   attention output are "parity unpinned"; the contract is the fp32
@@ -670,6 +675,29 @@ int pmx_oracle_rotary_position_embedding(
                         }
                     }
                 }
+        }
+    }
+    return 0;
+}
+
+/* Single-rank row_parallel_linear (src/ppl/kernel/llm/cuda/pmx/row_parallel_linear.cu:25-110 with
+ * nccl_param->size == 1): output(M, N) = input(M, K) * weight(N, K)^T + bias, half tensors; the reference's
+ * cublasLt GEMM accumulates in float32 and rounds once to half (alpha 1, beta 0, bias as epilogue).  Here the
+ * float32 sum runs over k in index order.  Strides in halves per row.  bias may be NULL. */
+int pmx_oracle_row_parallel_linear(const uint16_t* input, const uint16_t* weight, const uint16_t* bias, int64_t m, int64_t n,
+                                   int64_t k, int64_t input_stride, int64_t weight_stride, int64_t output_stride,
+                                   uint16_t* output)
+{
+    if (m < 0 || n < 0 || k < 0 || !input || !weight || !output) return 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < m; ++i) {
+        for (int64_t j = 0; j < n; ++j) {
+            const uint16_t* a = input + i * input_stride;
+            const uint16_t* w = weight + j * weight_stride;
+            float acc = 0.0f;
+            for (int64_t c = 0; c < k; ++c) acc += pmx_oracle_half_to_float(a[c]) * pmx_oracle_half_to_float(w[c]);
+            if (bias) acc += pmx_oracle_half_to_float(bias[j]);
+            output[i * output_stride + j] = pmx_oracle_float_to_half(acc);
         }
     }
     return 0;

@@ -34,6 +34,7 @@ EXPORTED_SYMBOLS = (
     "pmxhip_mhca_forward",
     "pmxhip_kv_cache_reorder", "pmxhip_kv_cache_invert_reorder",
     "pmxhip_rotary_position_embedding", "pmxhip_rope_kv_cache_quantize",
+    "pmxhip_row_parallel_linear", "pmxhip_row_parallel_linear_workspace_size",
 )
 
 
@@ -209,6 +210,10 @@ def lib():
     L.pmxhip_key_value_cache.argtypes = [c_vp] * 6 + [c_i64] * 6 + [c_i32] + [c_i64] * 6 + [c_vp] * 2
     L.pmxhip_decode_plan_make.restype = ctypes.c_int
     L.pmxhip_decode_plan_make.argtypes = [c_i64] * 5 + [c_i32, c_i32, ctypes.POINTER(DecodePlan)]
+    L.pmxhip_row_parallel_linear.restype = ctypes.c_int
+    L.pmxhip_row_parallel_linear.argtypes = [c_vp] * 4 + [c_i64] * 7 + [c_vp, c_vp]
+    L.pmxhip_row_parallel_linear_workspace_size.restype = c_i64
+    L.pmxhip_row_parallel_linear_workspace_size.argtypes = [c_i64] * 3
     L.pmxhip_init.restype = ctypes.c_int
     L.pmxhip_init.argtypes = []
     L.pmxhip_decode_plan_make_kernel.restype = ctypes.c_int

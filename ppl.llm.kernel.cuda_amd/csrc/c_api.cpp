@@ -639,4 +639,40 @@ int pmxhip_rope_kv_cache_quantize(const pmxhip_rope_params* rope, const pmxhip_k
     return rope_common("rope_kv_cache_quantize", rope, store, stream);
 }
 
+int64_t pmxhip_row_parallel_linear_workspace_size(int64_t m, int64_t in_features, int64_t out_features)
+{
+    if (m <= 0 || in_features <= 0 || out_features <= 0) return 0;
+    return pmxhip::linear_workspace_bytes(m, out_features, in_features, current_compute_units());
+}
+
+int pmxhip_row_parallel_linear(pmxhip_stream_t stream, const void* input, const void* weight, const void* bias, int64_t m,
+                               int64_t in_features, int64_t out_features, int64_t input_stride, int64_t weight_stride,
+                               int64_t output_stride, int64_t workspace_size, void* workspace, void* output)
+{
+    if (m < 0 || in_features <= 0 || out_features <= 0) return fail(PMXHIP_INVALID_VALUE, "row_parallel_linear: bad sizes");
+    if (m == 0) return PMXHIP_SUCCESS;
+    if (!input || !weight || !output) return fail(PMXHIP_INVALID_VALUE, "row_parallel_linear: null device pointer");
+    if (out_features % 16 != 0 || in_features % 32 != 0)
+        return fail(PMXHIP_UNSUPPORTED, "row_parallel_linear: out_features must be a multiple of 16 and in_features of 32 "
+                                        "(got %lld, %lld)", (long long)out_features, (long long)in_features);
+    if (input_stride < in_features || weight_stride < in_features || output_stride < out_features)
+        return fail(PMXHIP_INVALID_VALUE, "row_parallel_linear: a row stride is shorter than its row");
+    if (!aligned16(input) || !aligned16(weight) || input_stride % 8 != 0 || weight_stride % 8 != 0 ||
+        (reinterpret_cast<uintptr_t>(output) & 7u) || output_stride % 4 != 0 || (bias && (reinterpret_cast<uintptr_t>(bias) & 7u)))
+        return fail(PMXHIP_UNSUPPORTED, "row_parallel_linear: input and weight rows must be 16-byte aligned, output rows and bias 8-byte aligned");
+    pmxhip::LinearLaunch a{};
+    a.input = input;
+    a.weight = weight;
+    a.bias = bias;
+    a.output = output;
+    a.m = m;
+    a.n = out_features;
+    a.k = in_features;
+    a.input_stride = input_stride;
+    a.weight_stride = weight_stride;
+    a.output_stride = output_stride;
+    return launch_result("row_parallel_linear",
+                         pmxhip::launch_linear(a, current_compute_units(), workspace, workspace ? workspace_size : 0, stream));
+}
+
 } // extern "C"

@@ -16,6 +16,7 @@
 #include "pmx_hip/key_value_cache.h"
 #include "pmx_hip/kv_cache_reorder.h"
 #include "pmx_hip/rotary_position_embedding.h"
+#include "pmx_hip/row_parallel_linear.h"
 
 namespace ppl { namespace kernel { namespace llm { namespace cuda { namespace pmx {
 
@@ -539,6 +540,38 @@ ppl::common::RetCode dynamic_batching_rotary_position_embedding_kv_cache(
     st.max_seqlen = max_seqlen;
     st.cache_mode = cache_mode;
     return to_retcode(pmxhip_rope_kv_cache_quantize(&p, &st, stream));
+}
+
+ppl::common::RetCode row_parallel_linear(
+    const hipStream_t stream,
+    const ppl::common::TensorShape* input_shape, const void* input,
+    const ppl::common::TensorShape* weight_shape, const void* weight,
+    const ppl::common::TensorShape* bias_shape, const void* bias,
+    const int64_t in_features, const int64_t out_features,
+    const bool input_is_parallel,
+    const int64_t workspace_size, void* workspace,
+    const ppl::common::TensorShape* output_shape, void* output)
+{
+    (void)bias_shape;
+    (void)output_shape;
+    if (!input_is_parallel) { // row_parallel_linear.cu:46-49
+        PMX_LOG_ERROR("currnetly only support parallel input");
+        return ppl::common::RC_UNSUPPORTED;
+    }
+    if (input_shape->GetDataType() != ppl::common::DATATYPE_FLOAT16 || weight_shape->GetDataType() != ppl::common::DATATYPE_FLOAT16) {
+        PMX_LOG_ERROR("row_parallel_linear only supports fp16");
+        return ppl::common::RC_UNSUPPORTED;
+    }
+    // M = all dimensions of the input but the last (row_parallel_linear.cu:55)
+    int64_t m = 1;
+    for (uint32_t i = 0; i + 1 < input_shape->GetDimCount(); ++i) m *= input_shape->GetDim(i);
+    return to_retcode(pmxhip_row_parallel_linear(stream, input, weight, bias, m, in_features, out_features, in_features, in_features,
+                                                 out_features, workspace_size, workspace, output));
+}
+
+int64_t row_parallel_linear_workspace_size(const int64_t m, const int64_t in_features, const int64_t out_features)
+{
+    return pmxhip_row_parallel_linear_workspace_size(m, in_features, out_features);
 }
 
 }}}}} // namespace ppl::kernel::llm::cuda::pmx

@@ -156,6 +156,19 @@ constexpr int kLaunchOk = 0;
 constexpr int kLaunchNoKernel = 1;      // no kernel serves the shape
 constexpr int kLaunchNeedsWarmup = 2;   // the kernel's one-time attribute call is due, but the stream is being captured
 
+// output(M, N) = input(M, K) * weight(N, K)^T + bias; half everywhere, strides in halves per row
+struct LinearLaunch {
+    const void* input;
+    const void* weight;
+    const void* bias;   // half (N) or nullptr
+    void* output;
+    int64_t m, n, k;
+    int64_t input_stride, weight_stride, output_stride;
+};
+// workspace: float32 partial tiles of the k ranges (linear_workspace_bytes; may be null: then one k range)
+int launch_linear(const LinearLaunch& a, int compute_units, void* workspace, int64_t workspace_bytes, hipStream_t stream);
+int64_t linear_workspace_bytes(int64_t m, int64_t n, int64_t k, int compute_units);
+
 // The one-time hipFuncSetAttribute of a kernel whose dynamic LDS exceeds the default limit.  It runs before the
 // kernel's first launch in the process (one GPU per process) and never while `stream` is being captured into a
 // graph: a caller that captures first gets kLaunchNeedsWarmup and calls pmxhip_init() or one eager step before.

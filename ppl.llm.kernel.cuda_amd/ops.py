@@ -290,6 +290,33 @@ def kv_cache_invert_reorder(outer_mem, page_ids, src_stride, dst_stride, *, laye
     return rc
 
 
+def row_parallel_linear_workspace_size(m, in_features, out_features):
+    """Bytes of workspace that let row_parallel_linear split the k range over the CUs (0 = none needed)."""
+    return int(_lib.lib().pmxhip_row_parallel_linear_workspace_size(m, in_features, out_features))
+
+
+def row_parallel_linear(input, weight, bias, output, *, workspace=None, stream=None, check=True):
+    """output (M, N) = input (M, K) @ weight (N, K)^T + bias (N) or None; fp16 tensors, rows contiguous along their
+    last dimension (row strides may exceed the row).  The single-rank case of the reference's row_parallel_linear.
+    `workspace`: a uint8 tensor of row_parallel_linear_workspace_size bytes, or None (slower at decode sizes)."""
+    n, k = int(weight.shape[0]), int(weight.shape[1])
+    m = input.numel() // k  # a contiguous (B, Hq, D) attention output is the (B, Hq * D) input in place
+
+    def row_stride(t, width):
+        if t.is_contiguous():
+            return width
+        if t.dim() != 2 or t.stride(1) != 1:
+            raise ValueError("a tensor with padded rows must be 2-d with unit stride along the row")
+        return int(t.stride(0))
+    rc = _lib.lib().pmxhip_row_parallel_linear(_stream(stream), _ptr(input), _ptr(weight), _ptr(bias), m, k, n,
+                                               row_stride(input, k), row_stride(weight, k), row_stride(output, n),
+                                               0 if workspace is None else workspace.numel() * workspace.element_size(),
+                                               _ptr(workspace), _ptr(output))
+    if check and rc != RC_SUCCESS:
+        raise PmxError(rc, "row_parallel_linear")
+    return rc
+
+
 class DynamicBatchingMultiHeadCacheAttention:
     """The operator class (C++ `dynamic_batching_multi_head_cache_attention`) behind its C handle."""
 

@@ -11,6 +11,7 @@
 #include "pmx_hip/key_value_cache.h"
 #include "pmx_hip/kv_cache_reorder.h"
 #include "pmx_hip/rotary_position_embedding.h"
+#include "pmx_hip/row_parallel_linear.h"
 
 namespace pmx = ppl::kernel::llm::cuda::pmx;
 
@@ -124,5 +125,14 @@ int main()
                                                            cachestarts, start_pos, 0, 1, num_layer, layer_idx, num_kv_heads,
                                                            head_dim, 1, 128, cache_stride_s, cache_stride_l, cache_stride_h,
                                                            cache_stride_kv, 64, cache, scale));
+    // the projection behind the attention: the reference's argument list without its cuBLASLt / NCCL arguments
+    ppl::common::TensorShape no_rows(ppl::common::DATATYPE_FLOAT16, {0, num_heads * head_dim});
+    ppl::common::TensorShape weight_shape(ppl::common::DATATYPE_FLOAT16, {4096, num_heads * head_dim});
+    ppl::common::TensorShape bias_shape(ppl::common::DATATYPE_FLOAT16, {4096});
+    printf("linear(no rows)=%u linear(not parallel)=%u\n",
+           (unsigned)pmx::row_parallel_linear(stream, &no_rows, output, &weight_shape, cache, &bias_shape, nullptr,
+                                              num_heads * head_dim, 4096, true, 0, nullptr, &no_rows, query),
+           (unsigned)pmx::row_parallel_linear(stream, &no_rows, output, &weight_shape, cache, &bias_shape, nullptr,
+                                              num_heads * head_dim, 4096, false, 0, nullptr, &no_rows, query));
     return 0;
 }

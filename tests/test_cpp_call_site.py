@@ -1,7 +1,7 @@
 """The drop-in claim at the source level, on the CPU: tests/callsite/call_site.cpp -- a translation unit that calls
 heuristic_prepare with the reference's 40 arguments (multi_head_cache_attention.h:107-148), the stage functions,
-kv_cache_reorder / kv_cache_invert_reorder and dynamic_batching_rotary_position_embedding through the reference's
-prototypes -- is compiled with g++ against include/pmx_hip/*.h, linked with libpmx_hip.so and run.  No GPU: the
+kv_cache_reorder / kv_cache_invert_reorder, dynamic_batching_rotary_position_embedding and row_parallel_linear
+through the reference's prototypes -- is compiled with g++ against include/pmx_hip/*.h, linked with libpmx_hip.so and run.  No GPU: the
 prepare step is host code and the stage calls are made on an empty batch."""
 import os
 import subprocess
@@ -35,4 +35,5 @@ def test_reference_style_call_site_compiles_links_and_runs(pkg, hip_lib, tmp_pat
     assert lines[5] == "reorder(no pages)=0 invert(no pages)=0"
     assert lines[6] == "rope(empty batch)=0"
     assert lines[7] == "kvcache(empty batch)=0"
+    assert lines[8] == "linear(no rows)=0 linear(not parallel)=2"
     assert out is not None
