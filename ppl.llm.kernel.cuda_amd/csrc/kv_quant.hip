@@ -109,7 +109,8 @@ __device__ __forceinline__ Quantised quantise_group(const u32x4 raw)
 
 // largest b in [0, n) with starts[b] <= v   (starts non-decreasing, starts[0] <= v < starts[n]);
 // being the largest, it is never an empty sequence
-__device__ __forceinline__ int sequence_of(const int64_t* __restrict__ starts, int n, int64_t v)
+template <typename PTR>
+__device__ __forceinline__ int sequence_of(PTR starts, int n, int64_t v)
 {
     int lo = 0, hi = n - 1;
     while (lo < hi) {
@@ -125,19 +126,26 @@ __device__ __forceinline__ int sequence_of(const int64_t* __restrict__ starts, i
 // stride_tokens: tokens between a thread's units, (workgroups * threads) / groups_per_token; the host sizes the launch
 // so that this division is exact whenever a thread takes more than one unit, which keeps a thread on one
 // (head, channel group) for all its units: the two integer divisions below then happen once, not once per unit.
-template <bool PAGED>
+// WAVE_TOKEN: a token row has a multiple of 64 groups, so the 64 lanes of a wave always work on one token: what
+// follows from the token alone (its sequence, position, cache row and the row bases) is then found once per wave
+// on the scalar unit, with scalar loads of the index arrays, and a lane adds only its offset inside the row.
+template <bool PAGED, bool WAVE_TOKEN>
 __global__ __launch_bounds__(kQuantThreads) void kv_quantize_kernel(const QuantLaunch a, const uint32_t stride_tokens)
 {
     const uint32_t groups_per_head = (uint32_t)a.head_dim >> 3;
     const uint32_t groups_per_token = (uint32_t)a.num_kv_heads * groups_per_head;
-    const int64_t first = a.seqstarts[0];
-    const int64_t n_tokens = a.seqstarts[a.batch] - first;
+    const const_i64_ptr seqstarts = as_constant(a.seqstarts);
+    const const_i64_ptr start_pos = as_constant(a.start_pos);
+    const const_i64_ptr cachestarts = as_constant(a.cachestarts);
+    const int64_t first = seqstarts[0];
+    const int64_t n_tokens = seqstarts[a.batch] - first;
     const uint32_t u0 = blockIdx.x * kQuantThreads + threadIdx.x; // the host keeps workgroups * threads below 2^31
-    const uint32_t tok0 = u0 / groups_per_token;
+    uint32_t tok0 = u0 / groups_per_token;
     const uint32_t gi = u0 - tok0 * groups_per_token;
+    if (WAVE_TOKEN) tok0 = __builtin_amdgcn_readfirstlane(tok0);
     const uint32_t h = gi / groups_per_head;
     const uint32_t d0 = (gi - h * groups_per_head) << 3;
-    const int64_t in_idx = (int64_t)h * a.head_dim + d0;
+    const uint32_t in_idx = h * (uint32_t)a.head_dim + d0;                   // halves inside a K/V row
     const int64_t out_idx = a.layer_idx * a.cache_stride_l + (int64_t)h * a.cache_stride_h + d0;
     for (int64_t tok = tok0; tok < n_tokens; tok += stride_tokens) {
         const int64_t in_tok = first + tok;
@@ -151,15 +159,16 @@ __global__ __launch_bounds__(kQuantThreads) void kv_quantize_kernel(const QuantL
         int b;
         int64_t pos;
         const int64_t ti = tok < a.batch ? tok : 0;
-        const int64_t s0 = a.seqstarts[ti], s1 = a.seqstarts[ti + 1], sp = a.start_pos[ti];
+        const int64_t s0 = seqstarts[ti], s1 = seqstarts[ti + 1], sp = start_pos[ti];
         if (tok < a.batch && s0 == in_tok && s1 > in_tok) {
             b = (int)tok;
             pos = sp;
         } else {
-            b = sequence_of(a.seqstarts, (int)a.batch, in_tok);
-            pos = a.start_pos[b] + (in_tok - a.seqstarts[b]);
+            b = sequence_of(seqstarts, (int)a.batch, in_tok);
+            pos = start_pos[b] + (in_tok - seqstarts[b]);
         }
-        const int64_t row = token_row<PAGED>(a.cachestarts, PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b, pos);
+        const int64_t tb = PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b;
+        const int64_t row = PAGED ? cachestarts[tb + (pos >> 7)] + (pos & (kPage - 1)) : cachestarts[tb] + pos;
 
         const Quantised kq = quantise_group(kraw);
         const Quantised vq = quantise_group(vraw);
@@ -197,13 +206,79 @@ __global__ __launch_bounds__(kQuantThreads) void rope_append_kernel(const RopeLa
     if (tok0 >= n_tokens) return;
     const bool append = a.cache != nullptr;
 
+    // the rows of this workgroup's tokens, as units of 8 channels: the query heads' groups, then the key heads' (a
+    // key unit also carries the same group of V when the step appends)
+    const int gph = a.head_dim >> 3; // groups of 8 channels per head
+    const int q_units = (int)a.num_heads * gph;
+    const int k_units = (int)a.num_key_heads * gph;
+    const int units = q_units + k_units;
+    int n_here = tokens_per_wg;
+    if (tok0 + n_here > n_tokens) n_here = (int)(n_tokens - tok0);
+    const int work = n_here * units;
+
+    struct Unit {
+        int tl, h, d0;
+        bool is_query;
+        int64_t in_tok, idx;
+    };
+    auto unit_of = [&](int w) -> Unit {
+        Unit r;
+        r.tl = w / units;
+        int u = w - r.tl * units;
+        r.is_query = u < q_units;
+        if (!r.is_query) u -= q_units;
+        r.h = u / gph;
+        r.d0 = (u - r.h * gph) << 3;
+        r.in_tok = first + tok0 + r.tl;
+        r.idx = (int64_t)r.h * a.head_dim + r.d0;
+        return r;
+    };
+    auto load_row = [&](const Unit& r) -> u32x4 {
+        return r.is_query ? *(const u32x4*)((const half_t*)a.query + r.in_tok * a.query_stride_s + r.idx)
+                          : *(const u32x4*)((const half_t*)a.key + r.in_tok * a.key_stride_s + r.idx);
+    };
+    auto load_value = [&](const Unit& r) -> u32x4 {
+        return *(const u32x4*)((const half_t*)a.value + r.in_tok * a.value_stride_s + r.idx);
+    };
+
+    // A decode step has a token per workgroup and a few units per thread: the kernel's time is then a chain of
+    // latencies (index arrays -> cos/sin -> rows -> stores).  The rows depend on none of the rest, so they are
+    // requested first and travel while the coefficients are computed.
+    constexpr int kEarly = 3;
+    const bool early = work <= kEarly * kQuantThreads;
+    u32x4 early_row[kEarly], early_value[kEarly];
+    if (early) {
+#pragma unroll
+        for (int j = 0; j < kEarly; ++j) {
+            const int w = threadIdx.x + j * kQuantThreads;
+            early_row[j] = u32x4{0, 0, 0, 0};
+            early_value[j] = u32x4{0, 0, 0, 0};
+            if (w < work) {
+                const Unit r = unit_of(w);
+                early_row[j] = load_row(r);
+                if (append && !r.is_query) early_value[j] = load_value(r);
+            }
+        }
+    }
+
     {
         const int tl = threadIdx.x / pairs, i = threadIdx.x - tl * pairs;
         const int64_t tok = tok0 + tl;
         if (tl < tokens_per_wg && tok < n_tokens) {
             const int64_t in_tok = first + tok;
-            const int b = sequence_of(a.seqstarts, (int)a.batch, in_tok);
-            const int64_t pos = a.start_pos[b] + (in_tok - a.seqstarts[b]);
+            // one new token per sequence (a decode step): token i belongs to sequence i, which two independent loads
+            // confirm; otherwise bisection, a chain of dependent loads
+            int b;
+            int64_t pos;
+            const int64_t ti = tok < a.batch ? tok : 0;
+            const int64_t s0 = a.seqstarts[ti], s1 = a.seqstarts[ti + 1], sp = a.start_pos[ti];
+            if (tok < a.batch && s0 == in_tok && s1 > in_tok) {
+                b = (int)tok;
+                pos = sp;
+            } else {
+                b = sequence_of(a.seqstarts, (int)a.batch, in_tok);
+                pos = a.start_pos[b] + (in_tok - a.seqstarts[b]);
+            }
             float c = 1.f, s = 0.f;
             if (i < rd2) {
                 float th = a.theta;
@@ -250,39 +325,39 @@ __global__ __launch_bounds__(kQuantThreads) void rope_append_kernel(const RopeLa
         return out;
     };
 
-    const int gph = a.head_dim >> 3; // groups of 8 channels per head
-    const int q_units = (int)a.num_heads * gph;
-    const int k_units = (int)a.num_key_heads * gph;
-    const int units = q_units + k_units;
-    int n_here = tokens_per_wg;
-    if (tok0 + n_here > n_tokens) n_here = (int)(n_tokens - tok0);
-    for (int w = threadIdx.x; w < n_here * units; w += kQuantThreads) {
-        const int tl = w / units, u = w - tl * units;
-        const int64_t in_tok = first + tok0 + tl;
-        if (u < q_units) {
-            const int h = u / gph, d0 = (u - h * gph) << 3;
-            const int64_t idx = (int64_t)h * a.head_dim + d0;
-            const u32x4 raw = *(const u32x4*)((const half_t*)a.query + in_tok * a.query_stride_s + idx);
-            *(u32x4*)((half_t*)a.rotated_query + in_tok * a.rotated_query_stride_s + idx) = rotate(raw, d0, tl);
-        } else {
-            const int uk = u - q_units;
-            const int h = uk / gph, d0 = (uk - h * gph) << 3;
-            const int64_t idx = (int64_t)h * a.head_dim + d0;
-            u32x4 kraw = *(const u32x4*)((const half_t*)a.key + in_tok * a.key_stride_s + idx);
-            if (!a.bypass_key) kraw = rotate(kraw, d0, tl);
-            if (a.rotated_key) *(u32x4*)((half_t*)a.rotated_key + in_tok * a.rotated_key_stride_s + idx) = kraw;
-            if (append) {
-                const u32x4 vraw = *(const u32x4*)((const half_t*)a.value + in_tok * a.value_stride_s + idx);
-                const Quantised kq = quantise_group(kraw);
-                const Quantised vq = quantise_group(vraw);
-                const int64_t k_out = s_row[tl] * a.cache_stride_s + a.layer_idx * a.cache_stride_l + (int64_t)h * a.cache_stride_h + d0;
-                const int64_t v_out = k_out + a.cache_stride_kv;
-                *(u32x2*)(a.cache + k_out) = kq.q;
-                *(u32x2*)(a.cache + v_out) = vq.q;
-                ((half_t*)a.scale)[k_out >> 3] = kq.scale;
-                ((half_t*)a.scale)[v_out >> 3] = vq.scale;
-            }
+    auto finish = [&](const Unit& r, u32x4 raw, const u32x4 vraw) {
+        if (r.is_query) {
+            *(u32x4*)((half_t*)a.rotated_query + r.in_tok * a.rotated_query_stride_s + r.idx) = rotate(raw, r.d0, r.tl);
+            return;
         }
+        if (!a.bypass_key) raw = rotate(raw, r.d0, r.tl);
+        if (a.rotated_key) *(u32x4*)((half_t*)a.rotated_key + r.in_tok * a.rotated_key_stride_s + r.idx) = raw;
+        if (append) {
+            const Quantised kq = quantise_group(raw);
+            const Quantised vq = quantise_group(vraw);
+            const int64_t k_out = s_row[r.tl] * a.cache_stride_s + a.layer_idx * a.cache_stride_l + (int64_t)r.h * a.cache_stride_h + r.d0;
+            const int64_t v_out = k_out + a.cache_stride_kv;
+            *(u32x2*)(a.cache + k_out) = kq.q;
+            *(u32x2*)(a.cache + v_out) = vq.q;
+            ((half_t*)a.scale)[k_out >> 3] = kq.scale;
+            ((half_t*)a.scale)[v_out >> 3] = vq.scale;
+        }
+    };
+
+    if (early) {
+#pragma unroll
+        for (int j = 0; j < kEarly; ++j) {
+            const int w = threadIdx.x + j * kQuantThreads;
+            if (w < work) finish(unit_of(w), early_row[j], early_value[j]);
+        }
+        return;
+    }
+    for (int w = threadIdx.x; w < work; w += kQuantThreads) {
+        const Unit r = unit_of(w);
+        const u32x4 raw = load_row(r);
+        u32x4 vraw = {0, 0, 0, 0};
+        if (append && !r.is_query) vraw = load_value(r);
+        finish(r, raw, vraw);
     }
 }
 
@@ -338,10 +413,15 @@ int launch_kv_quantize(const QuantLaunch& a, int compute_units, hipStream_t stre
     // exact when blocks was rounded above; otherwise no thread takes a second unit and the value only has to carry
     // a thread beyond the last token
     const uint32_t stride_tokens = (uint32_t)((blocks * kQuantThreads + groups_per_token - 1) / groups_per_token);
-    if (a.cache_mode == 1)
-        hipLaunchKernelGGL(kv_quantize_kernel<true>, dim3((unsigned)blocks), dim3(kQuantThreads), 0, stream, a, stride_tokens);
-    else
-        hipLaunchKernelGGL(kv_quantize_kernel<false>, dim3((unsigned)blocks), dim3(kQuantThreads), 0, stream, a, stride_tokens);
+    const bool wave_token = groups_per_token % kWave == 0;
+    const dim3 grid((unsigned)blocks), block(kQuantThreads);
+    if (a.cache_mode == 1) {
+        if (wave_token) hipLaunchKernelGGL((kv_quantize_kernel<true, true>), grid, block, 0, stream, a, stride_tokens);
+        else hipLaunchKernelGGL((kv_quantize_kernel<true, false>), grid, block, 0, stream, a, stride_tokens);
+    } else {
+        if (wave_token) hipLaunchKernelGGL((kv_quantize_kernel<false, true>), grid, block, 0, stream, a, stride_tokens);
+        else hipLaunchKernelGGL((kv_quantize_kernel<false, false>), grid, block, 0, stream, a, stride_tokens);
+    }
     return kLaunchOk;
 }
 
