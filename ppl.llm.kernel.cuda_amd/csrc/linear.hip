@@ -240,6 +240,153 @@ __global__ __launch_bounds__(kSplitThreads) void split_linear_kernel(const Linea
     }
 }
 
+// ---- the same decomposition without LDS staging: a wave owns a k range, not a column range ------------------------
+// In the kernel above the input passes through LDS in stages of 64 k behind a barrier each, one stage ahead: a
+// workgroup's time is then eight L2 latencies in a row, not its bytes.  Here the four waves of a workgroup split the
+// workgroup's k range between them (in turns of 64 k, so that the four waves together read 512-byte runs of a row)
+// and each computes all 64 columns over its k: the weight fragments and the input fragments of a wave are then its
+// own -- both come straight from memory in the MFMA operand layout (16 bytes of a row per lane), nothing is shared,
+// and there is no barrier before the end.  A weight fragment serves MT row blocks and an input fragment four column
+// blocks, as before.  A turn is 32 k (4 weight and MT input fragments); a wave requests a turn three turns ahead
+// of its products, so with MT = 8 it has up to 36 KB on its way (one workgroup per CU, up to 512 registers per
+// lane).  The four partial tiles of a workgroup are added pairwise through LDS in a fixed order.
+template <int MT>
+__global__ __launch_bounds__(256, 1) void wavek_linear_kernel(const LinearLaunch a, const int splits, float* __restrict__ partial)
+{
+    constexpr int kTiles = 4 * MT;
+    __shared__ __attribute__((aligned(16))) f32x4 s_red[2][kTiles][64]; // MT = 8: 64 KB
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r16 = lane & 15;
+    const int kq = lane >> 4;
+    const int64_t n0 = (int64_t)blockIdx.x * 64;
+    const int64_t m0 = (int64_t)blockIdx.z * (16 * MT);
+    const int64_t k_len = a.k / splits; // a multiple of 512: every wave has the same, even number of turns
+    const int64_t k_begin = (int64_t)blockIdx.y * k_len;
+    const int turns = (int)(k_len >> 8);
+
+    const half_t* wp = (const half_t*)a.weight + (n0 + r16) * a.weight_stride + k_begin + 64 * wave + 8 * kq;
+    const int64_t w16 = 16 * a.weight_stride;
+    const half_t* ip[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        int64_t m = m0 + 16 * mt + r16;
+        if (m > a.m - 1) m = a.m - 1; // rows beyond the batch re-read its last row; their results are not stored
+        ip[mt] = (const half_t*)a.input + m * a.input_stride + k_begin + 64 * wave + 8 * kq;
+    }
+
+    // a turn: 64 k (one 128-byte line of each row, both halves requested together) of the wave's 64 columns and
+    // 16 MT rows
+    struct Turn {
+        f16x8 w[2][4];
+        f16x8 in[2][MT];
+    };
+    Turn r0, r1;
+    auto request = [&](int t, Turn& dst) {
+        const int64_t k = (int64_t)t * 256;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) dst.w[h][nt] = __builtin_nontemporal_load((const f16x8*)(wp + nt * w16 + k + 32 * h));
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) dst.in[h][mt] = *(const f16x8*)(ip[mt] + k + 32 * h);
+        __builtin_amdgcn_sched_barrier(0); // the requests stay where they are written: ahead of the products below
+    };
+
+    f32x4 acc[4][MT];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    auto products = [&](const Turn& u) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(u.w[h][nt], u.in[h][mt], acc[nt][mt], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // Straight-line code between the loop's branches, so that the waits the compiler places count exactly the
+    // requests that may still be on their way; the last two turns are peeled because they have nothing to request.
+    request(0, r0);
+    request(1, r1);
+    int t = 0;
+    for (; t + 4 <= turns; t += 2) {
+        products(r0);
+        request(t + 2, r0);
+        products(r1);
+        request(t + 3, r1);
+    }
+    products(r0);
+    products(r1);
+
+    // (wave 0 + wave 2) + (wave 1 + wave 3): a lane reads back the slots it would have written itself
+    if (wave >= 2) {
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) s_red[wave - 2][nt * MT + mt][lane] = acc[nt][mt];
+    }
+    __syncthreads();
+    if (wave < 2) {
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) acc[nt][mt] += s_red[wave][nt * MT + mt][lane];
+    }
+    __syncthreads();
+    if (wave == 1) {
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) s_red[0][nt * MT + mt][lane] = acc[nt][mt];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[nt][mt] += s_red[0][nt * MT + mt][lane];
+
+    // accumulator element e of tile (nt, mt): row m0 + 16 mt + r16, column n0 + 16 nt + 4 kq + e
+    if (splits > 1) {
+        float* part = partial + ((int64_t)blockIdx.y * a.m + m0) * a.n + n0 + 4 * kq;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            if (m0 + 16 * mt + r16 < a.m) {
+#pragma unroll
+                for (int nt = 0; nt < 4; ++nt) *(f32x4*)(part + (int64_t)(16 * mt + r16) * a.n + 16 * nt) = acc[nt][mt];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+            f32x4 bias = {0.f, 0.f, 0.f, 0.f};
+            if (a.bias) {
+                const f16x4 b = *(const f16x4*)((const half_t*)a.bias + n0 + 16 * nt + 4 * kq);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) bias[e] = (float)b[e];
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const int64_t row = m0 + 16 * mt + r16;
+                if (row < a.m) {
+                    f16x4 o;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = (half_t)(acc[nt][mt][e] + bias[e]);
+                    *(f16x4*)((half_t*)a.output + row * a.output_stride + n0 + 16 * nt + 4 * kq) = o;
+                }
+            }
+        }
+    }
+}
+
 // output = half(sum over the k ranges of the partial tiles, in range order, + bias); four columns per thread
 __global__ __launch_bounds__(256) void linear_reduce_kernel(const LinearLaunch a, const int splits, const float* __restrict__ partial)
 {
@@ -260,7 +407,27 @@ __global__ __launch_bounds__(256) void linear_reduce_kernel(const LinearLaunch a
     *(f16x4*)((half_t*)a.output + row * a.output_stride + c4) = o;
 }
 
-// k ranges for the decode-step form: as many as give every CU two workgroups, a power of two up to 16, each a multiple
+// Row blocks of 16 a workgroup of wavek_linear_kernel takes: the smallest of 1, 2, 4, 8 that covers m, else 8
+static int wavek_row_blocks(int64_t m)
+{
+    return m > 64 ? 8 : m > 32 ? 4 : m > 16 ? 2 : 1;
+}
+
+// k ranges for wavek_linear_kernel: the largest power of two up to 16 that still gives every workgroup a CU of its
+// own in one round, each range a multiple of 512 (four turns of 32 k for each of four waves); 0 when the shape is
+// not for that kernel
+static int wavek_splits(int64_t m, int64_t n, int64_t k, int compute_units)
+{
+    if (n % 64 != 0 || k % 512 != 0) return 0;
+    const int64_t rows = 16 * wavek_row_blocks(m);
+    const int64_t wgs = (n / 64) * ((m + rows - 1) / rows);
+    const int64_t cus = compute_units > 0 ? compute_units : 256;
+    int s = 1;
+    while (s < 16 && wgs * s * 2 <= cus && k % (s * 2 * 512) == 0) s *= 2;
+    return s;
+}
+
+// k ranges for split_linear_kernel: as many as give every CU two workgroups, a power of two up to 16, each a multiple
 // of 64 and at least 256 long; 0 when the shape is for the general kernel (N not in 64s, K not in 64s)
 int linear_splits(int64_t m, int64_t n, int64_t k, int compute_units)
 {
@@ -274,7 +441,8 @@ int linear_splits(int64_t m, int64_t n, int64_t k, int compute_units)
 
 int64_t linear_workspace_bytes(int64_t m, int64_t n, int64_t k, int compute_units)
 {
-    const int s = linear_splits(m, n, k, compute_units);
+    int s = wavek_splits(m, n, k, compute_units);
+    if (s == 0) s = linear_splits(m, n, k, compute_units);
     return s > 1 ? (int64_t)s * m * n * (int64_t)sizeof(float) : 0;
 }
 
@@ -284,19 +452,38 @@ int launch_linear(const LinearLaunch& a, int compute_units, void* workspace, int
     if (a.n % kLinCols != 0 || a.k % kLinKStep != 0 || a.k <= 0) return kLaunchNoKernel;
     const int64_t mblocks = (a.m + kLinRows - 1) / kLinRows;
     if (a.n / kLinCols > 0x7fffffff || mblocks > 65535) return kLaunchNoKernel;
-    int splits = linear_splits(a.m, a.n, a.k, compute_units);
     // as many k ranges as the workspace holds partial tiles for; none: one k range per column block (fewer workgroups
     // than CUs at decode sizes)
     if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 15u)) workspace_bytes = 0;
-    while (splits > 1 && workspace_bytes < (int64_t)splits * a.m * a.n * (int64_t)sizeof(float)) splits /= 2;
+    auto fit = [&](int splits) {
+        while (splits > 1 && workspace_bytes < (int64_t)splits * a.m * a.n * (int64_t)sizeof(float)) splits /= 2;
+        return splits;
+    };
+    auto reduce = [&](int splits) {
+        if (splits <= 1) return;
+        const int64_t threads = a.m * (a.n >> 2);
+        hipLaunchKernelGGL(linear_reduce_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, a, splits,
+                           (const float*)workspace);
+    };
+    int splits = fit(wavek_splits(a.m, a.n, a.k, compute_units));
+    if (splits >= 1) {
+        const int mt = wavek_row_blocks(a.m);
+        const dim3 grid((unsigned)(a.n / 64), (unsigned)splits, (unsigned)((a.m + 16 * mt - 1) / (16 * mt)));
+        float* part = (float*)workspace;
+        switch (mt) {
+        case 8: hipLaunchKernelGGL(wavek_linear_kernel<8>, grid, dim3(256), 0, stream, a, splits, part); break;
+        case 4: hipLaunchKernelGGL(wavek_linear_kernel<4>, grid, dim3(256), 0, stream, a, splits, part); break;
+        case 2: hipLaunchKernelGGL(wavek_linear_kernel<2>, grid, dim3(256), 0, stream, a, splits, part); break;
+        default: hipLaunchKernelGGL(wavek_linear_kernel<1>, grid, dim3(256), 0, stream, a, splits, part); break;
+        }
+        reduce(splits);
+        return kLaunchOk;
+    }
+    splits = fit(linear_splits(a.m, a.n, a.k, compute_units));
     if (splits >= 1) {
         hipLaunchKernelGGL(split_linear_kernel, dim3((unsigned)(a.n / kSplitCols), (unsigned)splits, (unsigned)mblocks),
                            dim3(kSplitThreads), 0, stream, a, splits, (float*)workspace);
-        if (splits > 1) {
-            const int64_t threads = a.m * (a.n >> 2);
-            hipLaunchKernelGGL(linear_reduce_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, a, splits,
-                               (const float*)workspace);
-        }
+        reduce(splits);
         return kLaunchOk;
     }
     hipLaunchKernelGGL(skinny_linear_kernel, dim3((unsigned)(a.n / kLinCols), (unsigned)mblocks), dim3(kLinThreads), 0, stream, a);

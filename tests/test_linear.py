@@ -73,7 +73,8 @@ def test_c_entry_point_rejects_bad_arguments_without_launching(pkg, hip_lib):
 @pytest.mark.gpu
 @pytest.mark.parametrize("shape", [(1, 16, 32), (7, 48, 96), (128, 4096, 4096), (64, 1024, 8192), (200, 256, 512),
                                    (128, 14336 // 8, 4096), (3, 4096, 32), (129, 32, 4064), (17, 64, 64), (128, 128, 3136),
-                                   (300, 8192, 1024), (5, 64, 2240)])
+                                   (300, 8192, 1024), (5, 64, 2240), (1, 64, 512), (16, 128, 1024), (17, 64, 1536), (33, 192, 2048),
+                                   (65, 64, 512), (130, 192, 2048), (240, 4096, 4096)])
 def test_hip_linear_matches_oracle(pkg, oracle, shape):
     import torch
     m, n, k = shape
