@@ -21,8 +21,9 @@
 //     one column, so the softmax max/sum are register-local apart from one
 //     exchange between the two half-waves, and the S^T accumulator layout is
 //     already the B-operand layout of O^T = V^T P^T -- no shuffle between the
-//     two MFMA stages.  V is stored transposed in LDS with tokens permuted to
-//     match that layout.
+//     two MFMA stages.  V lies row-major ([token][channel], like K) in LDS and its
+//     A fragments (rows = channels) are read with transposing 8-byte LDS loads
+//     in the token order that layout asks for.
 //   * v_mfma_f32_32x32x16_f16, fp32 accumulate, base-2 online softmax.
 #include "device_common.h"
 #include "launch_params.h"

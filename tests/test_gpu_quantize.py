@@ -81,6 +81,30 @@ def test_append_exhaustive_numerators(pkg, oracle):
     assert np.array_equal(_bits(got_s[0, 0, tok, 0].reshape(-1)), _bits(sn))
 
 
+def test_append_every_absmax(pkg, oracle):
+    """Every positive finite half once as a group's absmax (the scale's only input), the other seven channels at
+    ratios that hit ties and near-ties: scales and bytes bit-exact against the C oracle and the numpy restatement."""
+    pos = np.arange(1, 0x7C00, dtype=np.uint16).view(np.float16)
+    fr = np.array([1.0, -1.0, 0.5, -0.25, 0.00390625, 0.9921875, -0.503937, 0.0118], dtype=np.float32)
+    groups = (pos.astype(np.float32)[:, None] * fr[None, :]).astype(np.float16)
+    pad = (-groups.shape[0]) % 16
+    groups = np.concatenate([groups, np.zeros((pad, 8), np.float16)])
+    tokens = groups.shape[0] // 16
+    k = groups.reshape(tokens, 1, 128)
+    v = (-groups[::-1]).copy().reshape(tokens, 1, 128)
+    bt, _ = pkg.workloads.custom_batch(1, num_heads=1, num_kv_heads=1, head_dim=128, cache_mode=1,
+                                       dec_kv_lens=[], prefill_q_lens=[tokens], prefill_prior=[0])
+    got_c, got_s = run_append(pkg, bt, k, v)
+    ref_c, ref_s = host_cache(bt, canary=(0x5A, 1.5))
+    oracle_append_step(oracle, bt, k, v, ref_c, ref_s)
+    assert np.array_equal(got_c, ref_c)
+    assert np.array_equal(_bits(got_s), _bits(ref_s))
+    qn, sn = oracle.quantize_groups_numpy(groups)
+    tok = bt.cachestarts[0, np.arange(tokens) // 128] + np.arange(tokens) % 128
+    assert np.array_equal(got_c[0, 0, tok, 0].reshape(-1, 8), qn)
+    assert np.array_equal(_bits(got_s[0, 0, tok, 0].reshape(-1)), _bits(sn))
+
+
 def test_append_empty_and_single(pkg, oracle):
     # sequences with zero new tokens in between, and a batch that appends nothing at all
     bt, rng = pkg.workloads.custom_batch(5, num_heads=4, num_kv_heads=4, head_dim=64, cache_mode=0,

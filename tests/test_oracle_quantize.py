@@ -88,6 +88,43 @@ def test_reciprocal_quotient_identity_over_every_pair(oracle):
     assert half_differs == 0x7C00 - 0x00A8
 
 
+def test_scale_without_division_equals_the_division_for_every_absmax(oracle):
+    """The HIP quantiser forms absmax / 127 as s0 = a * r, s = fma(fma(-s0, 127, a), r, s0) with r = fl(1 / 127)
+    (binary32, every fma rounded once) and rounds s to half.  For every positive finite half a that half equals
+    half(a / 127) with the binary32 division of the reference (kernel.cu:137-139).  The fmas are evaluated in
+    exact rational arithmetic and rounded to binary32 here, so the check does not lean on the host's fma."""
+    from fractions import Fraction
+
+    def to_f32(fr):  # an exact rational rounded once to binary32, ties to even
+        if fr == 0:
+            return np.float32(0.0)
+        sign, mag = (-1, -fr) if fr < 0 else (1, fr)
+        e = mag.numerator.bit_length() - mag.denominator.bit_length() - 24
+        while mag >= Fraction(2) ** (e + 24):
+            e += 1
+        while mag < Fraction(2) ** (e + 23):
+            e -= 1
+        e = max(e, -149)
+        scaled = mag / Fraction(2) ** e
+        n = scaled.numerator // scaled.denominator
+        rem = scaled - n
+        if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and n % 2 == 1):
+            n += 1
+        return np.float32(sign * float(Fraction(n) * Fraction(2) ** e))  # n < 2^24 + 1: exact in binary64
+
+    r = np.float32(1.0) / np.float32(127.0)
+    rf = Fraction(float(r))
+    pos = np.arange(1, 0x7C00, dtype=np.uint16).view(np.float16)
+    want = (pos.astype(np.float32) / np.float32(127.0)).astype(np.float16)
+    got = np.empty_like(want)
+    for i, a in enumerate(pos):
+        af = Fraction(float(a))
+        s0 = Fraction(float(to_f32(af * rf)))
+        e = Fraction(float(to_f32(af - s0 * 127)))
+        got[i] = np.float16(to_f32(e * rf + s0))
+    assert np.array_equal(_bits(got), _bits(want))
+
+
 def test_random_groups_c_equals_numpy_and_error_bound(oracle):
     rng = np.random.default_rng(5)
     x = (rng.standard_normal((20000, 8)) * 10.0 ** rng.integers(-6, 3, (20000, 1))).astype(np.float16)
