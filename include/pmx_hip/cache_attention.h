@@ -22,9 +22,9 @@
  *     holds the range count.
  *   * cfg.workspace_size follows this implementation (float32 partial outputs
  *     and (max, sum) pairs; no arrival counters), not utils.cu:334-343.
- *   * The prefill stage serves head_dim 64 and 128 (the reference's flash_attn2 also has 96 and 256).
- *     heuristic_prepare rejects a batch with prefill sequences at any other head_dim with
- *     RC_UNSUPPORTED, before anything is enqueued; decode-only batches take 64, 96, 128 and 256.
+ *   * Decode and prefill serve head_dim 64, 96, 128 and 256 (the reference's set: kernel.cu:1962 and the
+ *     flash_fwd_hdim{64,96,128,256}_int8_g8 kernels).  heuristic_prepare rejects a batch with prefill
+ *     sequences at any other head_dim with RC_UNSUPPORTED, before anything is enqueued.
  */
 #ifndef PMX_HIP_CACHE_ATTENTION_H_
 #define PMX_HIP_CACHE_ATTENTION_H_

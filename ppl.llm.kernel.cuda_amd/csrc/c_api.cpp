@@ -422,8 +422,8 @@ int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t str
     if (prefill_batches < 0 || p->decoding_batches < 0)
         return fail(PMXHIP_INVALID_VALUE, "prefill_attention: decoding_batches out of range");
     if (prefill_batches == 0 || p->max_seqlen == 0) return PMXHIP_SUCCESS; // kernel.cu:2130, 2214-2216
-    if (p->head_dim != 64 && p->head_dim != 128)
-        return fail(PMXHIP_UNSUPPORTED, "prefill_attention: head dim %lld not supported (64, 128)", (long long)p->head_dim);
+    if (p->head_dim != 64 && p->head_dim != 96 && p->head_dim != 128 && p->head_dim != 256)
+        return fail(PMXHIP_UNSUPPORTED, "prefill_attention: head dim %lld not supported (64, 96, 128, 256)", (long long)p->head_dim);
     if (p->num_kv_heads <= 0 || p->num_heads % p->num_kv_heads != 0)
         return fail(PMXHIP_UNSUPPORTED, "only support num_heads %% num_kv_heads == 0.");
     const bool from_current = p->current_key != nullptr;

@@ -99,10 +99,10 @@ ppl::common::RetCode dynamic_batching_multi_head_cache_attention::heuristic_prep
 
     // ---- derived values (utils.cu:107-131) ----
     const int64_t prefill_batches = batch - decoding_batches;
-    // The prefill stage of this build has head_dim 64 and 128.  Rejected here, not in forward_prefill, so that no
-    // stage of a step that cannot complete is enqueued (the append and the decode rows would already be written).
-    if (prefill_batches > 0 && max_seqlen > 0 && head_dim != 64 && head_dim != 128) {
-        PMX_LOG_ERROR("prefill attention supports head dim 64 and 128, currently get %lld", (long long)head_dim);
+    // The prefill stage serves the head dims of the reference's flash attention (64, 96, 128, 256).  Others are
+    // rejected here, not in forward_prefill, so that no stage is enqueued for a call that cannot complete.
+    if (prefill_batches > 0 && max_seqlen > 0 && head_dim != 64 && head_dim != 96 && head_dim != 128 && head_dim != 256) {
+        PMX_LOG_ERROR("prefill attention supports head dim 64, 96, 128 and 256, currently get %lld", (long long)head_dim);
         return ppl::common::RC_UNSUPPORTED;
     }
     const float attn_scale = float(1.0 / std::sqrt(float(head_dim)));

@@ -647,6 +647,336 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     } // items
 }
 
+// ---- the 16-column form: head dims whose accumulators and query fragments the kernel above cannot hold ----
+// head_dim 256 needs 128 accumulator and 64 query registers per lane with 32 columns per wave; head_dim 96 does not
+// divide into that kernel's 512 staging units.  Here a wave has 16 columns and the products run on
+// v_mfma_f32_16x16x32_f16: S^T tiles of 16 tokens x 16 columns (4 registers), O^T tiles of 16 channels x 16 columns.
+// Same decomposition otherwise (one workgroup = one kv head x a tile of query positions x all query heads of the
+// group: 128 columns; K/V tiles dequantised once per workgroup into one of two LDS buffers, one barrier per tile;
+// hi + lo pairs for K^, V^ and p), in a plain order: stage the next tile, then S^T, softmax, O^T of this one.
+// A lane (column c = lane % 16, quarter kq = lane / 16) holds of each S^T tile the tokens 4 kq .. 4 kq + 3; a tile of
+// 32 tokens is two S^T tiles, and its 8 values per lane are the lane's share of the k dimension of the O^T step
+// (slot e of quarter kq = token 16 (e / 4) + 4 kq + e % 4), which is the order the transposing V reads deliver.
+namespace {
+constexpr int kBN16 = 32;    // kv tokens per tile
+constexpr int kCols16 = 128; // (position, head) columns per workgroup, 16 per wave
+template <int D>
+struct PrefillTile16 {
+    static constexpr int K_STRIDE = D + 8;
+    static constexpr int V_STRIDE = ((D + 32) * 2) % 128 == 64 ? D + 32 : D + 64; // an odd multiple of 64 bytes
+};
+static_assert((PrefillTile16<96>::V_STRIDE * 2) % 128 == 64 && (PrefillTile16<256>::V_STRIDE * 2) % 128 == 64, "V row stride");
+} // namespace
+
+template <int D, int SRC, bool EXTRA>
+__global__ __launch_bounds__(kPrefillThreads, D <= 128 ? 4 : 2) void prefill_attention16_kernel(const PrefillLaunch a)
+{
+    constexpr bool PAGED = SRC == 0;
+    constexpr bool KV16 = SRC == 2;
+    constexpr int KSTEPS = D / 32;          // MFMA k-steps over channels for S
+    constexpr int CT = D / 16;              // 16-channel tiles of O^T
+    constexpr int GPT = D / 8;              // quantisation groups per token row
+    constexpr int K_STRIDE = PrefillTile16<D>::K_STRIDE;
+    constexpr int V_STRIDE = PrefillTile16<D>::V_STRIDE;
+    constexpr int TILE_UNITS = kBN16 * GPT; // (token, group) units of a tile, of K and of V each
+    constexpr int UNITS = (TILE_UNITS + kPrefillThreads - 1) / kPrefillThreads;
+    constexpr int K_HALVES = kBN16 * K_STRIDE, V_HALVES = kBN16 * V_STRIDE;
+    constexpr int TILE_HALVES = (KV16 ? 1 : 2) * (K_HALVES + V_HALVES);
+
+    extern __shared__ __attribute__((aligned(16))) char smem_raw[];
+    half_t* const smem = (half_t*)smem_raw;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int r16 = lane & 15;
+    const int kq = lane >> 4;
+    const int k_frag_off = r16 * K_STRIDE + 8 * kq;                            // + 16 mb rows + 32 s
+    const int v_frag_off = (4 * kq + (r16 >> 2)) * V_STRIDE + 4 * (lane & 3);  // + 16 rows for slots 4..7, + 16 ct
+
+    const int G = (int)(a.num_heads / a.num_kv_heads);
+    const int ppw = kCols16 / G > 0 ? kCols16 / G : 1;
+    const int kvh = blockIdx.x % (int)a.num_kv_heads;
+    const int item_stride = gridDim.x / (int)a.num_kv_heads;
+
+    const int8_t* __restrict__ cache = (const int8_t*)a.cache;
+    const half_t* __restrict__ scale = (const half_t*)a.scale;
+    const int64_t head_off = a.layer_idx * a.cache_stride_l + (int64_t)kvh * a.cache_stride_h;
+    const int8_t* const cache_k = cache + head_off;
+    const int8_t* const cache_v = cache_k + a.cache_stride_kv;
+    const half_t* const scale_k = scale + (head_off >> 3);
+    const half_t* const scale_v = scale_k + (a.cache_stride_kv >> 3);
+    const const_i64_ptr cachestarts = as_constant(a.cachestarts);
+    const float sm_scale = a.attn_scale * kLog2e;
+
+    // this thread's units of a tile: unit tid + 512 u = (token, group)
+    const uint32_t stride_s32 = (uint32_t)a.cache_stride_s; // the host checks that a tile's span fits 32 bits
+    const uint32_t kstride16 = (uint32_t)a.key_stride_s, vstride16 = (uint32_t)a.value_stride_s;
+    int u_t[UNITS], u_g[UNITS];
+    bool u_on[UNITS];
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u) {
+        const int idx = tid + u * kPrefillThreads;
+        u_on[u] = idx < TILE_UNITS;
+        u_t[u] = u_on[u] ? idx / GPT : 0;
+        u_g[u] = u_on[u] ? idx % GPT : 0;
+    }
+
+    for (int item = blockIdx.x / (int)a.num_kv_heads;; item += item_stride) {
+    int b_pick = 0, tile_pick = 0;
+    if (!pick_query_tile(a, ppw, item, lane, b_pick, tile_pick)) return;
+    const int b = __builtin_amdgcn_readfirstlane(b_pick);
+    const int64_t q_row0 = a.seqstarts[b];
+    const int qlen = (int)(a.seqstarts[b + 1] - q_row0);
+    const int kvlen = (int)(a.kvstarts[b + 1] - a.kvstarts[b]);
+    const int p0 = __builtin_amdgcn_readfirstlane(tile_pick) * ppw;
+    if (p0 < 0 || p0 >= qlen) continue;
+
+    // ---- this lane's column ----
+    const int col = wave * 16 + r16;
+    const int pos = p0 + col / G;
+    const int g = col % G;
+    const bool col_on = (col < ppw * G) && (pos < qlen);
+    const int pos_c = pos < qlen ? pos : qlen - 1;
+    const int h = kvh * G + (col < ppw * G ? g : 0);
+    int lim = kvlen; // this column attends tokens [0, lim)
+    if (a.is_causal) {
+        lim = pos_c + 1 + kvlen - qlen;
+        lim = lim < 0 ? 0 : (lim > kvlen ? kvlen : lim);
+    }
+    if (!col_on) lim = 0;
+    int last_pos = p0 + ppw - 1;
+    if (last_pos > qlen - 1) last_pos = qlen - 1;
+    int wg_lim = kvlen;
+    if (a.is_causal) {
+        wg_lim = last_pos + 1 + kvlen - qlen;
+        wg_lim = wg_lim < 0 ? 0 : (wg_lim > kvlen ? kvlen : wg_lim);
+    }
+    const int n_tiles = (wg_lim + kBN16 - 1) / kBN16;
+    int wave_lim = lim;
+#pragma unroll
+    for (int sh = 32; sh >= 1; sh >>= 1) {
+        const int o = __shfl_xor(wave_lim, sh);
+        wave_lim = o > wave_lim ? o : wave_lim;
+    }
+    wave_lim = __builtin_amdgcn_readfirstlane(wave_lim);
+
+    // ---- Q fragments: B operand of S^T = K Q^T; lane holds Q[col][32 s + 8 kq .. +8] ----
+    f16x8 qf[KSTEPS];
+    {
+        const half_t* qp = (const half_t*)a.query + (q_row0 + pos_c) * a.query_stride_s + (int64_t)h * D + 8 * kq;
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) qf[s] = *(const f16x8*)(qp + 32 * s);
+    }
+
+    f32x4 o_acc[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) o_acc[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = kNegBig, l_run = 0.f;
+    const half_t* mask_row = nullptr;
+    float slope = 0.f;
+    if (EXTRA) {
+        if (a.attn_mask)
+            mask_row = (const half_t*)a.attn_mask + (int64_t)h * a.mask_stride_h + (q_row0 + pos_c) * a.mask_stride_s + a.kvstarts[b];
+        if (a.alibi_slopes) slope = a.alibi_slopes[h];
+    }
+
+    // ---- global -> register staging of one tile's raw bytes ----
+    const int64_t table_base = PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b;
+    u32x2 k_raw[UNITS], v_raw[UNITS];
+    half_t k_sc[UNITS], v_sc[UNITS];
+    u32x4 k16[UNITS], v16[UNITS];
+    // a tile of 32 tokens starts at a multiple of 32, so it lies inside one 128-token page
+    auto tile_row = [&](int tile) -> int64_t {
+        int t_base = tile * kBN16;
+        if (t_base > kvlen - 1) t_base = kvlen > 0 ? kvlen - 1 : 0;
+        if (KV16) return q_row0 + t_base;
+        if (PAGED) return cachestarts[table_base + (t_base >> 7)] + (t_base & (kPage - 1));
+        return cachestarts[table_base] + t_base;
+    };
+    auto load_tile = [&](int tile) {
+        const int64_t row = tile_row(tile);
+        const int left = kvlen - 1 - tile * kBN16; // offset of the sequence's last token inside this tile
+#pragma unroll
+        for (int u = 0; u < UNITS; ++u) {
+            if (!u_on[u]) continue;
+            // tokens beyond the sequence re-read its last token (masked later)
+            const uint32_t t = (uint32_t)(u_t[u] < left ? u_t[u] : (left > 0 ? left : 0));
+            if (KV16) {
+                const half_t* bk = (const half_t*)a.current_key + row * a.key_stride_s + (int64_t)kvh * D;
+                const half_t* bv = (const half_t*)a.current_value + row * a.value_stride_s + (int64_t)kvh * D;
+                k16[u] = *(const u32x4*)(bk + t * kstride16 + 8 * u_g[u]);
+                v16[u] = *(const u32x4*)(bv + t * vstride16 + 8 * u_g[u]);
+            } else {
+                const int64_t boff = row * a.cache_stride_s;
+                const uint32_t off = t * stride_s32 + 8 * (uint32_t)u_g[u];
+                k_raw[u] = *(const u32x2*)(cache_k + boff + off);
+                k_sc[u] = (scale_k + (boff >> 3))[off >> 3];
+                v_raw[u] = *(const u32x2*)(cache_v + boff + off);
+                v_sc[u] = (scale_v + (boff >> 3))[off >> 3];
+            }
+        }
+    };
+    auto split_store = [&](half_t* dst, half_t* dst_lo, const u32x2 raw, const half_t scl) {
+        const half2_t sc = {scl, scl};
+        const uint32_t f0 = raw[0] ^ kFlipSigns, f1 = raw[1] ^ kFlipSigns;
+        const half2_t x0 = cvt_bytes01(f0), x1 = cvt_bytes23(f0), x2 = cvt_bytes01(f1), x3 = cvt_bytes23(f1);
+        const half2_t h0 = x0 * sc, h1 = x1 * sc, h2 = x2 * sc, h3 = x3 * sc;
+        u32x4 w, wl;
+        w[0] = bitcast<uint32_t>(h0);
+        w[1] = bitcast<uint32_t>(h1);
+        w[2] = bitcast<uint32_t>(h2);
+        w[3] = bitcast<uint32_t>(h3);
+        wl[0] = bitcast<uint32_t>(__builtin_elementwise_fma(x0, sc, -h0));
+        wl[1] = bitcast<uint32_t>(__builtin_elementwise_fma(x1, sc, -h1));
+        wl[2] = bitcast<uint32_t>(__builtin_elementwise_fma(x2, sc, -h2));
+        wl[3] = bitcast<uint32_t>(__builtin_elementwise_fma(x3, sc, -h3));
+        *(u32x4*)dst = w;
+        *(u32x4*)dst_lo = wl;
+    };
+    auto store_tile = [&](int buf) {
+        half_t* const sK = smem + buf * TILE_HALVES;
+        half_t* const sKlo = sK + K_HALVES;
+        half_t* const sV = KV16 ? sKlo : sKlo + K_HALVES;
+        half_t* const sVlo = sV + V_HALVES;
+#pragma unroll
+        for (int u = 0; u < UNITS; ++u) {
+            if (!u_on[u]) continue;
+            half_t* const dk = &sK[u_t[u] * K_STRIDE + 8 * u_g[u]];
+            half_t* const dv = &sV[u_t[u] * V_STRIDE + 8 * u_g[u]];
+            if (KV16) {
+                *(u32x4*)dk = k16[u];
+                *(u32x4*)dv = v16[u];
+            } else {
+                split_store(dk, &sKlo[u_t[u] * K_STRIDE + 8 * u_g[u]], k_raw[u], k_sc[u]);
+                split_store(dv, &sVlo[u_t[u] * V_STRIDE + 8 * u_g[u]], v_raw[u], v_sc[u]);
+            }
+        }
+    };
+
+    __syncthreads(); // the previous item's last tile has been read by every wave
+    if (n_tiles > 0) {
+        load_tile(0);
+        store_tile(0);
+        if (n_tiles > 1) load_tile(1);
+        __syncthreads();
+    }
+
+    for (int tile = 0; tile < n_tiles; ++tile) {
+        const int buf = tile & 1;
+        // the next tile into the other buffer (every wave is past its reads of it since the barrier that ended the
+        // previous iteration), and the raw bytes of the tile after next into the freed registers
+        if (tile + 1 < n_tiles) store_tile(buf ^ 1);
+        if (tile + 2 < n_tiles) load_tile(tile + 2);
+
+        const int t_base = tile * kBN16;
+        if (t_base < wave_lim) { // a wave whose columns end before this tile only helps to stage it
+            const half_t* const sK = smem + buf * TILE_HALVES;
+            const half_t* const sKlo = sK + K_HALVES;
+            const half_t* const sV = KV16 ? sKlo : sKlo + K_HALVES;
+            const half_t* const sVlo = sV + V_HALVES;
+
+            // ---- S^T: two tiles of 16 tokens ----
+            f32x4 sacc[2];
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb) {
+                sacc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < KSTEPS; ++s) {
+                    const f16x8 fh = *(const f16x8*)&sK[k_frag_off + 16 * mb * K_STRIDE + 32 * s];
+                    if (!KV16) {
+                        const f16x8 fl = *(const f16x8*)&sKlo[k_frag_off + 16 * mb * K_STRIDE + 32 * s];
+                        sacc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fl, qf[s], sacc[mb], 0, 0, 0);
+                    }
+                    sacc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fh, qf[s], sacc[mb], 0, 0, 0);
+                }
+            }
+
+            // ---- softmax: element j of tile mb is token t_base + 16 mb + 4 kq + j ----
+            float v[8];
+            float mx = kNegBig;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const int t = t_base + 16 * (e >> 2) + 4 * kq + (e & 3);
+                float x = -INFINITY;
+                if (t < lim) {
+                    if (EXTRA) {
+                        float add = 0.f;
+                        if (mask_row) add = (float)mask_row[t];
+                        if (a.alibi_slopes) add += a.is_causal ? slope * (float)t : -slope * fabsf((float)(pos_c + kvlen - qlen - t));
+                        x = __builtin_fmaf(sacc[e >> 2][e & 3], sm_scale, add * kLog2e);
+                    } else {
+                        x = sacc[e >> 2][e & 3] * sm_scale;
+                    }
+                }
+                v[e] = x;
+                mx = fmaxf(mx, x);
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_run, mx);
+            if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) { // rare after the first tiles (wave-uniform)
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                l_run *= alpha;
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) o_acc[ct] *= alpha;
+                m_run = m_new;
+            }
+            // p = 2^(logit - max) * 2^14 as hi + lo halves (hi rounded toward zero, lo the exact remainder)
+            const float bias = kPShift - m_run;
+            f16x8 ph, pl;
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                const float q0 = __builtin_amdgcn_exp2f(v[e] + bias), q1 = __builtin_amdgcn_exp2f(v[e + 1] + bias);
+                l_run += q0 + q1;
+                const half2_t h2 = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(q0, q1));
+                const half2_t l2 = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(sub_half_lo(q0, h2), sub_half_hi(q1, h2)));
+                ph[e] = h2.x;
+                ph[e + 1] = h2.y;
+                pl[e] = l2.x;
+                pl[e + 1] = l2.y;
+            }
+
+            // ---- O^T += V^T P^T: channel tile ct, the lane's 8 tokens from two transposing reads ----
+            typedef short s16x4 __attribute__((ext_vector_type(4)));
+            typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
+            auto read_vt = [&](const half_t* base, int ct) -> f16x8 {
+                const half_t* p = base + v_frag_off + 16 * ct;
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 16 * V_STRIDE));
+                return bitcast<f16x8>(__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+            };
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                const f16x8 vh = read_vt(sV, ct);
+                if (!KV16) {
+                    const f16x8 vl = read_vt(sVlo, ct);
+                    o_acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vl, ph, o_acc[ct], 0, 0, 0);
+                }
+                o_acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vh, pl, o_acc[ct], 0, 0, 0);
+                o_acc[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vh, ph, o_acc[ct], 0, 0, 0);
+            }
+        }
+        __syncthreads(); // tile + 1 is complete in the other buffer; this buffer may be overwritten
+    }
+
+    // ---- normalise and store: element j of tile ct <-> channel 16 ct + 4 kq + j ----
+    float l_tot = l_run + __shfl_xor(l_run, 16);
+    l_tot += __shfl_xor(l_tot, 32);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (col_on) {
+        half_t* op = (half_t*)a.output + (q_row0 + pos) * a.output_stride_s + (int64_t)h * D + 4 * kq;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            f16x4 w;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = (half_t)(o_acc[ct][e] * inv);
+            *(f16x4*)(op + 16 * ct) = w;
+        }
+    }
+    } // items
+}
+
 template <int D, int SRC>
 constexpr size_t prefill_lds_bytes()
 {
@@ -698,12 +1028,62 @@ static int launch_prefill_d(const PrefillLaunch& a, hipStream_t stream)
     return launch_prefill_variant<D, 2, false>(a, grid, stream);
 }
 
+template <int D, int SRC>
+constexpr size_t prefill16_lds_bytes()
+{
+    return 2 * (SRC == 2 ? 1 : 2) * kBN16 * (PrefillTile16<D>::K_STRIDE + PrefillTile16<D>::V_STRIDE) * sizeof(half_t);
+}
+
+template <int D, int SRC, bool EXTRA>
+static std::atomic<int>& prefill16_variant_ready()
+{
+    static std::atomic<int> ready{0};
+    return ready;
+}
+
+template <int D, int SRC, bool EXTRA>
+static int launch_prefill16_variant(const PrefillLaunch& a, dim3 grid, hipStream_t stream)
+{
+    constexpr size_t lds_bytes = prefill16_lds_bytes<D, SRC>();
+    if (int rc = ensure_dynamic_lds((const void*)prefill_attention16_kernel<D, SRC, EXTRA>, (int)lds_bytes, stream,
+                                    prefill16_variant_ready<D, SRC, EXTRA>()))
+        return rc;
+    hipLaunchKernelGGL((prefill_attention16_kernel<D, SRC, EXTRA>), grid, dim3(kPrefillThreads), lds_bytes, stream, a);
+    return kLaunchOk;
+}
+
+template <int D>
+static int launch_prefill16_d(const PrefillLaunch& a, hipStream_t stream)
+{
+    const int G = (int)(a.num_heads / a.num_kv_heads);
+    if (G > kCols16) return kLaunchNoKernel;
+    const int ppw = kCols16 / G > 0 ? kCols16 / G : 1;
+    int64_t items = a.prefill_batches * ((a.max_seqlen + ppw - 1) / ppw);
+    if (a.query_rows > 0 && a.prefill_batches <= 64 * kPickSlots) {
+        const int64_t by_rows = a.query_rows / ppw + a.prefill_batches;
+        if (by_rows < items) items = by_rows;
+    }
+    if (items * a.num_kv_heads > 0x7fffffff) return kLaunchNoKernel;
+    const dim3 grid((unsigned)(items * a.num_kv_heads), 1, 1);
+    const bool extra = a.attn_mask != nullptr || a.alibi_slopes != nullptr;
+    const int src = a.current_key ? 2 : (a.cache_mode == 1 ? 0 : 1);
+    if (extra) {
+        if (src == 0) return launch_prefill16_variant<D, 0, true>(a, grid, stream);
+        if (src == 1) return launch_prefill16_variant<D, 1, true>(a, grid, stream);
+        return launch_prefill16_variant<D, 2, true>(a, grid, stream);
+    }
+    if (src == 0) return launch_prefill16_variant<D, 0, false>(a, grid, stream);
+    if (src == 1) return launch_prefill16_variant<D, 1, false>(a, grid, stream);
+    return launch_prefill16_variant<D, 2, false>(a, grid, stream);
+}
+
 int launch_prefill(const PrefillLaunch& a, hipStream_t stream)
 {
-    if (a.num_heads / a.num_kv_heads > kCols) return kLaunchNoKernel;
     switch (a.head_dim) {
-        case 64: return launch_prefill_d<64>(a, stream);
-        case 128: return launch_prefill_d<128>(a, stream);
+        case 64: return a.num_heads / a.num_kv_heads > kCols ? kLaunchNoKernel : launch_prefill_d<64>(a, stream);
+        case 128: return a.num_heads / a.num_kv_heads > kCols ? kLaunchNoKernel : launch_prefill_d<128>(a, stream);
+        case 96: return launch_prefill16_d<96>(a, stream);
+        case 256: return launch_prefill16_d<256>(a, stream);
         default: return kLaunchNoKernel;
     }
 }
@@ -729,10 +1109,33 @@ static int init_prefill_d()
     if (int rc = init_prefill_variant<D, 2, false>()) return rc;
     return init_prefill_variant<D, 2, true>();
 }
+template <int D, int SRC, bool EXTRA>
+static int init_prefill16_variant()
+{
+    std::atomic<int>& ready = prefill16_variant_ready<D, SRC, EXTRA>();
+    if (ready.load() != 0) return kLaunchOk;
+    if (hipFuncSetAttribute((const void*)prefill_attention16_kernel<D, SRC, EXTRA>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)prefill16_lds_bytes<D, SRC>()) != hipSuccess)
+        return kLaunchNoKernel;
+    ready.store(1);
+    return kLaunchOk;
+}
+template <int D>
+static int init_prefill16_d()
+{
+    if (int rc = init_prefill16_variant<D, 0, false>()) return rc;
+    if (int rc = init_prefill16_variant<D, 0, true>()) return rc;
+    if (int rc = init_prefill16_variant<D, 1, false>()) return rc;
+    if (int rc = init_prefill16_variant<D, 1, true>()) return rc;
+    if (int rc = init_prefill16_variant<D, 2, false>()) return rc;
+    return init_prefill16_variant<D, 2, true>();
+}
 int init_prefill_kernels()
 {
     if (int rc = init_prefill_d<64>()) return rc;
-    return init_prefill_d<128>();
+    if (int rc = init_prefill_d<128>()) return rc;
+    if (int rc = init_prefill16_d<96>()) return rc;
+    return init_prefill16_d<256>();
 }
 
 } // namespace pmxhip

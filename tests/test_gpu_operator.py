@@ -50,6 +50,17 @@ def test_mixed_batch_through_the_operator(pkg, oracle, multi_block):
         assert op.cfg.decoding_multi_block_size == 1 and op.cfg.workspace_size == 0
 
 
+@pytest.mark.parametrize("heads", [(16, 8, 256), (8, 8, 256), (12, 4, 96), (32, 4, 256)])
+def test_mixed_batch_at_the_other_head_dims(pkg, oracle, heads):
+    """head_dim 96 and 256 (the reference's flash attention and decode kernels serve 64, 96, 128, 256): append,
+    decode and the 16-column prefill kernel in one forward()."""
+    hq, hkv, d = heads
+    bt, rng = pkg.workloads.custom_batch(420 + hq + d, num_heads=hq, num_kv_heads=hkv, head_dim=d, cache_mode=1,
+                                         dec_kv_lens=[300, 33, 700, 1], prefill_q_lens=[100, 17, 130],
+                                         prefill_prior=[150, 0, 31], outliers=True, num_layer=2, layer_idx=1)
+    full_step(pkg, oracle, bt, rng)
+
+
 def test_scaled_c5_through_the_operator(pkg, oracle):
     bt, rng = pkg.workloads.make_batch("C5", scale=0.06)
     full_step(pkg, oracle, bt, rng)

@@ -37,7 +37,8 @@ def run_prefill(pkg, dev, is_causal=None, **extra):
 
 
 @pytest.mark.parametrize("cache_mode", [0, 1])
-@pytest.mark.parametrize("shape", [(8, 2, 128), (4, 4, 128), (12, 2, 128), (8, 8, 64), (16, 2, 64), (2, 1, 128), (16, 1, 128)])
+@pytest.mark.parametrize("shape", [(8, 2, 128), (4, 4, 128), (12, 2, 128), (8, 8, 64), (16, 2, 64), (2, 1, 128), (16, 1, 128),
+                                   (8, 2, 256), (4, 4, 256), (16, 1, 256), (8, 2, 96), (6, 6, 96), (12, 2, 96)])
 def test_prefill_matches_oracle(pkg, oracle, shape, cache_mode):
     hq, hkv, d = shape
     bt, dev, q, cache, scale = make_case(pkg, oracle, 300 + hq + d, num_heads=hq, num_kv_heads=hkv, head_dim=d,
@@ -51,7 +52,7 @@ def test_prefill_matches_oracle(pkg, oracle, shape, cache_mode):
     assert_attention_close(got[n_dec:], ref[n_dec:], "prefill %s mode %d" % (shape, cache_mode))
 
 
-@pytest.mark.parametrize("shape", [(32, 8, 128), (8, 1, 128), (8, 8, 64), (64, 8, 128)])
+@pytest.mark.parametrize("shape", [(32, 8, 128), (8, 1, 128), (8, 8, 64), (64, 8, 128), (16, 8, 256), (8, 4, 96)])
 def test_prefill_short_chunks_over_long_histories(pkg, oracle, shape):
     """A few query tokens per sequence over many kv tiles: most waves of a workgroup have no live column."""
     hq, hkv, d = shape
@@ -150,7 +151,8 @@ def test_prefill_full_size_c5(pkg, oracle):
 
 
 @pytest.mark.parametrize("is_causal", [True, False])
-@pytest.mark.parametrize("shape,cache_mode,per_head", [((8, 2, 128), 1, True), ((4, 4, 64), 0, False), ((8, 8, 128), 1, False)])
+@pytest.mark.parametrize("shape,cache_mode,per_head", [((8, 2, 128), 1, True), ((4, 4, 64), 0, False), ((8, 8, 128), 1, False),
+                                                       ((8, 2, 256), 1, True), ((6, 2, 96), 0, False)])
 def test_prefill_mask_and_alibi_match_oracle(pkg, oracle, shape, cache_mode, per_head, is_causal):
     """The optional inputs of the prefill stage: additive attn_mask (2-d and per-head 3-d) and alibi slopes."""
     hq, hkv, d = shape
@@ -174,7 +176,7 @@ def test_prefill_mask_and_alibi_match_oracle(pkg, oracle, shape, cache_mode, per
         assert_attention_close(got[n_dec:], ref[n_dec:], "prefill mask=%s alibi=%s %s" % (use_mask, use_alibi, shape))
 
 
-@pytest.mark.parametrize("shape", [(8, 2, 128), (4, 4, 64), (32, 8, 128)])
+@pytest.mark.parametrize("shape", [(8, 2, 128), (4, 4, 64), (32, 8, 128), (8, 2, 256), (6, 3, 96)])
 def test_prefill_from_current_key_value(pkg, oracle, shape):
     """enable_cache_prefill = false: attention over the step's own fp16 K/V rows, no cache read."""
     hq, hkv, d = shape

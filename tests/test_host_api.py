@@ -75,10 +75,10 @@ def test_prepare_derives_the_reference_values(pkg, hip_lib):
     (dict(specify_decoding_tpb=128), 4),
     (dict(enable_sharemem_mhca=False, enable_infinity_mhca=False, enable_infinity_gqca=False), 1),  # no algorithm
     # prefill sequences at a head_dim the prefill stage does not have: refused before anything is enqueued
-    (dict(batch=9, decoding_batches=6, max_seqlen=40, head_dim=256, query_shape=(90, 32, 256),
-          current_key_shape=(90, 8, 256), current_value_shape=(90, 8, 256), output_shape=(90, 32, 256)), 2),
-    (dict(batch=9, decoding_batches=6, max_seqlen=40, head_dim=96, query_shape=(90, 32, 96),
-          current_key_shape=(90, 8, 96), current_value_shape=(90, 8, 96), output_shape=(90, 32, 96)), 2),
+    (dict(batch=9, decoding_batches=6, max_seqlen=40, head_dim=80, query_shape=(90, 32, 80),
+          current_key_shape=(90, 8, 80), current_value_shape=(90, 8, 80), output_shape=(90, 32, 80)), 2),
+    (dict(batch=9, decoding_batches=6, max_seqlen=40, head_dim=32, query_shape=(90, 32, 32),
+          current_key_shape=(90, 8, 32), current_value_shape=(90, 8, 32), output_shape=(90, 32, 32)), 2),
 ])
 def test_prepare_error_branches(pkg, hip_lib, over, code):
     _, rc = prepare(pkg, **over)
@@ -93,7 +93,12 @@ def test_prepare_accepts_what_the_reference_accepts(pkg, hip_lib):
                  dict(head_dim=256, query_shape=(6, 32, 256), current_key_shape=(6, 8, 256),
                       current_value_shape=(6, 8, 256), output_shape=(6, 32, 256)),
                  dict(head_dim=96, query_shape=(6, 32, 96), current_key_shape=(6, 8, 96),
-                      current_value_shape=(6, 8, 96), output_shape=(6, 32, 96))):
+                      current_value_shape=(6, 8, 96), output_shape=(6, 32, 96)),
+                 # and batches with prefill sequences the four head dims of the reference's flash attention
+                 dict(batch=9, decoding_batches=6, max_seqlen=40, head_dim=256, query_shape=(90, 32, 256),
+                      current_key_shape=(90, 8, 256), current_value_shape=(90, 8, 256), output_shape=(90, 32, 256)),
+                 dict(batch=9, decoding_batches=6, max_seqlen=40, head_dim=96, query_shape=(90, 32, 96),
+                      current_key_shape=(90, 8, 96), current_value_shape=(90, 8, 96), output_shape=(90, 32, 96))):
         op, rc = prepare(pkg, **over)
         assert rc == 0, over
     op, _ = prepare(pkg, specify_decoding_multi_block=0)
