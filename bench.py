@@ -87,6 +87,50 @@ def cpu_baseline(oracle, bt, q, cache_host, scale_host, budget_s=2.0):
             "us_per_layer_extrapolated": dt * 1e6 * bt.decode_kv_tokens / max(tokens, 1)}
 
 
+def extras(torch, ops, dev, bt, replay_times):
+    """Microseconds per call, in the replayed-graph regime of the rest of the line, of the kernels either side of
+    the layer call: RoPE on the step's query and key rows, RoPE fused with the quantise/append, the append alone,
+    and kv_cache_reorder / kv_cache_invert_reorder of 64 pages of a (4 layers, 8 kv heads, 128 channels) cache."""
+    lk = dev.layout_kwargs()
+    kw = dict(theta=10000.0, rotary_dim=bt.head_dim, batch=bt.batch, max_seqlen=bt.max_seqlen)
+    rq, rk = torch.empty_like(dev.query), torch.empty_like(dev.new_key)
+    n_new = int(bt.q_lens.sum())
+    res = {"new_tokens": n_new}
+    res["rope_us"] = float(np.median(replay_times(lambda st: ops.rotary_position_embedding(
+        dev.query, dev.new_key, dev.start_pos, dev.seqstarts, rq, rk, stream=st, **kw))))
+    res["append_us"] = float(np.median(replay_times(lambda st: ops.key_value_cache(
+        dev.new_key, dev.new_value, dev.seqstarts, dev.cachestarts, dev.start_pos, dev.cache, dev.scale, batch=bt.batch,
+        max_seqlen=bt.max_seqlen, num_layer=bt.num_layer, layer_idx=bt.layer_idx, num_kv_heads=bt.num_kv_heads,
+        head_dim=bt.head_dim, stream=st, **lk))))
+    res["rope_append_fused_us"] = float(np.median(replay_times(lambda st: ops.rope_key_value_cache(
+        dev.query, dev.new_key, dev.new_value, dev.start_pos, dev.seqstarts, dev.cachestarts, rq, None, dev.cache,
+        dev.scale, num_layer=bt.num_layer, layer_idx=bt.layer_idx, stream=st, **lk, **kw))))
+    # the fused call rewrote this step's cache rows from rotated keys: put the plain ones back
+    ops.key_value_cache(dev.new_key, dev.new_value, dev.seqstarts, dev.cachestarts, dev.start_pos, dev.cache, dev.scale,
+                        batch=bt.batch, max_seqlen=bt.max_seqlen, num_layer=bt.num_layer, layer_idx=bt.layer_idx,
+                        num_kv_heads=bt.num_kv_heads, head_dim=bt.head_dim, **lk)
+    layers, heads, d, group, pool_pages = 4, 8, 128, 8, 256
+    t_page, sb = 128, d // group * 2
+    tok = pool_pages * t_page
+    src = [0, 2 * heads * tok * d, heads * tok * d, tok * d, d, 1, 0, 2 * heads * tok * sb, heads * tok * sb, tok * sb, sb, 1]
+    pcb, psb = t_page * heads * 2 * layers * d, t_page * heads * 2 * layers * sb
+    dst = [0, d, layers * d, 2 * layers * d, heads * 2 * layers * d, 1, 0, sb, layers * sb, 2 * layers * sb, heads * 2 * layers * sb, 1]
+    src[0], src[6] = pcb, psb
+    cache = torch.randint(0, 255, (layers, 2, heads, tok, d), dtype=torch.uint8, device="cuda")
+    scale = torch.randint(0, 255, (layers, 2, heads, tok, sb), dtype=torch.uint8, device="cuda")
+    ids = torch.randperm(pool_pages, device="cuda")[:64].to(torch.int64)
+    outer = torch.empty(64 * (pcb + psb), dtype=torch.uint8, device="cuda")
+    pk = dict(layers=layers, kv_heads=heads, tokens=t_page, head_dim=d, group_size=group, tp_rank=0, tp_size=1)
+    moved = 64 * (pcb + psb)
+    res["reorder_bytes_moved"] = moved
+    res["kv_cache_reorder_us"] = float(np.median(replay_times(lambda st: ops.kv_cache_reorder(
+        cache, scale, ids, src, dst, outer_mem=outer, stream=st, **pk))))
+    inv_src = [pcb] + dst[1:6] + [psb] + dst[7:]
+    res["kv_cache_invert_reorder_us"] = float(np.median(replay_times(lambda st: ops.kv_cache_invert_reorder(
+        outer, ids, inv_src, src, kv_cache=cache, kv_scale=scale, stream=st, **pk))))
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -97,6 +141,12 @@ def main():
     ap.add_argument("--eager", action="store_true", help="time host-launched kernels only (no HIP graph)")
     ap.add_argument("--ranges", type=int, default=0, help="token ranges for decode (0 = planned)")
     ap.add_argument("--replays", type=int, default=12, help="timed replays of the K-step graph (at least 10)")
+    ap.add_argument("--custom", default="",
+                    help="a decode-only batch instead of --workload, e.g. 'hq=8,hkv=1,d=128,batch=64,kvmin=1024,"
+                         "kvmax=4096,mode=1' (kv lengths uniform in [kvmin, kvmax], seed 7, outlier channels)")
+    ap.add_argument("--extras", action="store_true",
+                    help="also time the kernels either side of the layer call on this batch's new tokens (RoPE alone, "
+                         "RoPE fused with the append) and a 64-page kv_cache_reorder; reported under `extras`")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (known traffic, for scaling rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -113,7 +163,14 @@ def main():
     wl, harness, ops = pkg.workloads, pkg.harness, pkg.ops
     torch.cuda.set_device(0)
 
-    bt, rng = wl.make_batch(args.workload)
+    if args.custom:
+        c = dict(hq=32, hkv=8, d=128, batch=64, kvmin=1024, kvmax=4096, mode=1)
+        c.update({k: int(v) for k, v in (kv.split("=") for kv in args.custom.split(","))})
+        lens = np.random.default_rng(7).integers(c["kvmin"], c["kvmax"] + 1, c["batch"])
+        bt, rng = wl.custom_batch(7, c["hq"], c["hkv"], c["d"], c["mode"], lens.tolist(), outliers=True)
+        bt.name = "custom(%s)" % args.custom
+    else:
+        bt, rng = wl.make_batch(args.workload)
     dev = harness.DeviceBatch(bt)
     # context already in the cache: quantised from seeded fp16 rows by the HIP append kernel
     dev.fill_history(rng, max_rows=1 << 15)
@@ -294,7 +351,7 @@ def main():
     }
     proj_us = float(np.mean(proj_replays)) if proj_replays else stages["o_proj"]["avg_us"]
     proj_bytes = hidden * hidden * 2
-    out["o_proj"] = {"kernel": "split_linear_kernel + linear_reduce_kernel" if proj_ws_bytes else "split_linear_kernel", "rows": int(bt.decoding_batches), "in_features": hidden,
+    out["o_proj"] = {"kernel": "wavek_linear_kernel + linear_reduce_kernel" if proj_ws_bytes else "wavek_linear_kernel", "rows": int(bt.decoding_batches), "in_features": hidden,
                      "out_features": hidden, "bound": "hbm", "weight_bytes": proj_bytes, "kernel_us": proj_us,
                      "achieved": proj_bytes / (proj_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": proj_bytes / (proj_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
@@ -307,6 +364,8 @@ def main():
                           "peak_tflops": 2500.0, "frac": fl / (pf_us * 1e-6) / 1e12 / 2500.0,
                           "kernel_us_replays": summary(prefill_replays) if prefill_replays else None,
                           "kernel_us_launch_loop": stages["prefill"]["avg_us"]}
+    if args.extras and not args.eager:
+        out["extras"] = extras(torch, ops, dev, bt, replay_times)
     if not args.no_cpu_baseline:
         oracle = entry.load_oracle()
         out["cpu_baseline"] = cpu_baseline(oracle, bt, q, dev.cache.cpu().numpy(), dev.scale.cpu().numpy())
