@@ -49,9 +49,11 @@ constexpr float kPShift = 14.0f;
 template <int D>
 struct PrefillTile {
     static constexpr int K_STRIDE = D + 8;
-    static constexpr int V_STRIDE = D + 32;
+    static constexpr int V_STRIDE = ((D + 32) * 2) % 128 == 64 ? D + 32 : D + 64;
 };
-static_assert((PrefillTile<128>::V_STRIDE * 2) % 256 == 64 && (PrefillTile<64>::V_STRIDE * 2) % 256 == 192, "V row stride");
+static_assert((PrefillTile<128>::V_STRIDE * 2) % 256 == 64 && (PrefillTile<64>::V_STRIDE * 2) % 256 == 192 &&
+                  (PrefillTile<96>::V_STRIDE * 2) % 256 == 64,
+              "V row stride");
 
 // sum over the wave of small non-negative integers, one ballot per bit (every lane of the wave must be here)
 __device__ __forceinline__ int wave_sum_small(int v)
@@ -179,8 +181,12 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     constexpr int GPT = D / 8;              // quantisation groups per token row
     constexpr int K_STRIDE = PrefillTile<D>::K_STRIDE; // halves per K row in LDS
     constexpr int V_STRIDE = PrefillTile<D>::V_STRIDE; // halves per V row in LDS (row-major, like K)
-    constexpr int UNITS = kBN * GPT / kPrefillThreads; // (token, group) units per thread, of K and of V each
-    constexpr int K_TSTEP = kPrefillThreads / GPT;     // tokens between a thread's units
+    // Staging: thread t takes group t % GPT of the tokens t / GPT, t / GPT + K_TSTEP, ...  With 12 groups per row
+    // (head_dim 96) the first 384 threads stage 32 tokens per pass and the last two waves stage nothing.
+    constexpr int K_TSTEP = GPT == 12 ? 32 : kPrefillThreads / GPT; // tokens between a thread's units
+    constexpr int STAGERS = K_TSTEP * GPT;                           // threads that stage (whole waves)
+    constexpr int UNITS = kBN / K_TSTEP;                             // (token, group) units per staging thread, of K and of V each
+    static_assert(STAGERS <= kPrefillThreads && STAGERS % 64 == 0 && UNITS * K_TSTEP == kBN, "staging units");
 
     // K is kept as an unevaluated sum hi + lo of two halves: hi = fp16(int8 * scale) and
     // lo = the rounding error of that product (exact, from one fused multiply-add), so that
@@ -225,8 +231,9 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     const float sm_scale = a.attn_scale * kLog2e;
 
     // this thread's (token, group) units of a tile: token u_t0 + u * K_TSTEP, group u_g, for K and for V alike
+    const bool stager = tid < STAGERS; // wave-uniform
     const int u_g = tid % GPT;
-    const int u_t0 = tid / GPT;
+    const int u_t0 = stager ? tid / GPT : 0;
     const uint32_t stride_s32 = (uint32_t)a.cache_stride_s; // the host checks that a tile's span fits 32 bits
     const uint32_t kstride16 = (uint32_t)a.key_stride_s, vstride16 = (uint32_t)a.value_stride_s;
     uint32_t u_off[UNITS];
@@ -309,6 +316,7 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         return cachestarts[table_base] + t_base;
     };
     auto load_tile = [&](int tile, int64_t row) {
+        if (!stager) return;
         const int left = kvlen - 1 - tile * kBN; // offset of the sequence's last token inside this tile
         if (KV16) {
             const half_t* bk = (const half_t*)a.current_key + row * a.key_stride_s + (int64_t)kvh * D;
@@ -351,6 +359,7 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     // UNITS + [0, UNITS) its V units.  Sliced so that the work can be spread between the MFMAs of phase 1.
     constexpr int N_SLICES = 2 * UNITS;
     auto store_slice = [&](int buf, int slice) {
+        if (!stager) return;
         half_t* const sK = smem + buf * TILE_HALVES;
         half_t* const sKlo = sK + K_HALVES;
         half_t* const sV = KV16 ? sKlo : sKlo + K_HALVES;
@@ -647,9 +656,8 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     } // items
 }
 
-// ---- the 16-column form: head dims whose accumulators and query fragments the kernel above cannot hold ----
-// head_dim 256 needs 128 accumulator and 64 query registers per lane with 32 columns per wave; head_dim 96 does not
-// divide into that kernel's 512 staging units.  Here a wave has 16 columns and the products run on
+// ---- the 16-column form: head_dim 256, whose accumulators and query fragments the kernel above cannot hold ----
+// (128 accumulator and 64 query registers per lane with 32 columns per wave).  Here a wave has 16 columns and the products run on
 // v_mfma_f32_16x16x32_f16: S^T tiles of 16 tokens x 16 columns (4 registers), O^T tiles of 16 channels x 16 columns.
 // Same decomposition otherwise (one workgroup = one kv head x a tile of query positions x all query heads of the
 // group: 128 columns; K/V tiles dequantised once per workgroup into one of two LDS buffers, one barrier per tile;
@@ -665,7 +673,7 @@ struct PrefillTile16 {
     static constexpr int K_STRIDE = D + 8;
     static constexpr int V_STRIDE = ((D + 32) * 2) % 128 == 64 ? D + 32 : D + 64; // an odd multiple of 64 bytes
 };
-static_assert((PrefillTile16<96>::V_STRIDE * 2) % 128 == 64 && (PrefillTile16<256>::V_STRIDE * 2) % 128 == 64, "V row stride");
+static_assert((PrefillTile16<256>::V_STRIDE * 2) % 128 == 64, "V row stride");
 } // namespace
 
 template <int D, int SRC, bool EXTRA>
@@ -1082,7 +1090,7 @@ int launch_prefill(const PrefillLaunch& a, hipStream_t stream)
     switch (a.head_dim) {
         case 64: return a.num_heads / a.num_kv_heads > kCols ? kLaunchNoKernel : launch_prefill_d<64>(a, stream);
         case 128: return a.num_heads / a.num_kv_heads > kCols ? kLaunchNoKernel : launch_prefill_d<128>(a, stream);
-        case 96: return launch_prefill16_d<96>(a, stream);
+        case 96: return a.num_heads / a.num_kv_heads > kCols ? kLaunchNoKernel : launch_prefill_d<96>(a, stream);
         case 256: return launch_prefill16_d<256>(a, stream);
         default: return kLaunchNoKernel;
     }
@@ -1133,8 +1141,8 @@ static int init_prefill16_d()
 int init_prefill_kernels()
 {
     if (int rc = init_prefill_d<64>()) return rc;
+    if (int rc = init_prefill_d<96>()) return rc;
     if (int rc = init_prefill_d<128>()) return rc;
-    if (int rc = init_prefill16_d<96>()) return rc;
     return init_prefill16_d<256>();
 }
 
