@@ -695,7 +695,7 @@ static int launch_decode_d(const DecodeLaunch& a, int stage, hipStream_t stream)
                 launch_decode_mfma(a, stream);
                 break;
             case kDecodeKernelQuad:
-                if (D != 128 && D != 256) return kLaunchNoKernel;
+                if (D != 64 && D != 128 && D != 256) return kLaunchNoKernel;
                 launch_decode_quad(a, stream);
                 break;
             case kDecodeKernelGeneral: {

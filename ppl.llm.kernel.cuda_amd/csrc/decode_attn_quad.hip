@@ -1,4 +1,4 @@
-// Decode attention over the int8 group-8 KV cache, variant for head_dim 128 (an even number of kv heads)
+// Decode attention over the int8 group-8 KV cache, variant for head_dim 64 and 128 (an even number of kv heads)
 // and 256, up to four query heads per kv head (MHA and the common GQA shapes; up to eight at head_dim 128
 // with kv heads in eights).  Same semantics, token ranges, pieces and workspace as decode_attn.hip
 // (reference: src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/kernel.cu:229-679,
@@ -94,23 +94,30 @@ __device__ __forceinline__ float quad_lane(float v)
 // GP: sets of four query heads per kv head (1 or 2); WP: pairs of kv heads per workgroup (4, 2 or 1); the workgroup
 // has WP * GP waves.  MASK: the additive attn_mask (kernel.cu:319-325), two more requests per block and lane.
 // HD: head_dim 128, or 256: the two half-waves then hold the two halves of ONE kv head's channels instead of two kv
-// heads, and a logit is the sum of the two half-waves' sums.
+// heads, and a logit is the sum of the two half-waves' sums; or 64: a kv head has four chunk lanes, so the two rows of a
+// half-wave are two groups of tokens (a block is 32 tokens, step j of a lane is token 16 (row) + 4 j + (lane in quad)),
+// the reduce-scatter ends after its two folds with four complete logits per lane, and the rows' token streams are
+// merged with the quad's at the end of a piece.
 template <bool PAGED, int GP, int WP, bool MASK, int HD>
 __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kernel(const DecodeLaunch a)
 {
     constexpr int D = HD;
     constexpr int KPW = HD == 256 ? 1 : 2; // kv heads per wave
+    constexpr bool H64 = HD == 64;         // four channel chunks per kv head: lane bit 4 is a second token group
+    constexpr int BLK = H64 ? 2 * kQuadBlock : kQuadBlock; // tokens per block
+    static_assert(!(H64 && (MASK || GP > 1)), "head_dim 64: one set of waves, no mask");
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wave = wave_id % WP;      // which pair of kv heads
     const int g_first = (wave_id / WP) * 4; // first query head (within the kv head's group) of this wave
     const int t4 = lane & 3;           // token within a step
-    const int chunk = (lane >> 2) & 7; // channels [16 chunk, 16 chunk + 16)
+    const int chunk = (lane >> 2) & (H64 ? 3 : 7); // channels [16 chunk, 16 chunk + 16)
     const int hsel = lane >> 5;        // which of the wave's two kv heads (head_dim 256: which half of the channels)
     // the head whose complete logits this lane receives from the reduce-scatter
     const int g_own = (((lane >> 2) & 1) << 1) | ((lane >> 3) & 1);
-    const int row_odd = (lane >> 4) & 1;
+    const int row_odd = (lane >> 4) & 1; // head_dim 64: the token group, tokens 16 row_odd + 4 j + t4 of a block
+    const int tok0 = t4 + (H64 ? 16 * row_odd : 0); // this lane's token of step 0
     const int G = (int)a.num_kv_repeats; // <= 4 * GP
     const int kvh = blockIdx.y * (KPW * WP) + wave * KPW + (KPW == 2 ? hsel : 0);
     const int ch0 = chunk * 16 + (KPW == 1 ? hsel * 128 : 0); // this lane's 16 channels
@@ -119,7 +126,7 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
     const const_i64_ptr cachestarts = as_constant(a.cachestarts);
     const int64_t kv_base = kvstarts[0];
     const int64_t total = stream_length(kvstarts[a.decoding_batches] - kv_base, a.decoding_batches);
-    const int64_t per = tokens_per_range(total, a.ranges, kQuadBlock, a.min_tokens_per_range);
+    const int64_t per = tokens_per_range(total, a.ranges, BLK, a.min_tokens_per_range);
     const int64_t r0 = (int64_t)blockIdx.x * per;
     if (r0 >= total) return;
     const int64_t r1 = (r0 + per < total) ? r0 + per : total;
@@ -140,11 +147,11 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
         const int64_t len = kvstarts[b + 1] - kv_base - first_token;
         const int64_t s_beg = sequence_origin(first_token, b);
         int64_t pa, pe;
-        piece_bounds(r0, r1, s_beg, len, kQuadBlock, pa, pe);
+        piece_bounds(r0, r1, s_beg, len, BLK, pa, pe);
         if (pe <= pa) continue;
         const int pa32 = (int)pa, pe32 = (int)pe;
-        const int nb = (pe32 - pa32 + kQuadBlock - 1) / kQuadBlock; // >= 1
-        const bool tail_partial = ((pe32 - pa32) & (kQuadBlock - 1)) != 0;
+        const int nb = (pe32 - pa32 + BLK - 1) / BLK; // >= 1
+        const bool tail_partial = ((pe32 - pa32) & (BLK - 1)) != 0;
 
         const int64_t table_base = PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b;
         const int64_t seq_row0 = PAGED ? 0 : cachestarts[b];
@@ -166,7 +173,7 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
         uint32_t vo[kTB], vo_sc[kTB];
 #pragma unroll
         for (int j = 0; j < kTB; ++j) {
-            vo[j] = (uint32_t)(4 * j + t4) * stride_s32 + lane_base;
+            vo[j] = (uint32_t)(4 * j + tok0) * stride_s32 + lane_base;
             vo_sc[j] = vo[j] >> 2;
         }
         // attn_mask: this lane's two complete logits belong to head g_own and the tokens 4 row_odd + t4 and + 8 of the
@@ -185,7 +192,7 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
         auto clamp_offsets = [&](int pos) { // tokens beyond the piece re-read its last token; their logits are masked
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
-                const int t = pos + 4 * j + t4;
+                const int t = pos + 4 * j + tok0;
                 const int tc = t < pe32 ? t : pe32 - 1;
                 vo[j] = (uint32_t)(tc - pos) * stride_s32 + lane_base;
                 vo_sc[j] = vo[j] >> 2;
@@ -292,6 +299,51 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
                 const float s0 = (float)sc.x, s1 = (float)sc.y; // the logit scale is applied to the two complete logits below
 #pragma unroll
                 for (int g = 0; g < 4; ++g) part[g][j] = __builtin_fmaf(d1[g], s1, d0[g] * s0);
+            }
+            if constexpr (H64) {
+                // four chunk lanes: after the two folds a lane holds the complete logits of head g_own for all four
+                // steps of its own tokens; nothing crosses the rows, whose lanes are separate token streams
+                float l[kTB];
+                float mx = kNegBig;
+#pragma unroll
+                for (int j = 0; j < kTB; ++j) {
+                    const float ra0 = fold_xor4(part[0][j], part[2][j]);
+                    const float ra1 = fold_xor4(part[1][j], part[3][j]);
+                    l[j] = fold_xor8(ra0, ra1) * logit_scale;
+                    if (beyond_piece) l[j] = kx.pos + 4 * j + tok0 < pe32 ? l[j] : -INFINITY;
+                    mx = fmaxf(mx, l[j]);
+                }
+                const float m_new = fmaxf(m_run, mx);
+                const bool moved = m_new > m_run;
+                float p[kTB];
+#pragma unroll
+                for (int j = 0; j < kTB; ++j) p[j] = __builtin_amdgcn_exp2f(l[j] - m_new);
+                if (__builtin_amdgcn_ballot_w64(moved) != 0) { // wave-uniform and rare: a running max moved
+                    float al[4];
+                    al[0] = __builtin_amdgcn_exp2f(m_run - m_new);
+                    l_run *= al[0];
+                    al[1] = dpp_f32<kDppRor8>(al[0]);
+                    al[2] = lane_xor4(al[0]);
+                    al[3] = lane_xor4(al[1]);
+#pragma unroll
+                    for (int s = 0; s < 4; ++s)
+#pragma unroll
+                        for (int c = 0; c < 16; ++c) acc[s][c] *= al[s];
+                }
+                m_run = m_new;
+                l_run += (p[0] + p[1]) + (p[2] + p[3]);
+                // all-gather of the heads over lane bits 3 and 2
+#pragma unroll
+                for (int j = 0; j < kTB; ++j) {
+                    prob[0][j] = p[j];
+                    prob[1][j] = dpp_f32<kDppRor8>(p[j]);
+                }
+#pragma unroll
+                for (int j = 0; j < kTB; ++j) {
+                    prob[2][j] = lane_xor4(prob[0][j]);
+                    prob[3][j] = lane_xor4(prob[1][j]);
+                }
+                return;
             }
             // reduce-scatter over the eight chunk lanes: lane bit 2 keeps heads {0,1} or {2,3}, bit 3 keeps
             // one of the pair, the row pair keeps steps {0,2} or {1,3}
@@ -409,7 +461,7 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
             // block of each other, so that the second set's requests find the lines in the cache levels
             // (every wave of the workgroup runs the same number of blocks).
             if (GP > 1) __syncthreads();
-            int npos = pos + (i + 1 < nb ? kQuadBlock : 0);
+            int npos = pos + (i + 1 < nb ? BLK : 0);
             if (tail_partial && i + 2 == nb) clamp_offsets(npos);
             request_k(kb, mkb, npos);
             logits_softmax(ka, mka, tail_partial && i + 1 == nb);
@@ -418,7 +470,7 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
             pin_acc();
             pos = npos;
             if (++i == nb) break;
-            npos = pos + (i + 1 < nb ? kQuadBlock : 0);
+            npos = pos + (i + 1 < nb ? BLK : 0);
             if (tail_partial && i + 2 == nb) clamp_offsets(npos);
             request_k(ka, mka, npos);
             logits_softmax(kb, mkb, tail_partial && i + 1 == nb);
@@ -439,11 +491,26 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
 
         // ---- end of the piece: exp-sum of the head over the row pair, (max, sum) of the four slots,
         // then the four token streams of the quad are merged ----
-        {
+        if constexpr (!H64) {
             float lx = l_run, ly = l_run;
             swap_rows(lx, ly);
             l_run = lx + ly;
         }
+        // head_dim 64: the two rows of a half-wave are two more token streams of the same heads and channels; their
+        // (max, sum, accumulators) are merged with those of the quad below (the swap hands a lane its own value and
+        // that of lane ^ 16, so a sum or a maximum of the two results needs no select)
+        auto across_rows_max = [&](float v) {
+            if constexpr (!H64) return v;
+            float x = v, y = v;
+            swap_rows(x, y);
+            return fmaxf(x, y);
+        };
+        auto across_rows_sum = [&](float v) {
+            if constexpr (!H64) return v;
+            float x = v, y = v;
+            swap_rows(x, y);
+            return x + y;
+        };
         float ms[4], lsum[4];
         ms[0] = m_run;
         lsum[0] = l_run;
@@ -460,10 +527,12 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
         for (int s = 0; s < 4; ++s) {
             float M = fmaxf(ms[s], dpp_f32<kDppXor1>(ms[s]));
             M = fmaxf(M, dpp_f32<kDppXor2>(M));
+            M = across_rows_max(M);
             const float w = __builtin_amdgcn_exp2f(ms[s] - M);
             float L = lsum[s] * w;
             L += dpp_f32<kDppXor1>(L);
             L += dpp_f32<kDppXor2>(L);
+            L = across_rows_sum(L);
             const float inv = L > 0.f ? 1.f / L : 0.f;
             float o[16];
 #pragma unroll
@@ -471,10 +540,10 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
                 float v = acc[s][c] * w;
                 v += dpp_f32<kDppXor1>(v);
                 v += dpp_f32<kDppXor2>(v);
-                o[c] = v * inv;
+                o[c] = across_rows_sum(v) * inv;
             }
             const int g = g_first + (g_own ^ s);
-            if (t4 == 0 && g < G) {
+            if (t4 == 0 && (!H64 || row_odd == 0) && g < G) {
                 const int h = kvh * G + g;
                 if (whole) {
                     typedef half_t half8_t __attribute__((ext_vector_type(8)));
@@ -528,6 +597,25 @@ void launch_decode_quad(const DecodeLaunch& a, hipStream_t stream)
         return;
     }
     const int waves = a.kv_heads_per_group / (a.head_dim == 256 ? 1 : 2);
+    if (a.head_dim == 64) { // no mask form: decode_quad_launch_ok sends masked steps to the general kernel
+        const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / (2 * waves)), 1);
+        const bool paged = a.cache_mode == 1;
+        switch (waves) {
+        case 4:
+            if (paged) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1, 4, false, 64>), grid, dim3(kWave * 4), 0, stream, a);
+            else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1, 4, false, 64>), grid, dim3(kWave * 4), 0, stream, a);
+            break;
+        case 2:
+            if (paged) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1, 2, false, 64>), grid, dim3(kWave * 2), 0, stream, a);
+            else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1, 2, false, 64>), grid, dim3(kWave * 2), 0, stream, a);
+            break;
+        default:
+            if (paged) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1, 1, false, 64>), grid, dim3(kWave), 0, stream, a);
+            else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1, 1, false, 64>), grid, dim3(kWave), 0, stream, a);
+            break;
+        }
+        return;
+    }
     if (a.head_dim == 256) {
         switch (waves) {
         case 4: launch_decode_quad_wp<4, 256>(a, stream); break;

@@ -14,13 +14,13 @@ int largest_pow2_divisor_upto(int64_t n, int cap)
     return r;
 }
 
-// head_dim 128 with an even number of kv heads, or head_dim 256: up to four query heads per kv head on one set of
-// waves; head_dim 128 with kv heads in eights: up to eight on two sets
+// head_dim 64 or 128 with an even number of kv heads, or head_dim 256: up to four query heads per kv head on one set
+// of waves; head_dim 128 with kv heads in eights: up to eight on two sets
 bool quad_serves(int64_t head_dim, int64_t g, int64_t num_kv_heads)
 {
     if (head_dim == 256) return g <= 4;
-    if (head_dim != 128 || num_kv_heads % 2 != 0) return false;
-    return g <= 4 || (g <= 8 && num_kv_heads % 8 == 0);
+    if ((head_dim != 128 && head_dim != 64) || num_kv_heads % 2 != 0) return false;
+    return g <= 4 || (head_dim == 128 && g <= 8 && num_kv_heads % 8 == 0);
 }
 
 } // namespace
@@ -46,8 +46,8 @@ bool decode_choose(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, in
         // Many query heads per kv head: their VALU arithmetic outweighs the cache stream, so they become MFMA
         // columns (five and more; three and four as well where the kv heads do not come in pairs, which the quad
         // kernel needs).  Up to four: the quad kernel, whose row loads stream whole lines.  Everything else
-        // (head_dim 64 and 96, odd kv-head counts with one or two query heads each, more than 32 query heads per
-        // kv head) stays on the general kernel.
+        // (head_dim 96, head_dim 64 with more than four query heads per kv head, odd kv-head counts with one or two
+        // query heads each, more than 32 query heads per kv head) stays on the general kernel.
         if (head_dim == 128 && g <= kDecodeMfmaColumns && (g >= 5 || (g >= 3 && num_kv_heads % 2 != 0)))
             kernel = g <= kDecodeMfma16Columns ? kDecodeKernelMfma16 : kDecodeKernelMfma32;
         else if (quad_serves(head_dim, g, num_kv_heads) && g <= 4)
@@ -78,7 +78,7 @@ bool decode_choose(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, in
             c.kv_heads_per_group = per_wave * (pairs % 4 == 0 ? 4 : (pairs % 2 == 0 ? 2 : 1));
             c.q_heads_per_pass = g <= 1 ? 1 : (g <= 2 ? 2 : (g <= 4 ? 4 : 8)); // rows of the 4x4x4 products in use
             c.num_passes = 1;
-            c.wg_tokens = kDecodeQuadTokens;
+            c.wg_tokens = head_dim == 64 ? 2 * kDecodeQuadTokens : kDecodeQuadTokens; // head_dim 64: blocks of 32 tokens
             c.wgs_per_cu = (head_dim == 256 ? 8 : 16) / c.kv_heads_per_group;
             break;
         }
@@ -103,6 +103,7 @@ bool decode_quad_launch_ok(const DecodeLaunch& a)
 {
     if (a.output_stride_s % 8 != 0 || (reinterpret_cast<uintptr_t>(a.output) & 15u) != 0) return false;
     if (a.attn_mask != nullptr) {
+        if (a.head_dim == 64) return false; // no mask form at head_dim 64
         if (a.num_kv_repeats > 4 || a.mask_stride_h < 0) return false;
         if (((double)a.num_heads * (double)a.mask_stride_h + 64.0) * 2.0 >= 4294967296.0) return false;
     }

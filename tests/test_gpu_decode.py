@@ -44,6 +44,8 @@ SHAPES = [
     (8, 2, 128), (6, 6, 128), (24, 12, 128), (16, 4, 128),
     # ... and with head_dim 256 (a wave per kv head)
     (16, 8, 256), (16, 16, 256), (3, 1, 256), (8, 2, 256), (5, 1, 256),
+    # ... and with head_dim 64 (blocks of 32 tokens: the rows of a half-wave are two token groups)
+    (32, 8, 64), (8, 4, 64), (6, 2, 64), (16, 16, 64), (18, 6, 64),
 ]
 
 
@@ -72,6 +74,8 @@ KERNEL_NAMES = {1: "decode_attention_kernel", 2: "decode_attention_quad_kernel",
     ((96, 4, 128), (1, 4)),         # 24 per kv head: three passes of the general kernel, or 32 columns
     ((16, 8, 256), (1, 2)),
     ((6, 3, 128), (1, 3)),
+    ((32, 8, 64), (1, 2)),
+    ((4, 4, 64), (1, 2)),
 ])
 def test_decode_requested_kernel(pkg, oracle, shape, kernels):
     """Every token-range kernel that serves a shape, requested through the C ABI: the library reports that it
@@ -88,7 +92,7 @@ def test_decode_requested_kernel(pkg, oracle, shape, kernels):
             assert_attention_close(got, ref, "shape %s kernel %d ranges %d" % (shape, k, plan.num_token_ranges))
 
 
-@pytest.mark.parametrize("shape", [(16, 4, 128), (8, 2, 128), (12, 6, 128), (8, 4, 256)])
+@pytest.mark.parametrize("shape", [(16, 4, 128), (8, 2, 128), (12, 6, 128), (8, 4, 256), (8, 4, 64)])
 def test_decode_output_rows_aligned_to_8_bytes_only(pkg, oracle, shape):
     """The C ABI admits output rows that are 8-byte aligned; the quad kernel needs 16.  Such a call runs on the
     general kernel, and the token-range kernel and the combine kernel must then cut the ranges by the same unit

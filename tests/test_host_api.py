@@ -154,7 +154,8 @@ def test_decode_plan_names_its_kernel(pkg, hip_lib):
     L = pkg._lib
     auto = {(32, 8, 128): L.DECODE_KERNEL_QUAD, (32, 32, 128): L.DECODE_KERNEL_QUAD, (64, 8, 128): L.DECODE_KERNEL_MFMA16,
             (96, 4, 128): L.DECODE_KERNEL_MFMA32, (9, 3, 128): L.DECODE_KERNEL_MFMA16, (6, 3, 128): L.DECODE_KERNEL_GENERAL,
-            (8, 8, 64): L.DECODE_KERNEL_GENERAL, (12, 4, 96): L.DECODE_KERNEL_GENERAL, (16, 16, 256): L.DECODE_KERNEL_QUAD,
+            (8, 8, 64): L.DECODE_KERNEL_QUAD, (32, 8, 64): L.DECODE_KERNEL_QUAD, (40, 8, 64): L.DECODE_KERNEL_GENERAL,
+            (9, 3, 64): L.DECODE_KERNEL_GENERAL, (12, 4, 96): L.DECODE_KERNEL_GENERAL, (16, 16, 256): L.DECODE_KERNEL_QUAD,
             (40, 8, 256): L.DECODE_KERNEL_GENERAL, (66, 2, 128): L.DECODE_KERNEL_GENERAL}
     for (hq, hkv, d), want in auto.items():
         assert pkg.ops.decode_plan(16, hq, hkv, d, 4096, cus=256).kernel == want, (hq, hkv, d)
@@ -163,7 +164,7 @@ def test_decode_plan_names_its_kernel(pkg, hip_lib):
                                   L.DECODE_KERNEL_MFMA16: (4, 16, 256), L.DECODE_KERNEL_MFMA32: (4, 32, 256)}.items():
         plan = pkg.ops.decode_plan(32, 64, 8, 128, 32768, cus=256, kernel=k)
         assert (plan.kernel, plan.kv_heads_per_group, plan.q_heads_per_pass, plan.num_token_ranges) == (k, kvhb, gt, ranges)
-    for hq, hkv, d, k in [(32, 8, 64, L.DECODE_KERNEL_QUAD), (32, 8, 64, L.DECODE_KERNEL_MFMA16),
+    for hq, hkv, d, k in [(40, 8, 64, L.DECODE_KERNEL_QUAD), (32, 8, 96, L.DECODE_KERNEL_QUAD), (32, 8, 64, L.DECODE_KERNEL_MFMA16),
                           (40, 2, 128, L.DECODE_KERNEL_MFMA16), (66, 2, 128, L.DECODE_KERNEL_MFMA32),
                           (10, 2, 128, L.DECODE_KERNEL_QUAD), (3, 3, 128, L.DECODE_KERNEL_QUAD), (32, 8, 128, 5), (32, 8, 128, -1)]:
         with pytest.raises(pkg.ops.PmxError):
