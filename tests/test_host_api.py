@@ -218,3 +218,14 @@ def test_c_entry_points_reject_bad_arguments_without_launching(pkg, hip_lib):
     assert hip_lib.pmxhip_prefill_attention(ctypes.byref(f), None) == 0  # no prefill sequences (kernel.cu:2130)
     f.batch, f.max_seqlen, f.head_dim = 4, 8, 96
     assert hip_lib.pmxhip_prefill_attention(ctypes.byref(f), None) == 2
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asking for more ends with a message that says so, before any device work."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2
+    assert "ONE GPU" in r.stderr and r.stdout.strip() == ""
