@@ -123,6 +123,8 @@ int pmxhip_init(void)
     void* ptr = nullptr;
     if (int rc = static_scratch("init", nullptr, &ptr)) return rc;
     (void)current_compute_units();
+    int device = 0;
+    if (hipGetDevice(&device) == hipSuccess) (void)pmxhip::init_linear_library(device);
     return PMXHIP_SUCCESS;
 }
 
@@ -642,7 +644,10 @@ int pmxhip_rope_kv_cache_quantize(const pmxhip_rope_params* rope, const pmxhip_k
 int64_t pmxhip_row_parallel_linear_workspace_size(int64_t m, int64_t in_features, int64_t out_features)
 {
     if (m <= 0 || in_features <= 0 || out_features <= 0) return 0;
-    return pmxhip::linear_workspace_bytes(m, out_features, in_features, current_compute_units());
+    const int64_t own = pmxhip::linear_workspace_bytes(m, out_features, in_features, current_compute_units());
+    if (m >= pmxhip::kLinearLibraryRows && pmxhip::linear_library_available() && own < pmxhip::kLinearLibraryWorkspace)
+        return pmxhip::kLinearLibraryWorkspace;
+    return own;
 }
 
 int pmxhip_row_parallel_linear(pmxhip_stream_t stream, const void* input, const void* weight, const void* bias, int64_t m,
@@ -671,6 +676,13 @@ int pmxhip_row_parallel_linear(pmxhip_stream_t stream, const void* input, const 
     a.input_stride = input_stride;
     a.weight_stride = weight_stride;
     a.output_stride = output_stride;
+    // many rows: a compute-bound GEMM for the vendor library, when it can be loaded and takes the problem
+    if (m >= pmxhip::kLinearLibraryRows && pmxhip::linear_library_available()) {
+        int device = 0;
+        if (hipGetDevice(&device) != hipSuccess) return fail(PMXHIP_OTHER_ERROR, "row_parallel_linear: no current device");
+        const int rc = pmxhip::launch_linear_library(a, device, workspace, workspace ? workspace_size : 0, stream);
+        if (rc != pmxhip::kLaunchNoKernel) return launch_result("row_parallel_linear", rc);
+    }
     return launch_result("row_parallel_linear",
                          pmxhip::launch_linear(a, current_compute_units(), workspace, workspace ? workspace_size : 0, stream));
 }

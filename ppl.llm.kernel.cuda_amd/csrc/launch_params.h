@@ -185,6 +185,13 @@ inline int ensure_dynamic_lds(const void* kernel, int bytes, hipStream_t stream,
     return kLaunchOk;
 }
 
+// Rows from which the output projection is a compute-bound GEMM and goes to the vendor library when that can be
+// loaded (linear_library.cpp); up to here this build's weight-streaming kernels are as fast or faster.
+constexpr int64_t kLinearLibraryRows = 384;
+constexpr int64_t kLinearLibraryWorkspace = 64 << 20; // what the library is offered when the caller asks how much to bring
+bool linear_library_available();
+int init_linear_library(int device);
+int launch_linear_library(const LinearLaunch& a, int device, void* workspace, int64_t workspace_bytes, hipStream_t stream);
 int launch_kv_quantize(const QuantLaunch& a, int compute_units, hipStream_t stream);
 int launch_rope(const RopeLaunch& a, int compute_units, hipStream_t stream);
 void launch_page_copy(const PageCopyLaunch& a, hipStream_t stream);

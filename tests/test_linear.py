@@ -74,7 +74,9 @@ def test_c_entry_point_rejects_bad_arguments_without_launching(pkg, hip_lib):
 @pytest.mark.parametrize("shape", [(1, 16, 32), (7, 48, 96), (128, 4096, 4096), (64, 1024, 8192), (200, 256, 512),
                                    (128, 14336 // 8, 4096), (3, 4096, 32), (129, 32, 4064), (17, 64, 64), (128, 128, 3136),
                                    (300, 8192, 1024), (5, 64, 2240), (1, 64, 512), (16, 128, 1024), (17, 64, 1536), (33, 192, 2048),
-                                   (65, 64, 512), (130, 192, 2048), (240, 4096, 4096)])
+                                   (65, 64, 512), (130, 192, 2048), (240, 4096, 4096),
+                                   # many rows: the compute-bound form (the vendor library where it loads)
+                                   (384, 256, 512), (1000, 512, 1024), (2500, 1024, 2048)])
 def test_hip_linear_matches_oracle(pkg, oracle, shape):
     import torch
     m, n, k = shape
@@ -103,12 +105,13 @@ def test_hip_linear_matches_oracle(pkg, oracle, shape):
 
 
 @pytest.mark.gpu
-def test_hip_linear_strided_rows_and_attention_hand_off(pkg, oracle):
+@pytest.mark.parametrize("m", [37, 700])
+def test_hip_linear_strided_rows_and_attention_hand_off(pkg, oracle, m):
     """Rows with padding between them (the strides of the C ABI), and the attention output (B, Hq, D) used in place
-    as the (B, Hq * D) input."""
+    as the (B, Hq * D) input; a decode-sized and a prefill-sized row count."""
     import torch
     rng = np.random.default_rng(7)
-    m, hq, d, n = 37, 8, 64, 128
+    hq, d, n = 8, 64, 128
     k = hq * d
     a, w, b = draw(rng, m, n, k)
     buf_in = torch.zeros((m, k + 64), dtype=torch.float16, device="cuda")
