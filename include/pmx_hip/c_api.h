@@ -447,14 +447,20 @@ PMXHIP_API int pmxhip_rope_kv_cache_quantize(const pmxhip_rope_params* rope, con
  * one rank, an all-reduce (one GPU here, so none).  The attention output (B, Hq * D) is this call's input in
  * place.  bias may be NULL.  Strides are in halves per row.  Needs N % 16 == 0, K % 32 == 0, 16-byte aligned
  * rows of input and weight and 8-byte aligned rows of output and bias; anything else returns
- * PMXHIP_UNSUPPORTED.  Written for the decode step (M up to a few hundred rows: bound by streaming the
- * K * N * 2 weight bytes); larger M is served 128 rows at a time.
+ * PMXHIP_UNSUPPORTED.  The kernels of this library are written for the decode step (M up to a few hundred rows:
+ * bound by streaming the K * N * 2 weight bytes).  From 384 rows on the problem is a compute-bound GEMM and goes to
+ * hipBLASLt, as the reference's goes to cublasLt, if libhipblaslt.so can be loaded at that moment (dlopen; there is
+ * no link-time dependency); without it, or when it declines the problem, the same kernels serve M 128 rows at a
+ * time.  The first such call of a process on a device creates the library's handle and must not come under stream
+ * capture (pmxhip_init makes it).
  * workspace: at decode sizes there are fewer blocks of 64 output columns than CUs, so the k range is split over
  * several workgroups whose float32 partial tiles pass through `workspace` (the role of the reference's
  * cublas_workspace argument) and are added in a fixed order by a second kernel.
  * pmxhip_row_parallel_linear_workspace_size gives the bytes that serve (M, in_features, out_features) on the
  * current device (0 = none needed); with a NULL or smaller workspace the call still computes the same function,
- * one k range per column block (slower at decode sizes).  The workspace needs 16-byte alignment and no clearing. */
+ * one k range per column block (slower at decode sizes).  For M from 384 rows on the figure is what the vendor
+ * library is offered as its own workspace (64 MiB; it picks an algorithm that fits what it is given).  The workspace
+ * needs 16-byte alignment and no clearing. */
 PMXHIP_API int64_t pmxhip_row_parallel_linear_workspace_size(int64_t m, int64_t in_features, int64_t out_features);
 PMXHIP_API int pmxhip_row_parallel_linear(pmxhip_stream_t stream, const void* input, const void* weight, const void* bias,
                                           int64_t m, int64_t in_features, int64_t out_features, int64_t input_stride,
