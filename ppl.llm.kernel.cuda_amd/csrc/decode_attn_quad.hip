@@ -82,6 +82,11 @@ __device__ __forceinline__ float sum_halves(float v)
     const u32x2_t r = __builtin_amdgcn_permlane32_swap(bitcast<uint32_t>(v), bitcast<uint32_t>(v), false, false);
     return bitcast<float>(r[0]) + bitcast<float>(r[1]);
 }
+// value of the lane with bits 2 and 3 cleared (the chunk lane that holds head 0): and 0x13, or 0, xor 0
+__device__ __forceinline__ float from_head0_lane(float v)
+{
+    return bitcast<float>(__builtin_amdgcn_ds_swizzle(bitcast<int>(v), 0x13));
+}
 // value held by quad lane i (compile-time i)
 template <int I>
 __device__ __forceinline__ float quad_lane(float v)
@@ -98,7 +103,10 @@ __device__ __forceinline__ float quad_lane(float v)
 // half-wave are two groups of tokens (a block is 32 tokens, step j of a lane is token 16 (row) + 4 j + (lane in quad)),
 // the reduce-scatter ends after its two folds with four complete logits per lane, and the rows' token streams are
 // merged with the quad's at the end of a piece.
-template <bool PAGED, int GP, int WP, bool MASK, int HD>
+// NS: head slots a lane accumulates: 4, or 1 when every kv head has ONE query head (MHA): the lanes that hold the
+// complete logits of the three absent heads then take head 0's probabilities (one swizzle per value instead of the
+// all-gather) and a single set of 16 accumulators -- a quarter of the PV arithmetic.
+template <bool PAGED, int GP, int WP, bool MASK, int HD, int NS = 4>
 __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kernel(const DecodeLaunch a)
 {
     constexpr int D = HD;
@@ -106,6 +114,8 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
     constexpr bool H64 = HD == 64;         // four channel chunks per kv head: lane bit 4 is a second token group
     constexpr int BLK = H64 ? 2 * kQuadBlock : kQuadBlock; // tokens per block
     static_assert(!(H64 && (MASK || GP > 1)), "head_dim 64: one set of waves, no mask");
+    constexpr bool ONE = NS == 1;
+    static_assert(NS == 4 || (NS == 1 && GP == 1), "head slots");
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -268,13 +278,13 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
         // online-softmax state: m_run / l_run for head g_own only (l_run over this lane's own logits);
         // acc[s] belongs to head g_first + (g_own ^ s)
         float m_run = kNegBig, l_run = 0.f;
-        float acc[4][16];
+        float acc[NS][16];
 #pragma unroll
-        for (int s = 0; s < 4; ++s)
+        for (int s = 0; s < NS; ++s)
 #pragma unroll
             for (int c = 0; c < 16; ++c) acc[s][c] = 0.f;
 
-        float prob[4][kTB]; // [slot][step]: probabilities of this lane's own tokens
+        float prob[NS][kTB]; // [slot][step]: probabilities of this lane's own tokens
         // loads in flight when a block's logits start: its own, the V block before it and the next K block;
         // a K block has two more requests with the mask
         constexpr int kMoreK = MASK ? 4 : 0, kMoreV = MASK ? 2 : 0;
@@ -322,26 +332,35 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
                     float al[4];
                     al[0] = __builtin_amdgcn_exp2f(m_run - m_new);
                     l_run *= al[0];
-                    al[1] = dpp_f32<kDppRor8>(al[0]);
-                    al[2] = lane_xor4(al[0]);
-                    al[3] = lane_xor4(al[1]);
+                    if constexpr (ONE) {
+                        al[0] = from_head0_lane(al[0]);
+                    } else {
+                        al[1] = dpp_f32<kDppRor8>(al[0]);
+                        al[2] = lane_xor4(al[0]);
+                        al[3] = lane_xor4(al[1]);
+                    }
 #pragma unroll
-                    for (int s = 0; s < 4; ++s)
+                    for (int s = 0; s < NS; ++s)
 #pragma unroll
                         for (int c = 0; c < 16; ++c) acc[s][c] *= al[s];
                 }
                 m_run = m_new;
                 l_run += (p[0] + p[1]) + (p[2] + p[3]);
-                // all-gather of the heads over lane bits 3 and 2
+                if constexpr (ONE) {
 #pragma unroll
-                for (int j = 0; j < kTB; ++j) {
-                    prob[0][j] = p[j];
-                    prob[1][j] = dpp_f32<kDppRor8>(p[j]);
-                }
+                    for (int j = 0; j < kTB; ++j) prob[0][j] = from_head0_lane(p[j]);
+                } else {
+                    // all-gather of the heads over lane bits 3 and 2
 #pragma unroll
-                for (int j = 0; j < kTB; ++j) {
-                    prob[2][j] = lane_xor4(prob[0][j]);
-                    prob[3][j] = lane_xor4(prob[1][j]);
+                    for (int j = 0; j < kTB; ++j) {
+                        prob[0][j] = p[j];
+                        prob[1][j] = dpp_f32<kDppRor8>(p[j]);
+                    }
+#pragma unroll
+                    for (int j = 0; j < kTB; ++j) {
+                        prob[2][j] = lane_xor4(prob[0][j]);
+                        prob[3][j] = lane_xor4(prob[1][j]);
+                    }
                 }
                 return;
             }
@@ -388,11 +407,15 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
                 float al[4];
                 al[0] = __builtin_amdgcn_exp2f(m_run - m_new);
                 l_run *= al[0];
-                al[1] = dpp_f32<kDppRor8>(al[0]);
-                al[2] = lane_xor4(al[0]);
-                al[3] = lane_xor4(al[1]);
+                if constexpr (ONE) {
+                    al[0] = from_head0_lane(al[0]);
+                } else {
+                    al[1] = dpp_f32<kDppRor8>(al[0]);
+                    al[2] = lane_xor4(al[0]);
+                    al[3] = lane_xor4(al[1]);
+                }
 #pragma unroll
-                for (int s = 0; s < 4; ++s)
+                for (int s = 0; s < NS; ++s)
 #pragma unroll
                     for (int c = 0; c < 16; ++c) acc[s][c] *= al[s];
             }
@@ -402,13 +425,20 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
             float q0 = p0, q1 = p1;
             swap_rows(p0, q0); // p0 = step 0, q0 = step 1
             swap_rows(p1, q1); // p1 = step 2, q1 = step 3
-            prob[0][0] = p0; prob[0][1] = q0; prob[0][2] = p1; prob[0][3] = q1;
+            if constexpr (ONE) {
+                prob[0][0] = from_head0_lane(p0);
+                prob[0][1] = from_head0_lane(q0);
+                prob[0][2] = from_head0_lane(p1);
+                prob[0][3] = from_head0_lane(q1);
+            } else {
+                prob[0][0] = p0; prob[0][1] = q0; prob[0][2] = p1; prob[0][3] = q1;
 #pragma unroll
-            for (int j = 0; j < kTB; ++j) prob[1][j] = dpp_f32<kDppRor8>(prob[0][j]);
+                for (int j = 0; j < kTB; ++j) prob[1][j] = dpp_f32<kDppRor8>(prob[0][j]);
 #pragma unroll
-            for (int j = 0; j < kTB; ++j) {
-                prob[2][j] = lane_xor4(prob[0][j]);
-                prob[3][j] = lane_xor4(prob[1][j]);
+                for (int j = 0; j < kTB; ++j) {
+                    prob[2][j] = lane_xor4(prob[0][j]);
+                    prob[3][j] = lane_xor4(prob[1][j]);
+                }
             }
         };
 
@@ -430,7 +460,7 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
                 const half2_t sc = bitcast<half2_t>(vx.sc[j]);
                 const float sv0 = (float)sc.x, sv1 = (float)sc.y;
 #pragma unroll
-                for (int s = 0; s < 4; ++s) {
+                for (int s = 0; s < NS; ++s) {
                     const float w0 = prob[s][j] * sv0, w1 = prob[s][j] * sv1;
 #pragma unroll
                     for (int c = 0; c < 8; ++c) {
@@ -446,7 +476,7 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
         // copies all 64 of them twice per loop iteration (8 % of the loop's instructions).
         auto pin_acc = [&]() {
 #pragma unroll
-            for (int s = 0; s < 4; ++s)
+            for (int s = 0; s < NS; ++s)
 #pragma unroll
                 for (int c = 0; c < 16; ++c) asm volatile("" : "+v"(acc[s][c]));
         };
@@ -514,17 +544,22 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
         float ms[4], lsum[4];
         ms[0] = m_run;
         lsum[0] = l_run;
-        ms[1] = dpp_f32<kDppRor8>(ms[0]);
-        lsum[1] = dpp_f32<kDppRor8>(lsum[0]);
-        ms[2] = lane_xor4(ms[0]);
-        ms[3] = lane_xor4(ms[1]);
-        lsum[2] = lane_xor4(lsum[0]);
-        lsum[3] = lane_xor4(lsum[1]);
+        if constexpr (ONE) { // head 0's state, which the lanes of the absent heads take from its chunk lane
+            ms[0] = from_head0_lane(ms[0]);
+            lsum[0] = from_head0_lane(lsum[0]);
+        } else {
+            ms[1] = dpp_f32<kDppRor8>(ms[0]);
+            lsum[1] = dpp_f32<kDppRor8>(lsum[0]);
+            ms[2] = lane_xor4(ms[0]);
+            ms[3] = lane_xor4(ms[1]);
+            lsum[2] = lane_xor4(lsum[0]);
+            lsum[3] = lane_xor4(lsum[1]);
+        }
 
         const bool whole = (pa == 0) && (pe == len);
         const int64_t piece = (int64_t)blockIdx.x + b;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
+        for (int s = 0; s < NS; ++s) {
             float M = fmaxf(ms[s], dpp_f32<kDppXor1>(ms[s]));
             M = fmaxf(M, dpp_f32<kDppXor2>(M));
             M = across_rows_max(M);
@@ -542,7 +577,7 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
                 v += dpp_f32<kDppXor2>(v);
                 o[c] = across_rows_sum(v) * inv;
             }
-            const int g = g_first + (g_own ^ s);
+            const int g = ONE ? 0 : g_first + (g_own ^ s);
             if (t4 == 0 && (!H64 || row_odd == 0) && g < G) {
                 const int h = kvh * G + g;
                 if (whole) {
@@ -579,11 +614,14 @@ static void launch_decode_quad_wp(const DecodeLaunch& a, hipStream_t stream)
     constexpr int KPW = HD == 256 ? 1 : 2;
     const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / (KPW * WP)), 1);
     const bool paged = a.cache_mode == 1, mask = a.attn_mask != nullptr;
+    const bool one = a.num_kv_repeats == 1; // MHA: a single head slot per lane
     if (paged) {
         if (mask) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1, WP, true, HD>), grid, dim3(kWave * WP), 0, stream, a);
+        else if (one) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1, WP, false, HD, 1>), grid, dim3(kWave * WP), 0, stream, a);
         else hipLaunchKernelGGL((decode_attention_quad_kernel<true, 1, WP, false, HD>), grid, dim3(kWave * WP), 0, stream, a);
     } else {
         if (mask) hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1, WP, true, HD>), grid, dim3(kWave * WP), 0, stream, a);
+        else if (one) hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1, WP, false, HD, 1>), grid, dim3(kWave * WP), 0, stream, a);
         else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 1, WP, false, HD>), grid, dim3(kWave * WP), 0, stream, a);
     }
 }
