@@ -732,18 +732,15 @@ static int launch_decode_d(const DecodeLaunch& a, int stage, hipStream_t stream)
 template <int D, int GT>
 static int init_decode_dgt()
 {
-    hipError_t e = hipSuccess;
+    int rc = kLaunchOk;
     auto one = [&](const void* k, std::atomic<int>& ready) {
-        if (e == hipSuccess && ready.load() == 0) {
-            e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)decode_lds_bytes(D, GT));
-            if (e == hipSuccess) ready.store(1);
-        }
+        if (rc == kLaunchOk) rc = set_dynamic_lds_once(k, (int)decode_lds_bytes(D, GT), ready);
     };
     one((const void*)decode_attention_kernel<D, GT, true, true>, decode_variant_ready<D, GT, true, true>());
     one((const void*)decode_attention_kernel<D, GT, true, false>, decode_variant_ready<D, GT, true, false>());
     one((const void*)decode_attention_kernel<D, GT, false, true>, decode_variant_ready<D, GT, false, true>());
     one((const void*)decode_attention_kernel<D, GT, false, false>, decode_variant_ready<D, GT, false, false>());
-    return e == hipSuccess ? kLaunchOk : kLaunchNoKernel;
+    return rc;
 }
 template <int D>
 static int init_decode_d()

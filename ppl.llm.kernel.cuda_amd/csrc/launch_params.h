@@ -169,20 +169,35 @@ struct LinearLaunch {
 int launch_linear(const LinearLaunch& a, int compute_units, void* workspace, int64_t workspace_bytes, hipStream_t stream);
 int64_t linear_workspace_bytes(int64_t m, int64_t n, int64_t k, int compute_units);
 
-// The one-time hipFuncSetAttribute of a kernel whose dynamic LDS exceeds the default limit.  It runs before the
-// kernel's first launch in the process (one GPU per process) and never while `stream` is being captured into a
-// graph: a caller that captures first gets kLaunchNeedsWarmup and calls pmxhip_init() or one eager step before.
+// The one-time hipFuncSetAttribute of a kernel whose dynamic LDS exceeds the default limit: once per kernel and
+// device (`ready` holds a bit per device, up to 32 devices in a process).  It runs before the kernel's first launch
+// on the device and never while `stream` is being captured into a graph: a caller that captures first gets
+// kLaunchNeedsWarmup and calls pmxhip_init() or one eager step before.
+inline int current_device_bit()
+{
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess) return 0;
+    return 1 << (device & 31);
+}
+inline int set_dynamic_lds_once(const void* kernel, int bytes, std::atomic<int>& ready)
+{
+    const int bit = current_device_bit();
+    if (bit == 0) return kLaunchNoKernel;
+    if (ready.load(std::memory_order_acquire) & bit) return kLaunchOk;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return kLaunchNoKernel;
+    ready.fetch_or(bit, std::memory_order_release);
+    return kLaunchOk;
+}
 inline int ensure_dynamic_lds(const void* kernel, int bytes, hipStream_t stream, std::atomic<int>& ready)
 {
-    if (ready.load(std::memory_order_acquire) != 0) return kLaunchOk;
+    const int bit = current_device_bit();
+    if (bit != 0 && (ready.load(std::memory_order_acquire) & bit)) return kLaunchOk;
     hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &st) != hipSuccess || st != hipStreamCaptureStatusNone) {
         (void)hipGetLastError();
         return kLaunchNeedsWarmup;
     }
-    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return kLaunchNoKernel;
-    ready.store(1, std::memory_order_release);
-    return kLaunchOk;
+    return set_dynamic_lds_once(kernel, bytes, ready);
 }
 
 // Rows from which the output projection is a compute-bound GEMM and goes to the vendor library when that can be

@@ -1099,13 +1099,8 @@ int launch_prefill(const PrefillLaunch& a, hipStream_t stream)
 template <int D, int SRC, bool EXTRA>
 static int init_prefill_variant()
 {
-    std::atomic<int>& ready = prefill_variant_ready<D, SRC, EXTRA>();
-    if (ready.load() != 0) return kLaunchOk;
-    if (hipFuncSetAttribute((const void*)prefill_attention_kernel<D, SRC, EXTRA>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)prefill_lds_bytes<D, SRC>()) != hipSuccess)
-        return kLaunchNoKernel;
-    ready.store(1);
-    return kLaunchOk;
+    return set_dynamic_lds_once((const void*)prefill_attention_kernel<D, SRC, EXTRA>, (int)prefill_lds_bytes<D, SRC>(),
+                                prefill_variant_ready<D, SRC, EXTRA>());
 }
 template <int D>
 static int init_prefill_d()
@@ -1120,13 +1115,8 @@ static int init_prefill_d()
 template <int D, int SRC, bool EXTRA>
 static int init_prefill16_variant()
 {
-    std::atomic<int>& ready = prefill16_variant_ready<D, SRC, EXTRA>();
-    if (ready.load() != 0) return kLaunchOk;
-    if (hipFuncSetAttribute((const void*)prefill_attention16_kernel<D, SRC, EXTRA>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)prefill16_lds_bytes<D, SRC>()) != hipSuccess)
-        return kLaunchNoKernel;
-    ready.store(1);
-    return kLaunchOk;
+    return set_dynamic_lds_once((const void*)prefill_attention16_kernel<D, SRC, EXTRA>, (int)prefill16_lds_bytes<D, SRC>(),
+                                prefill16_variant_ready<D, SRC, EXTRA>());
 }
 template <int D>
 static int init_prefill16_d()
