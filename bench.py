@@ -200,6 +200,8 @@ def main():
     step_s, launch = eager_s, "one launch per kernel from the host (eager)"
     replays = max(10, args.replays)
     ws = op.workspace
+    if ws is None or ws.numel() < int(plan.workspace_size):  # --ranges asked for more ranges than the operator plans
+        ws = torch.empty(int(plan.workspace_size), dtype=torch.uint8, device=dev.device)
     side = torch.cuda.Stream()
 
     def replay_times(record):

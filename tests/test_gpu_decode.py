@@ -210,11 +210,13 @@ def test_decode_gqa_identical_queries_and_mha_equivalence(pkg, oracle):
         assert np.array_equal(got[:, g], got[:, 0])
 
 
-@pytest.mark.parametrize("heads", [(8, 4), (32, 4), (96, 4), (8, 8), (32, 8), (6, 2), (2, 1), (24, 8), (8, 4, 256), (2, 1, 256)])
+@pytest.mark.parametrize("heads", [(8, 4), (32, 4), (96, 4), (8, 8), (32, 8), (6, 2), (2, 1), (24, 8), (8, 4, 256), (2, 1, 256),
+                                   # one query head per kv head: (heads, kv heads, head_dim, cache_mode)
+                                   (16, 16, 128, 0), (4, 4, 256, 1), (2, 2, 256, 0)])
 def test_decode_with_mask(pkg, oracle, heads):
     bt, dev, q, cache, scale = make_case(pkg, oracle, 79, num_heads=heads[0], num_kv_heads=heads[1],
                                          head_dim=heads[2] if len(heads) > 2 else 128,
-                                         cache_mode=1, dec_kv_lens=[70, 300, 5])
+                                         cache_mode=heads[3] if len(heads) > 3 else 1, dec_kv_lens=[70, 300, 5])
     total = int(bt.kvstarts[-1])
     width = (total + 7) // 8 * 8
     rng = np.random.default_rng(3)
