@@ -138,7 +138,7 @@ typedef enum pmxhip_decode_kernel_t {
     PMXHIP_DECODE_KERNEL_QUAD = 2,    /* head_dim 64 or 128 (even number of kv heads) or 256, up to 4 query heads per
                                          kv head (8 at head_dim 128 with kv heads in eights) */
     PMXHIP_DECODE_KERNEL_MFMA16 = 3,  /* head_dim 128, up to 16 query heads per kv head as MFMA columns */
-    PMXHIP_DECODE_KERNEL_MFMA32 = 4   /* head_dim 128, up to 32 */
+    PMXHIP_DECODE_KERNEL_MFMA32 = 4   /* head_dim 128 or 64, 32 columns; more query heads per kv head in passes of 32 */
 } pmxhip_decode_kernel_t;
 
 typedef struct pmxhip_decode_plan {

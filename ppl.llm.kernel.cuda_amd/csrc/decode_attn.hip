@@ -691,7 +691,7 @@ static int launch_decode_d(const DecodeLaunch& a, int stage, hipStream_t stream)
         switch (a.kernel) {
             case kDecodeKernelMfma16:
             case kDecodeKernelMfma32:
-                if (D != 128) return kLaunchNoKernel;
+                if (D != 128 && !(D == 64 && a.kernel == kDecodeKernelMfma32)) return kLaunchNoKernel;
                 launch_decode_mfma(a, stream);
                 break;
             case kDecodeKernelQuad:

@@ -1,5 +1,5 @@
-// Decode attention over the int8 group-8 KV cache, variant for head_dim 128 and five to thirty-two
-// query heads per kv head (reference: src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/kernel.cu:1090-1891,
+// Decode attention over the int8 group-8 KV cache, variant for five and more query heads per kv head at
+// head_dim 128 or 64 (reference: src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/kernel.cu:1090-1891,
 // the GQCA kernel, which also puts the query heads of a kv head on tensor cores).
 //
 // With that many query heads the per-head arithmetic of the VALU kernels outweighs the cache stream.
@@ -9,8 +9,10 @@
 // so the arithmetic per cache byte no longer grows with the number of query heads; what stays on the
 // VALU is the dequantisation (once per byte) and a softmax over 32 x 32 logits per block.
 //
-// Two variants: up to sixteen query heads per kv head use v_mfma_f32_16x16x32_f16 (half the columns, half the
-// MFMA time, half the logits per lane), seventeen to thirty-two the 32x32x16 form.
+// Two variants: up to sixteen query heads per kv head at head_dim 128 use v_mfma_f32_16x16x32_f16 (half the columns,
+// half the MFMA time, half the logits per lane); the 32x32x16 form serves seventeen and more, and head_dim 64.  More
+// than 32 query heads per kv head (multi-query models: 48 or 71 query heads on one kv head) run as passes of 32
+// columns (blockIdx.z), each of which reads the cache again: the bytes of one kv head are few and stay in the L2.
 //
 // Exactness follows the prefill kernel: K^ = int8 * scale, V^ and p are kept as hi + lo pairs of halves
 // (2 MFMAs per QK step, 3 per PV step), so no fp16 rounding of the dequantised cache enters the result.
@@ -56,10 +58,18 @@ __device__ __forceinline__ int vt_index(int row /* from vt_row */, int pos /* 0.
 
 } // namespace
 
-template <int NW, bool PAGED, bool MASK>
+// D: head_dim 128 or 64 (half the k-steps, channel blocks and V units).  blockIdx.z: which 32 query heads of the
+// kv head's group are this launch's columns (more than 32 query heads per kv head take several passes over the cache).
+template <int NW, bool PAGED, bool MASK, int D>
 __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(const DecodeLaunch a)
 {
-    constexpr int D = kMfmaD;
+    static_assert(D == 128 || D == 64, "head_dim");
+    constexpr int HALF = D / 2; // channels of a token that a half-wave's lanes hold as K bytes
+    constexpr int KW = D / 32;  // 16-byte words of those bytes
+    constexpr int KS = D / 16;  // k-steps of S^T
+    constexpr int CB = D / 32;  // 32-channel blocks of O^T
+    constexpr int GPT = D / 8;  // quantisation groups per token
+    constexpr int VU = D / 64;  // (token quad, group) units of V per lane
     __shared__ __attribute__((aligned(16))) half_t s_vt[NW][2][D * kMfmaBlock]; // [wave][hi, lo]
 
     const int tid = threadIdx.x;
@@ -68,6 +78,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
     const int l32 = lane & 31; // token row (K operand), channel row (V operand) or column (query head)
     const int hh = lane >> 5;
     const int G = (int)a.num_kv_repeats;
+    const int gq = blockIdx.z * kMfmaBlock + l32; // this lane's column: query head gq of the kv head's group
     const int kvh = blockIdx.y * NW + wave;
     half_t* const sV = s_vt[wave][0];
     half_t* const sVlo = s_vt[wave][1];
@@ -89,11 +100,11 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
     const half_t* const scale_v = scale_k + (a.cache_stride_kv >> 3);
     const float sm_scale = a.attn_scale * kLog2e;
 
-    // V units of this lane: (token quad, channel group) pairs idx = lane + 64 u, group = idx % 16, quad = idx / 16
-    const int v_g = lane & 15;
-    int v_q[2];
-    v_q[0] = lane >> 4;
-    v_q[1] = 4 + (lane >> 4);
+    // V units of this lane: (token quad, channel group) pairs idx = lane + 64 u, group = idx % GPT, quad = idx / GPT
+    const int v_g = lane % GPT;
+    int v_q[VU];
+#pragma unroll
+    for (int u = 0; u < VU; ++u) v_q[u] = (lane + 64 * u) / GPT;
 
     int b = find_sequence(kvstarts, a.kvstarts, (int)a.decoding_batches, r0, lane);
     for (; b < a.decoding_batches; ++b) {
@@ -116,13 +127,13 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
         };
 
         // ---- Q fragments (B operand of S^T): column = query head l32; k-step s of half-wave hh covers the
-        // channels [64 hh + 16 (s / 2) + 8 (s % 2), + 8), so that a lane's K bytes are 64 consecutive ones ----
-        f16x8 qf[8];
+        // channels [HALF hh + 16 (s / 2) + 8 (s % 2), + 8), so that a lane's K bytes are HALF consecutive ones ----
+        f16x8 qf[KS];
         {
-            const bool on = l32 < G;
-            const half_t* qp = (const half_t*)a.query + (int64_t)b * a.query_stride_s + (int64_t)(kvh * G + (on ? l32 : 0)) * D + 64 * hh;
+            const bool on = gq < G;
+            const half_t* qp = (const half_t*)a.query + (int64_t)b * a.query_stride_s + (int64_t)(kvh * G + (on ? gq : 0)) * D + HALF * hh;
 #pragma unroll
-            for (int s = 0; s < 8; ++s) {
+            for (int s = 0; s < KS; ++s) {
                 qf[s] = *(const f16x8*)(qp + 8 * s);
                 if (!on) {
 #pragma unroll
@@ -132,28 +143,28 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
         }
         const half_t* mask_row = nullptr;
         if (MASK) {
-            const int h = kvh * G + (l32 < G ? l32 : 0);
+            const int h = kvh * G + (gq < G ? gq : 0);
             mask_row = (const half_t*)a.attn_mask + (int64_t)h * a.mask_stride_h + (int64_t)b * a.mask_stride_s + kvstarts[b];
         }
 
-        // ---- raw bytes of one block: K as (token l32, channels 64 hh .. + 64), V as two (token quad, group) units ----
-        u32x4 kq[4];
-        uint32_t ksc[4]; // eight half scales
-        u32x2 vq[2][4];
-        half_t vsc[2][4];
+        // ---- raw bytes of one block: K as (token l32, channels HALF hh .. + HALF), V as (token quad, group) units ----
+        u32x4 kq[KW];
+        uint32_t ksc[KW]; // two half scales each
+        u32x2 vq[VU][4];
+        half_t vsc[VU][4];
         // per-lane offsets inside a block: constant except in a piece's last block, whose tokens beyond the
         // piece re-read its last token (their logits are masked)
-        uint32_t k_off = (uint32_t)l32 * stride_s32 + 64 * hh;
-        uint32_t v_off[2][4];
+        uint32_t k_off = (uint32_t)l32 * stride_s32 + HALF * hh;
+        uint32_t v_off[VU][4];
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+        for (int u = 0; u < VU; ++u)
 #pragma unroll
             for (int r = 0; r < 4; ++r) v_off[u][r] = (uint32_t)(4 * v_q[u] + r) * stride_s32 + 8 * v_g;
         auto clamp_offsets = [&](int pos) {
             const int last = pe32 - 1 - pos; // offset of the piece's last token inside this block (>= 0)
-            k_off = (uint32_t)(l32 < last ? l32 : last) * stride_s32 + 64 * hh;
+            k_off = (uint32_t)(l32 < last ? l32 : last) * stride_s32 + HALF * hh;
 #pragma unroll
-            for (int u = 0; u < 2; ++u)
+            for (int u = 0; u < VU; ++u)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int t = 4 * v_q[u] + r;
@@ -165,7 +176,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
             const char* bk = cache_k + boff;
             const half_t* sk = scale_k + (boff >> 3);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < KW; ++j) {
                 kq[j] = *(const u32x4*)(bk + k_off + 16 * j);
                 ksc[j] = *(const uint32_t*)(sk + (k_off >> 3) + 2 * j);
             }
@@ -175,7 +186,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
             const char* bv = cache_v + boff;
             const half_t* sv = scale_v + (boff >> 3);
 #pragma unroll
-            for (int u = 0; u < 2; ++u)
+            for (int u = 0; u < VU; ++u)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     vq[u][r] = *(const u32x2*)(bv + v_off[u][r]);
@@ -183,9 +194,9 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
                 }
         };
 
-        f32x16 o_acc[4];
+        f32x16 o_acc[CB];
 #pragma unroll
-        for (int cb = 0; cb < 4; ++cb)
+        for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) o_acc[cb][i] = 0.f;
         float m_run = kNegBig, l_run = 0.f;
@@ -199,7 +210,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
             // ---- V: dequantise (hi + lo halves) and store transposed into the wave's LDS tile ----
             wave_lds_handoff(); // every lane is past its reads of the previous block's tile
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
+            for (int u = 0; u < VU; ++u) {
                 const half2_t s01 = {vsc[u][0], vsc[u][1]}, s23 = {vsc[u][2], vsc[u][3]};
                 const int posv = 16 * (v_q[u] >> 2) + vt_pos16(4 * (v_q[u] & 3));
 #pragma unroll
@@ -233,7 +244,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
 #pragma unroll
             for (int e = 0; e < 16; ++e) s_acc[e] = 0.f;
 #pragma unroll
-            for (int s = 0; s < 8; ++s) {
+            for (int s = 0; s < KS; ++s) {
                 const int j = s >> 1, e = s & 1;
                 const half_t sc1 = bitcast<half2_t>(ksc[j])[e];
                 const half2_t sc = {sc1, sc1};
@@ -276,7 +287,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
                 const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
                 l_run *= alpha;
 #pragma unroll
-                for (int cb = 0; cb < 4; ++cb)
+                for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) o_acc[cb][e] *= alpha;
                 m_run = m_new;
@@ -302,7 +313,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int cb = 0; cb < 4; ++cb) {
+                for (int cb = 0; cb < CB; ++cb) {
                     const int idx = vt_index(vt_row(32 * cb + l32), 16 * t + 8 * hh);
                     const f16x8 vh = *(const f16x8*)&sV[idx];
                     const f16x8 vl = *(const f16x8*)&sVlo[idx];
@@ -315,13 +326,13 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
         // ---- end of the piece: element e of block cb <-> channel 32 cb + 8 (e / 4) + 4 hh + e % 4 ----
         const float l_tot = l_run + __shfl_xor(l_run, 32);
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-        if (l32 < G) {
-            const int h = kvh * G + l32;
+        if (gq < G) {
+            const int h = kvh * G + gq;
             const bool whole = (pa == 0) && (pe == len);
             if (whole) {
                 half_t* op = (half_t*)a.output + (int64_t)b * a.output_stride_s + (int64_t)h * D;
 #pragma unroll
-                for (int cb = 0; cb < 4; ++cb)
+                for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         f16x4 w;
@@ -333,7 +344,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
                 const int64_t piece = (int64_t)blockIdx.x + b;
                 float* op = a.partial_out + (piece * a.num_heads + h) * D;
 #pragma unroll
-                for (int cb = 0; cb < 4; ++cb)
+                for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
                         *(f32x4*)(op + 32 * cb + 8 * r + 4 * hh) =
@@ -700,6 +711,19 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
     }
 }
 
+template <int NW, int D>
+static void launch_decode_mfma32(const DecodeLaunch& a, dim3 grid, dim3 block, hipStream_t stream)
+{
+    const bool paged = a.cache_mode == 1, mask = a.attn_mask != nullptr;
+    if (paged) {
+        if (mask) hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, true, true, D>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, true, false, D>), grid, block, 0, stream, a);
+    } else {
+        if (mask) hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, false, true, D>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, false, false, D>), grid, block, 0, stream, a);
+    }
+}
+
 template <int NW>
 static void launch_decode_mfma_nw(const DecodeLaunch& a, hipStream_t stream)
 {
@@ -716,13 +740,10 @@ static void launch_decode_mfma_nw(const DecodeLaunch& a, hipStream_t stream)
         }
         return;
     }
-    if (paged) {
-        if (mask) hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, true, true>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, true, false>), grid, block, 0, stream, a);
-    } else {
-        if (mask) hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, false, true>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, false, false>), grid, block, 0, stream, a);
-    }
+    // the 32-column form: head_dim 128 or 64, and as many passes as the query heads of a kv head need
+    const dim3 grid32((unsigned)a.ranges, (unsigned)(a.num_kv_heads / NW), (unsigned)a.num_passes);
+    if (a.head_dim == 64) launch_decode_mfma32<NW, 64>(a, grid32, block, stream);
+    else launch_decode_mfma32<NW, 128>(a, grid32, block, stream);
 }
 
 void launch_decode_mfma(const DecodeLaunch& a, hipStream_t stream)

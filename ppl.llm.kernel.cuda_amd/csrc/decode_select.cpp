@@ -45,11 +45,14 @@ bool decode_choose(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, in
     if (kernel == kDecodeKernelAuto) {
         // Many query heads per kv head: their VALU arithmetic outweighs the cache stream, so they become MFMA
         // columns (five and more; three and four as well where the kv heads do not come in pairs, which the quad
-        // kernel needs).  Up to four: the quad kernel, whose row loads stream whole lines.  Everything else
-        // (head_dim 96, head_dim 64 with more than four query heads per kv head, odd kv-head counts with one or two
-        // query heads each, more than 32 query heads per kv head) stays on the general kernel.
-        if (head_dim == 128 && g <= kDecodeMfmaColumns && (g >= 5 || (g >= 3 && num_kv_heads % 2 != 0)))
+        // kernel needs): 16 or 32 columns at head_dim 128, 32 at head_dim 64, and beyond 32 query heads per kv head
+        // (multi-query models) as many passes of 32 columns as they need.  Up to four: the quad kernel, whose row
+        // loads stream whole lines.  Everything else (head_dim 96, odd kv-head counts with one or two query heads
+        // each, head_dim 256 with more than four) stays on the general kernel.
+        if (head_dim == 128 && (g >= 5 || (g >= 3 && num_kv_heads % 2 != 0)))
             kernel = g <= kDecodeMfma16Columns ? kDecodeKernelMfma16 : kDecodeKernelMfma32;
+        else if (head_dim == 64 && (g >= 5 || (g >= 3 && num_kv_heads % 2 != 0)))
+            kernel = kDecodeKernelMfma32;
         else if (quad_serves(head_dim, g, num_kv_heads) && g <= 4)
             kernel = kDecodeKernelQuad;
         else
@@ -85,10 +88,11 @@ bool decode_choose(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, in
         case kDecodeKernelMfma16:
         case kDecodeKernelMfma32: {
             const int cols = kernel == kDecodeKernelMfma16 ? kDecodeMfma16Columns : kDecodeMfmaColumns;
-            if (head_dim != 128 || g > cols) return false;
+            // the 16-column form: head_dim 128, one pass; the 32-column form: head_dim 128 or 64, any number of passes
+            if (kernel == kDecodeKernelMfma16 ? (head_dim != 128 || g > cols) : (head_dim != 128 && head_dim != 64)) return false;
             c.kv_heads_per_group = num_kv_heads % 4 == 0 ? 4 : (num_kv_heads % 2 == 0 ? 2 : 1); // a wave per kv head
             c.q_heads_per_pass = cols;
-            c.num_passes = 1;
+            c.num_passes = (int32_t)((g + cols - 1) / cols);
             c.wg_tokens = kDecodeMfmaTokens;
             c.wgs_per_cu = kDecodeMfmaWavesPerCu / c.kv_heads_per_group;
             break;

@@ -46,6 +46,9 @@ SHAPES = [
     (16, 8, 256), (16, 16, 256), (3, 1, 256), (8, 2, 256), (5, 1, 256),
     # ... and with head_dim 64 (blocks of 32 tokens: the rows of a half-wave are two token groups)
     (32, 8, 64), (8, 4, 64), (6, 2, 64), (16, 16, 64), (18, 6, 64),
+    # the 32-column MFMA kernel at head_dim 64, and with more than 32 query heads per kv head (passes of 32 columns:
+    # multi-query models)
+    (128, 8, 64), (14, 2, 64), (9, 3, 64), (71, 1, 64), (66, 2, 64), (48, 1, 128), (40, 1, 128), (132, 4, 128),
 ]
 
 
@@ -74,8 +77,10 @@ KERNEL_NAMES = {1: "decode_attention_kernel", 2: "decode_attention_quad_kernel",
     ((96, 4, 128), (1, 4)),         # 24 per kv head: three passes of the general kernel, or 32 columns
     ((16, 8, 256), (1, 2)),
     ((6, 3, 128), (1, 3)),
-    ((32, 8, 64), (1, 2)),
+    ((32, 8, 64), (1, 2, 4)),
     ((4, 4, 64), (1, 2)),
+    ((48, 1, 128), (1, 4)),         # multi-query: six passes of the general kernel, or two of 32 columns
+    ((71, 1, 64), (1, 4)),
 ])
 def test_decode_requested_kernel(pkg, oracle, shape, kernels):
     """Every token-range kernel that serves a shape, requested through the C ABI: the library reports that it
@@ -212,7 +217,9 @@ def test_decode_gqa_identical_queries_and_mha_equivalence(pkg, oracle):
 
 @pytest.mark.parametrize("heads", [(8, 4), (32, 4), (96, 4), (8, 8), (32, 8), (6, 2), (2, 1), (24, 8), (8, 4, 256), (2, 1, 256),
                                    # one query head per kv head: (heads, kv heads, head_dim, cache_mode)
-                                   (16, 16, 128, 0), (4, 4, 256, 1), (2, 2, 256, 0)])
+                                   (16, 16, 128, 0), (4, 4, 256, 1), (2, 2, 256, 0),
+                                   # passes of 32 columns, and head_dim 64 on the 32-column kernel
+                                   (48, 1, 128, 1), (14, 2, 64, 1), (71, 1, 64, 0)])
 def test_decode_with_mask(pkg, oracle, heads):
     bt, dev, q, cache, scale = make_case(pkg, oracle, 79, num_heads=heads[0], num_kv_heads=heads[1],
                                          head_dim=heads[2] if len(heads) > 2 else 128,

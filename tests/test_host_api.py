@@ -137,7 +137,9 @@ def test_decode_plan(pkg, hip_lib):
     assert plan.q_heads_per_pass == 16 and plan.kv_heads_per_group == 2 and plan.num_token_ranges == 1024
     plan = pkg.ops.decode_plan(64, 16, 4, 128, 8192, cus=256)  # four kv heads: two waves per workgroup, four workgroups per CU
     assert plan.q_heads_per_pass == 4 and plan.kv_heads_per_group == 4 and plan.num_token_ranges == 1024
-    plan = pkg.ops.decode_plan(4, 48, 3, 64, 512, cus=256)  # G = 16 -> two passes of 8; 3 kv heads -> 1 per group
+    plan = pkg.ops.decode_plan(4, 48, 3, 64, 512, cus=256)  # G = 16 at head_dim 64: 32 MFMA columns; 3 kv heads -> 1 per group
+    assert plan.q_heads_per_pass == 32 and plan.num_passes == 1 and plan.kv_heads_per_group == 1
+    plan = pkg.ops.decode_plan(4, 48, 3, 64, 512, cus=256, kernel=pkg._lib.DECODE_KERNEL_GENERAL)  # -> two passes of 8
     assert plan.q_heads_per_pass == 8 and plan.num_passes == 2 and plan.kv_heads_per_group == 1
     plan = pkg.ops.decode_plan(1, 8, 8, 64, 100, cus=256)   # tiny: one range, no workspace
     assert plan.num_token_ranges == 1 and plan.workspace_size == 0
@@ -154,18 +156,23 @@ def test_decode_plan_names_its_kernel(pkg, hip_lib):
     L = pkg._lib
     auto = {(32, 8, 128): L.DECODE_KERNEL_QUAD, (32, 32, 128): L.DECODE_KERNEL_QUAD, (64, 8, 128): L.DECODE_KERNEL_MFMA16,
             (96, 4, 128): L.DECODE_KERNEL_MFMA32, (9, 3, 128): L.DECODE_KERNEL_MFMA16, (6, 3, 128): L.DECODE_KERNEL_GENERAL,
-            (8, 8, 64): L.DECODE_KERNEL_QUAD, (32, 8, 64): L.DECODE_KERNEL_QUAD, (40, 8, 64): L.DECODE_KERNEL_GENERAL,
-            (9, 3, 64): L.DECODE_KERNEL_GENERAL, (12, 4, 96): L.DECODE_KERNEL_GENERAL, (16, 16, 256): L.DECODE_KERNEL_QUAD,
-            (40, 8, 256): L.DECODE_KERNEL_GENERAL, (66, 2, 128): L.DECODE_KERNEL_GENERAL}
+            (8, 8, 64): L.DECODE_KERNEL_QUAD, (32, 8, 64): L.DECODE_KERNEL_QUAD, (40, 8, 64): L.DECODE_KERNEL_MFMA32,
+            (9, 3, 64): L.DECODE_KERNEL_MFMA32, (12, 4, 96): L.DECODE_KERNEL_GENERAL, (16, 16, 256): L.DECODE_KERNEL_QUAD,
+            (40, 8, 256): L.DECODE_KERNEL_GENERAL, (66, 2, 128): L.DECODE_KERNEL_MFMA32, (48, 1, 128): L.DECODE_KERNEL_MFMA32,
+            (71, 1, 64): L.DECODE_KERNEL_MFMA32, (2, 1, 64): L.DECODE_KERNEL_GENERAL}
     for (hq, hkv, d), want in auto.items():
         assert pkg.ops.decode_plan(16, hq, hkv, d, 4096, cus=256).kernel == want, (hq, hkv, d)
+    # more than 32 query heads per kv head: passes of 32 columns (multi-query models)
+    for (hq, hkv, d), passes in {(48, 1, 128): 2, (71, 1, 64): 3, (66, 2, 128): 2, (128, 4, 128): 1, (128, 8, 64): 1}.items():
+        plan = pkg.ops.decode_plan(16, hq, hkv, d, 4096, cus=256)
+        assert (plan.kernel, plan.q_heads_per_pass, plan.num_passes) == (L.DECODE_KERNEL_MFMA32, 32, passes), (hq, hkv, d)
     # requests: every kernel on the Llama-3-70B shape (8 query heads per kv head, kv heads in eights)
     for k, (kvhb, gt, ranges) in {L.DECODE_KERNEL_GENERAL: (8, 8, 512), L.DECODE_KERNEL_QUAD: (8, 8, 512),
                                   L.DECODE_KERNEL_MFMA16: (4, 16, 256), L.DECODE_KERNEL_MFMA32: (4, 32, 256)}.items():
         plan = pkg.ops.decode_plan(32, 64, 8, 128, 32768, cus=256, kernel=k)
         assert (plan.kernel, plan.kv_heads_per_group, plan.q_heads_per_pass, plan.num_token_ranges) == (k, kvhb, gt, ranges)
     for hq, hkv, d, k in [(40, 8, 64, L.DECODE_KERNEL_QUAD), (32, 8, 96, L.DECODE_KERNEL_QUAD), (32, 8, 64, L.DECODE_KERNEL_MFMA16),
-                          (40, 2, 128, L.DECODE_KERNEL_MFMA16), (66, 2, 128, L.DECODE_KERNEL_MFMA32),
+                          (40, 2, 128, L.DECODE_KERNEL_MFMA16), (32, 8, 96, L.DECODE_KERNEL_MFMA32), (16, 4, 256, L.DECODE_KERNEL_MFMA32),
                           (10, 2, 128, L.DECODE_KERNEL_QUAD), (3, 3, 128, L.DECODE_KERNEL_QUAD), (32, 8, 128, 5), (32, 8, 128, -1)]:
         with pytest.raises(pkg.ops.PmxError):
             pkg.ops.decode_plan(16, hq, hkv, d, 4096, cus=256, kernel=k)
