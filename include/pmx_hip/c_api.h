@@ -135,8 +135,8 @@ typedef struct pmxhip_decode_params {
 typedef enum pmxhip_decode_kernel_t {
     PMXHIP_DECODE_KERNEL_AUTO = 0,
     PMXHIP_DECODE_KERNEL_GENERAL = 1, /* VALU; every head_dim and head count */
-    PMXHIP_DECODE_KERNEL_QUAD = 2,    /* head_dim 64 or 128 (even number of kv heads) or 256, up to 4 query heads per
-                                         kv head (8 at head_dim 128 with kv heads in eights) */
+    PMXHIP_DECODE_KERNEL_QUAD = 2,    /* head_dim 64 or 128 (two or more kv heads) or 256, up to 4 query heads per
+                                         kv head (8 at head_dim 256, and at head_dim 128 with kv heads in eights) */
     PMXHIP_DECODE_KERNEL_MFMA16 = 3,  /* head_dim 128, up to 16 query heads per kv head as MFMA columns */
     PMXHIP_DECODE_KERNEL_MFMA32 = 4   /* head_dim 128 or 64, 32 columns; more query heads per kv head in passes of 32 */
 } pmxhip_decode_kernel_t;

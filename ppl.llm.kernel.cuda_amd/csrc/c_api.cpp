@@ -236,7 +236,7 @@ int pmxhip_decode_plan_make_kernel(int64_t decoding_batches, int64_t num_heads, 
 
     int64_t ranges = num_token_ranges_hint;
     if (ranges == 0) {
-        const int64_t groups = (num_kv_heads / c.kv_heads_per_group) * c.num_passes;
+        const int64_t groups = ((num_kv_heads + c.kv_heads_per_group - 1) / c.kv_heads_per_group) * c.num_passes;
         int cus = compute_units > 0 ? compute_units : current_compute_units();
         if (cus <= 0) return fail(PMXHIP_INVALID_VALUE, "decode_plan: compute_units not given and no current device");
         // as many ranges as fill the workgroup slots of the chip: two workgroups of four waves per CU, or as many as

@@ -129,7 +129,12 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
     const int row_odd = (lane >> 4) & 1; // head_dim 64: the token group, tokens 16 row_odd + 4 j + t4 of a block
     const int tok0 = t4 + (H64 ? 16 * row_odd : 0); // this lane's token of step 0
     const int G = (int)a.num_kv_repeats; // <= 4 * GP
-    const int kvh = blockIdx.y * (KPW * WP) + wave * KPW + (KPW == 2 ? hsel : 0);
+    // An odd number of kv heads leaves the last half-wave of the last workgroup without one: it repeats its
+    // neighbour's work (the same addresses, so no further memory traffic) and stores nothing.
+    const int slot_raw = wave * KPW + (KPW == 2 ? hsel : 0); // kv head within the workgroup
+    const bool head_on = blockIdx.y * (KPW * WP) + slot_raw < (int)a.num_kv_heads;
+    const int head_slot = head_on ? slot_raw : slot_raw - 1;
+    const int kvh = blockIdx.y * (KPW * WP) + head_slot;
     const int ch0 = chunk * 16 + (KPW == 1 ? hsel * 128 : 0); // this lane's 16 channels
 
     const const_i64_ptr kvstarts = as_constant(a.kvstarts);
@@ -143,7 +148,7 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
 
     const int64_t group_off = a.layer_idx * a.cache_stride_l + (int64_t)(blockIdx.y * (KPW * WP)) * a.cache_stride_h;
     const uint32_t stride_s32 = (uint32_t)a.cache_stride_s; // the host checks that a block's span fits 32 bits
-    const uint32_t lane_base = (uint32_t)((int64_t)(wave * KPW + (KPW == 2 ? hsel : 0)) * a.cache_stride_h + ch0);
+    const uint32_t lane_base = (uint32_t)((int64_t)head_slot * a.cache_stride_h + ch0);
     const char* const cache_k = (const char*)a.cache + group_off;
     const char* const cache_v = cache_k + a.cache_stride_kv;
     const char* const scale_k = (const char*)a.scale + (group_off >> 3) * 2;
@@ -578,7 +583,7 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
                 o[c] = across_rows_sum(v) * inv;
             }
             const int g = ONE ? 0 : g_first + (g_own ^ s);
-            if (t4 == 0 && (!H64 || row_odd == 0) && g < G) {
+            if (t4 == 0 && (!H64 || row_odd == 0) && g < G && head_on) {
                 const int h = kvh * G + g;
                 if (whole) {
                     typedef half_t half8_t __attribute__((ext_vector_type(8)));
@@ -612,7 +617,7 @@ template <int WP, int HD>
 static void launch_decode_quad_wp(const DecodeLaunch& a, hipStream_t stream)
 {
     constexpr int KPW = HD == 256 ? 1 : 2;
-    const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / (KPW * WP)), 1);
+    const dim3 grid((unsigned)a.ranges, (unsigned)((a.num_kv_heads + KPW * WP - 1) / (KPW * WP)), 1);
     const bool paged = a.cache_mode == 1, mask = a.attn_mask != nullptr;
     const bool one = a.num_kv_repeats == 1; // MHA: a single head slot per lane
     if (paged) {
@@ -626,17 +631,32 @@ static void launch_decode_quad_wp(const DecodeLaunch& a, hipStream_t stream)
     }
 }
 
+template <int WP, int HD>
+static void launch_decode_quad_two_sets(const DecodeLaunch& a, hipStream_t stream)
+{
+    constexpr int KPW = HD == 256 ? 1 : 2;
+    const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / (KPW * WP)), 1);
+    if (a.cache_mode == 1) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 2, WP, false, HD>), grid, dim3(2 * WP * kWave), 0, stream, a);
+    else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 2, WP, false, HD>), grid, dim3(2 * WP * kWave), 0, stream, a);
+}
+
 void launch_decode_quad(const DecodeLaunch& a, hipStream_t stream)
 {
-    if (a.num_kv_repeats > 4) { // two sets of four waves on eight kv heads
-        const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / kQuadMaxHeads), 1);
-        if (a.cache_mode == 1) hipLaunchKernelGGL((decode_attention_quad_kernel<true, 2, 4, false, 128>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
-        else hipLaunchKernelGGL((decode_attention_quad_kernel<false, 2, 4, false, 128>), grid, dim3(2 * kDecodeThreads), 0, stream, a);
+    const int waves = a.kv_heads_per_group / (a.head_dim == 256 ? 1 : 2);
+    if (a.num_kv_repeats > 4) { // two sets of waves: the second takes query heads 4-7 of the same kv heads
+        if (a.head_dim == 256) { // a wave per kv head
+            switch (waves) {
+            case 4: launch_decode_quad_two_sets<4, 256>(a, stream); break;
+            case 2: launch_decode_quad_two_sets<2, 256>(a, stream); break;
+            default: launch_decode_quad_two_sets<1, 256>(a, stream); break;
+            }
+        } else {
+            launch_decode_quad_two_sets<4, 128>(a, stream); // eight kv heads
+        }
         return;
     }
-    const int waves = a.kv_heads_per_group / (a.head_dim == 256 ? 1 : 2);
     if (a.head_dim == 64) { // no mask form: decode_quad_launch_ok sends masked steps to the general kernel
-        const dim3 grid((unsigned)a.ranges, (unsigned)(a.num_kv_heads / (2 * waves)), 1);
+        const dim3 grid((unsigned)a.ranges, (unsigned)((a.num_kv_heads + 2 * waves - 1) / (2 * waves)), 1);
         const bool paged = a.cache_mode == 1;
         switch (waves) {
         case 4:

@@ -14,12 +14,13 @@ int largest_pow2_divisor_upto(int64_t n, int cap)
     return r;
 }
 
-// head_dim 64 or 128 with an even number of kv heads, or head_dim 256: up to four query heads per kv head on one set
-// of waves; head_dim 128 with kv heads in eights: up to eight on two sets
+// head_dim 64, 128 or 256: up to four query heads per kv head on one set of waves; head_dim 256, and head_dim 128
+// with kv heads in eights: up to eight on two sets.  At head_dim 64 and 128 a wave holds two kv heads: an odd number of them leaves
+// the last half-wave idle, which a single kv head does not pay for (half of every wave).
 bool quad_serves(int64_t head_dim, int64_t g, int64_t num_kv_heads)
 {
-    if (head_dim == 256) return g <= 4;
-    if ((head_dim != 128 && head_dim != 64) || num_kv_heads % 2 != 0) return false;
+    if (head_dim == 256) return g <= 8;
+    if ((head_dim != 128 && head_dim != 64) || num_kv_heads == 1) return false;
     return g <= 4 || (head_dim == 128 && g <= 8 && num_kv_heads % 8 == 0);
 }
 
@@ -44,16 +45,17 @@ bool decode_choose(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, in
     int32_t kernel = requested;
     if (kernel == kDecodeKernelAuto) {
         // Many query heads per kv head: their VALU arithmetic outweighs the cache stream, so they become MFMA
-        // columns (five and more; three and four as well where the kv heads do not come in pairs, which the quad
-        // kernel needs): 16 or 32 columns at head_dim 128, 32 at head_dim 64, and beyond 32 query heads per kv head
+        // columns (five and more; three and four as well on a single kv head, which would use half of the quad
+        // kernel's lanes): 16 or 32 columns at head_dim 128, 32 at head_dim 64, and beyond 32 query heads per kv head
         // (multi-query models) as many passes of 32 columns as they need.  Up to four: the quad kernel, whose row
-        // loads stream whole lines.  Everything else (head_dim 96, odd kv-head counts with one or two query heads
-        // each, head_dim 256 with more than four) stays on the general kernel.
-        if (head_dim == 128 && (g >= 5 || (g >= 3 && num_kv_heads % 2 != 0)))
+        // loads stream whole lines (head_dim 256: up to eight, on two sets of waves).  Everything else (head_dim 96,
+        // a single kv head with one or two query heads, head_dim 256 with more than eight per kv head) stays on
+        // the general kernel.
+        if (head_dim == 128 && (g >= 5 || (g >= 3 && num_kv_heads == 1)))
             kernel = g <= kDecodeMfma16Columns ? kDecodeKernelMfma16 : kDecodeKernelMfma32;
-        else if (head_dim == 64 && (g >= 5 || (g >= 3 && num_kv_heads % 2 != 0)))
+        else if (head_dim == 64 && (g >= 5 || (g >= 3 && num_kv_heads == 1)))
             kernel = kDecodeKernelMfma32;
-        else if (quad_serves(head_dim, g, num_kv_heads) && g <= 4)
+        else if (quad_serves(head_dim, g, num_kv_heads) && (g <= 4 || head_dim == 256))
             kernel = kDecodeKernelQuad;
         else
             kernel = kDecodeKernelGeneral;
@@ -77,12 +79,13 @@ bool decode_choose(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, in
             if (!quad_serves(head_dim, g, num_kv_heads)) return false;
             // a wave holds two kv heads of 128 channels or one of 256; four, two or one waves per set
             const int per_wave = head_dim == 256 ? 1 : 2;
-            const int64_t pairs = num_kv_heads / per_wave;
+            const int64_t pairs = (num_kv_heads + per_wave - 1) / per_wave;
             c.kv_heads_per_group = per_wave * (pairs % 4 == 0 ? 4 : (pairs % 2 == 0 ? 2 : 1));
             c.q_heads_per_pass = g <= 1 ? 1 : (g <= 2 ? 2 : (g <= 4 ? 4 : 8)); // rows of the 4x4x4 products in use
             c.num_passes = 1;
             c.wg_tokens = head_dim == 64 ? 2 * kDecodeQuadTokens : kDecodeQuadTokens; // head_dim 64: blocks of 32 tokens
             c.wgs_per_cu = (head_dim == 256 ? 8 : 16) / c.kv_heads_per_group;
+            if (head_dim == 256 && g > 4) c.wgs_per_cu = c.wgs_per_cu > 1 ? c.wgs_per_cu / 2 : 1; // twice the waves per workgroup
             break;
         }
         case kDecodeKernelMfma16:

@@ -48,7 +48,11 @@ SHAPES = [
     (32, 8, 64), (8, 4, 64), (6, 2, 64), (16, 16, 64), (18, 6, 64),
     # the 32-column MFMA kernel at head_dim 64, and with more than 32 query heads per kv head (passes of 32 columns:
     # multi-query models)
-    (128, 8, 64), (14, 2, 64), (9, 3, 64), (71, 1, 64), (66, 2, 64), (48, 1, 128), (40, 1, 128), (132, 4, 128),
+    (128, 8, 64), (14, 2, 64), (3, 1, 64), (71, 1, 64), (66, 2, 64), (48, 1, 128), (40, 1, 128), (132, 4, 128),
+    # the quad kernel with an odd number of kv heads (the last half-wave has none)
+    (5, 5, 128), (9, 3, 128), (14, 7, 128), (9, 9, 64), (12, 3, 64), (36, 9, 128),
+    # head_dim 256 with five to eight query heads per kv head: two sets of waves
+    (8, 1, 256), (32, 4, 256), (12, 2, 256), (40, 8, 256), (21, 3, 256),
 ]
 
 
@@ -76,7 +80,9 @@ KERNEL_NAMES = {1: "decode_attention_kernel", 2: "decode_attention_quad_kernel",
     ((12, 2, 128), (1, 3, 4)),
     ((96, 4, 128), (1, 4)),         # 24 per kv head: three passes of the general kernel, or 32 columns
     ((16, 8, 256), (1, 2)),
-    ((6, 3, 128), (1, 3)),
+    ((6, 3, 128), (1, 2, 3)),
+    ((5, 5, 128), (1, 2)),
+    ((8, 1, 256), (1, 2)),
     ((32, 8, 64), (1, 2, 4)),
     ((4, 4, 64), (1, 2)),
     ((48, 1, 128), (1, 4)),         # multi-query: six passes of the general kernel, or two of 32 columns
@@ -219,7 +225,9 @@ def test_decode_gqa_identical_queries_and_mha_equivalence(pkg, oracle):
                                    # one query head per kv head: (heads, kv heads, head_dim, cache_mode)
                                    (16, 16, 128, 0), (4, 4, 256, 1), (2, 2, 256, 0),
                                    # passes of 32 columns, and head_dim 64 on the 32-column kernel
-                                   (48, 1, 128, 1), (14, 2, 64, 1), (71, 1, 64, 0)])
+                                   (48, 1, 128, 1), (14, 2, 64, 1), (71, 1, 64, 0),
+                                   # an odd number of kv heads on the quad kernel
+                                   (5, 5, 128, 1), (12, 3, 128, 0)])
 def test_decode_with_mask(pkg, oracle, heads):
     bt, dev, q, cache, scale = make_case(pkg, oracle, 79, num_heads=heads[0], num_kv_heads=heads[1],
                                          head_dim=heads[2] if len(heads) > 2 else 128,

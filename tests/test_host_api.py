@@ -155,10 +155,11 @@ def test_decode_plan_names_its_kernel(pkg, hip_lib):
     """The plan reports the token-range kernel it was made for, and a requested kernel is honoured or refused."""
     L = pkg._lib
     auto = {(32, 8, 128): L.DECODE_KERNEL_QUAD, (32, 32, 128): L.DECODE_KERNEL_QUAD, (64, 8, 128): L.DECODE_KERNEL_MFMA16,
-            (96, 4, 128): L.DECODE_KERNEL_MFMA32, (9, 3, 128): L.DECODE_KERNEL_MFMA16, (6, 3, 128): L.DECODE_KERNEL_GENERAL,
+            (96, 4, 128): L.DECODE_KERNEL_MFMA32, (9, 3, 128): L.DECODE_KERNEL_QUAD, (6, 3, 128): L.DECODE_KERNEL_QUAD, (3, 1, 128): L.DECODE_KERNEL_MFMA16,
+            (5, 5, 128): L.DECODE_KERNEL_QUAD, (2, 1, 128): L.DECODE_KERNEL_GENERAL, (3, 1, 64): L.DECODE_KERNEL_MFMA32,
             (8, 8, 64): L.DECODE_KERNEL_QUAD, (32, 8, 64): L.DECODE_KERNEL_QUAD, (40, 8, 64): L.DECODE_KERNEL_MFMA32,
-            (9, 3, 64): L.DECODE_KERNEL_MFMA32, (12, 4, 96): L.DECODE_KERNEL_GENERAL, (16, 16, 256): L.DECODE_KERNEL_QUAD,
-            (40, 8, 256): L.DECODE_KERNEL_GENERAL, (66, 2, 128): L.DECODE_KERNEL_MFMA32, (48, 1, 128): L.DECODE_KERNEL_MFMA32,
+            (9, 3, 64): L.DECODE_KERNEL_QUAD, (12, 4, 96): L.DECODE_KERNEL_GENERAL, (16, 16, 256): L.DECODE_KERNEL_QUAD,
+            (40, 8, 256): L.DECODE_KERNEL_QUAD, (8, 1, 256): L.DECODE_KERNEL_QUAD, (72, 8, 256): L.DECODE_KERNEL_GENERAL, (66, 2, 128): L.DECODE_KERNEL_MFMA32, (48, 1, 128): L.DECODE_KERNEL_MFMA32,
             (71, 1, 64): L.DECODE_KERNEL_MFMA32, (2, 1, 64): L.DECODE_KERNEL_GENERAL}
     for (hq, hkv, d), want in auto.items():
         assert pkg.ops.decode_plan(16, hq, hkv, d, 4096, cus=256).kernel == want, (hq, hkv, d)
@@ -173,7 +174,7 @@ def test_decode_plan_names_its_kernel(pkg, hip_lib):
         assert (plan.kernel, plan.kv_heads_per_group, plan.q_heads_per_pass, plan.num_token_ranges) == (k, kvhb, gt, ranges)
     for hq, hkv, d, k in [(40, 8, 64, L.DECODE_KERNEL_QUAD), (32, 8, 96, L.DECODE_KERNEL_QUAD), (32, 8, 64, L.DECODE_KERNEL_MFMA16),
                           (40, 2, 128, L.DECODE_KERNEL_MFMA16), (32, 8, 96, L.DECODE_KERNEL_MFMA32), (16, 4, 256, L.DECODE_KERNEL_MFMA32),
-                          (10, 2, 128, L.DECODE_KERNEL_QUAD), (3, 3, 128, L.DECODE_KERNEL_QUAD), (32, 8, 128, 5), (32, 8, 128, -1)]:
+                          (10, 2, 128, L.DECODE_KERNEL_QUAD), (2, 1, 128, L.DECODE_KERNEL_QUAD), (32, 8, 128, 5), (32, 8, 128, -1)]:
         with pytest.raises(pkg.ops.PmxError):
             pkg.ops.decode_plan(16, hq, hkv, d, 4096, cus=256, kernel=k)
 
