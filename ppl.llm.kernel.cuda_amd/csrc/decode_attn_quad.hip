@@ -254,6 +254,11 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
         if (nb == 1 && tail_partial) clamp_offsets(pos);
         request_k(ka, mka, pos);
         request_v(va, ka.boff);
+        // the second block's K travels together with the first block: the loop's first iteration finds it requested
+        // (a piece would otherwise pay a second memory latency before its second block)
+        const int npos_first = pos + (nb > 1 ? BLK : 0);
+        if (tail_partial && nb == 2) clamp_offsets(npos_first);
+        request_k(kb, mkb, npos_first);
 
         // ---- A operands: this lane supplies row t4 = query head t4, its chunk's 16 channels ----
         half4_t qa[4];
@@ -496,9 +501,12 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
             // block of each other, so that the second set's requests find the lines in the cache levels
             // (every wave of the workgroup runs the same number of blocks).
             if (GP > 1) __syncthreads();
-            int npos = pos + (i + 1 < nb ? BLK : 0);
-            if (tail_partial && i + 2 == nb) clamp_offsets(npos);
-            request_k(kb, mkb, npos);
+            int npos = npos_first;
+            if (i > 0) {
+                npos = pos + (i + 1 < nb ? BLK : 0);
+                if (tail_partial && i + 2 == nb) clamp_offsets(npos);
+                request_k(kb, mkb, npos);
+            }
             logits_softmax(ka, mka, tail_partial && i + 1 == nb);
             request_v(vb, kb.boff);
             accumulate_pv(va);
