@@ -38,7 +38,9 @@ def run_prefill(pkg, dev, is_causal=None, **extra):
 
 @pytest.mark.parametrize("cache_mode", [0, 1])
 @pytest.mark.parametrize("shape", [(8, 2, 128), (4, 4, 128), (12, 2, 128), (8, 8, 64), (16, 2, 64), (2, 1, 128), (16, 1, 128),
-                                   (8, 2, 256), (4, 4, 256), (16, 1, 256), (8, 2, 96), (6, 6, 96), (12, 2, 96)])
+                                   (8, 2, 256), (4, 4, 256), (16, 1, 256), (8, 2, 96), (6, 6, 96), (12, 2, 96),
+                                   # multi-query models: the query heads of one kv head fill most of a workgroup's columns
+                                   (48, 1, 128), (71, 1, 64), (24, 1, 256)])
 def test_prefill_matches_oracle(pkg, oracle, shape, cache_mode):
     hq, hkv, d = shape
     bt, dev, q, cache, scale = make_case(pkg, oracle, 300 + hq + d, num_heads=hq, num_kv_heads=hkv, head_dim=d,
