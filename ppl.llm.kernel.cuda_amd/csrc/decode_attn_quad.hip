@@ -1,6 +1,6 @@
-// Decode attention over the int8 group-8 KV cache, variant for head_dim 64 and 128 (an even number of kv heads)
-// and 256, up to four query heads per kv head (MHA and the common GQA shapes; up to eight at head_dim 128
-// with kv heads in eights).  Same semantics, token ranges, pieces and workspace as decode_attn.hip
+// Decode attention over the int8 group-8 KV cache, variant for head_dim 64 and 128 (two or more kv heads; with an
+// odd number the last half-wave idles) and 256, up to four query heads per kv head (MHA and the common GQA shapes;
+// up to eight at head_dim 256, and at head_dim 128 with kv heads in eights).  Same semantics, token ranges, pieces and workspace as decode_attn.hip
 // (reference: src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/kernel.cu:229-679,
 // 1115-1891); what differs is the lane layout, chosen so that the matrix pipe computes
 // the q.k products while the vector pipe converts and accumulates:

@@ -217,7 +217,7 @@ int launch_decode(const DecodeLaunch& a, int stage, hipStream_t stream); // stag
 enum DecodeKernel : int32_t {
     kDecodeKernelAuto = 0,    // as a request: by shape
     kDecodeKernelGeneral = 1, // decode_attn.hip: VALU, every head_dim and head count, up to 8 query heads per pass
-    kDecodeKernelQuad = 2,    // decode_attn_quad.hip: 4x4x4 MFMA per quad; head_dim 128 (even number of kv heads) or 256
+    kDecodeKernelQuad = 2,    // decode_attn_quad.hip: 4x4x4 MFMA per quad; head_dim 64 or 128 (two or more kv heads) or 256
     kDecodeKernelMfma16 = 3,  // decode_attn_mfma.hip: 16 query-head columns, head_dim 128
     kDecodeKernelMfma32 = 4,  // decode_attn_mfma.hip: 32 query-head columns per pass, head_dim 128 or 64
 };
