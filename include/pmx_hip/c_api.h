@@ -262,9 +262,25 @@ typedef struct pmxhip_prefill_params {
      * batch has at most rows / (positions per workgroup) + sequences query tiles, far fewer than
      * sequences * tiles of max_seqlen when one long sequence sits among short ones. */
     int64_t prefill_query_rows;
+    /* Optional workspace, NULL = none.  No counterpart in the reference's call (its flash_attn2 split-KV path keeps
+     * its partial results inside the kernel's own allocation, flash_api.cu:169-178).  With at least
+     * pmxhip_prefill_workspace_size() bytes (16-byte aligned) a batch of short chunks -- max_seqlen * (Hq / KVH)
+     * <= 32, head_dim 64 or 128, no attn_mask, alibi or current_key -- runs on the decode step's MFMA kernel over
+     * token ranges, with (query position, query head) pairs as its columns and the split-KV pieces in this
+     * workspace; without it, or for any other batch, the tile kernel runs.  Results are the same within the tolerance. */
+    void* workspace;
+    int64_t workspace_size;
 } pmxhip_prefill_params;
 
 PMXHIP_API int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t stream);
+
+/* Bytes of pmxhip_prefill_params::workspace with which a batch runs its short chunks on the decode step's kernel;
+ * 0 when the batch is not one of short chunks (the tile kernel needs no workspace).  compute_units 0 = those of the
+ * current device.  The operator class adds this to what it reports as cfg.workspace_size (the decode and the
+ * prefill stage run one after the other on the stream and share the buffer). */
+PMXHIP_API int64_t pmxhip_prefill_workspace_size(int64_t batch, int64_t decoding_batches, int64_t max_seqlen,
+                                                 int64_t max_kvlen, int64_t num_heads, int64_t num_kv_heads,
+                                                 int64_t head_dim, int32_t compute_units);
 
 /* ---- the operator class behind a C handle -----------------------------------
  * Drives the C++ class (heuristic_prepare / forward_*) so that a non-C++ host

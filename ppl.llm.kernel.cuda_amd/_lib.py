@@ -27,7 +27,7 @@ EXPORTED_SYMBOLS = (
     "pmxhip_decode_plan_make", "pmxhip_decode_plan_make_kernel", "pmxhip_decode_attention",
     "pmxhip_decode_attention_stage", "pmxhip_decode_attention_static", "pmxhip_decode_kernel_name",
     "pmxhip_splitkv_combine",
-    "pmxhip_prefill_attention",
+    "pmxhip_prefill_attention", "pmxhip_prefill_workspace_size",
     "pmxhip_mhca_create", "pmxhip_mhca_destroy", "pmxhip_mhca_heuristic_prepare",
     "pmxhip_mhca_get_derived", "pmxhip_mhca_set_workspace",
     "pmxhip_mhca_forward_kvstore", "pmxhip_mhca_forward_decode", "pmxhip_mhca_forward_prefill",
@@ -101,6 +101,7 @@ class PrefillParams(ctypes.Structure):
         ("attn_mask", c_vp), ("mask_stride_s", c_i64), ("mask_stride_h", c_i64), ("alibi_slopes", c_vp),
         ("current_key", c_vp), ("current_value", c_vp), ("key_stride_s", c_i64), ("value_stride_s", c_i64),
         ("prefill_query_rows", c_i64),
+        ("workspace", c_vp), ("workspace_size", c_i64),
     ]
 
 
@@ -228,6 +229,8 @@ def lib():
     L.pmxhip_decode_attention_stage.argtypes = [ctypes.POINTER(DecodeParams), c_i32, c_vp]
     L.pmxhip_splitkv_combine.restype = ctypes.c_int
     L.pmxhip_splitkv_combine.argtypes = [c_vp] * 4 + [c_i64, c_i64, c_vp, c_vp]
+    L.pmxhip_prefill_workspace_size.restype = c_i64
+    L.pmxhip_prefill_workspace_size.argtypes = [c_i64] * 7 + [c_i32]
     L.pmxhip_prefill_attention.restype = ctypes.c_int
     L.pmxhip_prefill_attention.argtypes = [ctypes.POINTER(PrefillParams), c_vp]
     L.pmxhip_mhca_create.restype = c_vp

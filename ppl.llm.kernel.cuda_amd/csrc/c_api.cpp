@@ -417,6 +417,44 @@ int pmxhip_splitkv_combine(const float* partial_out, const float* partial_ml, co
     return launch_status("splitkv_combine");
 }
 
+namespace {
+
+// Short chunks (a few query tokens per sequence: speculative decoding's candidates, the tail of a chunked prefill)
+// leave most of the tile kernel's 256 columns empty and are bound by its tile staging.  Where a kv head's (query
+// position, query head) pairs fit the 32 columns of the decode step's MFMA kernel they run there instead, over token
+// ranges with a combine kernel, which streams the cache at the decode rate.  That path has no mask, alibi or fp16-K/V
+// form and serves head_dim 64 and 128.
+constexpr int64_t kPrefillChunkColumns = 32;
+
+bool prefill_chunk_shape(int64_t max_seqlen, int64_t num_heads, int64_t num_kv_heads, int64_t head_dim)
+{
+    if (head_dim != 64 && head_dim != 128) return false;
+    if (num_kv_heads <= 0 || num_heads % num_kv_heads != 0 || max_seqlen <= 0) return false;
+    return max_seqlen * (num_heads / num_kv_heads) <= kPrefillChunkColumns;
+}
+
+// the plan of that path: a decode step of `prefill_batches` sequences whose kv heads have max_seqlen * G columns each
+int prefill_chunk_plan(int64_t prefill_batches, int64_t max_seqlen, int64_t max_kvlen, int64_t num_heads, int64_t num_kv_heads,
+                       int64_t head_dim, int32_t compute_units, pmxhip_decode_plan* plan)
+{
+    const int64_t columns = max_seqlen * (num_heads / num_kv_heads);
+    return pmxhip_decode_plan_make_kernel(prefill_batches, num_kv_heads * columns, num_kv_heads, head_dim, max_kvlen,
+                                          compute_units, 0, PMXHIP_DECODE_KERNEL_MFMA32, plan);
+}
+
+} // namespace
+
+int64_t pmxhip_prefill_workspace_size(int64_t batch, int64_t decoding_batches, int64_t max_seqlen, int64_t max_kvlen,
+                                      int64_t num_heads, int64_t num_kv_heads, int64_t head_dim, int32_t compute_units)
+{
+    const int64_t prefill_batches = batch - decoding_batches;
+    if (prefill_batches <= 0 || decoding_batches < 0 || !prefill_chunk_shape(max_seqlen, num_heads, num_kv_heads, head_dim)) return 0;
+    pmxhip_decode_plan plan;
+    if (prefill_chunk_plan(prefill_batches, max_seqlen, max_kvlen, num_heads, num_kv_heads, head_dim, compute_units, &plan) != PMXHIP_SUCCESS)
+        return 0;
+    return plan.workspace_size;
+}
+
 int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t stream)
 {
     if (!p) return fail(PMXHIP_INVALID_VALUE, "prefill_attention: null params");
@@ -452,6 +490,51 @@ int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t str
         return fail(PMXHIP_UNSUPPORTED, "prefill_attention: query must be 16-byte aligned with a row stride that is a multiple of 8");
     if ((reinterpret_cast<uintptr_t>(p->output) & 7u) || p->output_stride_s % 4 != 0)
         return fail(PMXHIP_UNSUPPORTED, "prefill_attention: output must be 8-byte aligned with a row stride that is a multiple of 4");
+
+    // short chunks on the decode step's kernels, where the shape, the inputs and the caller's workspace allow
+    if (!from_current && !p->attn_mask && !p->alibi_slopes && p->workspace && aligned16(p->workspace) &&
+        prefill_chunk_shape(p->max_seqlen, p->num_heads, p->num_kv_heads, p->head_dim)) {
+        pmxhip_decode_plan plan;
+        if (prefill_chunk_plan(prefill_batches, p->max_seqlen, p->max_kvlen, p->num_heads, p->num_kv_heads, p->head_dim, 0, &plan) ==
+                PMXHIP_SUCCESS &&
+            plan.workspace_size <= p->workspace_size && aligned16(p->cache) && !(reinterpret_cast<uintptr_t>(p->scale) & 3u)) {
+            const int64_t g = p->num_heads / p->num_kv_heads;
+            pmxhip_decode_params d;
+            memset(&d, 0, sizeof(d));
+            d.query = p->query;
+            d.output = p->output;
+            d.cache = p->cache;
+            d.scale = p->scale;
+            d.cachestarts = p->cachestarts + p->decoding_batches * p->cachestarts_stride_b;
+            d.kvstarts = p->kvstarts + p->decoding_batches;
+            d.attn_scale = p->attn_scale;
+            d.layer_idx = p->layer_idx;
+            d.num_kv_repeats = p->max_seqlen * g; // columns per kv head
+            d.page_size = p->page_size;
+            d.query_stride_s = p->query_stride_s;
+            d.output_stride_s = p->output_stride_s;
+            d.cache_stride_s = p->cache_stride_s;
+            d.cache_stride_l = p->cache_stride_l;
+            d.cache_stride_h = p->cache_stride_h;
+            d.cache_stride_kv = p->cache_stride_kv;
+            d.cachestarts_stride_b = p->cachestarts_stride_b;
+            d.decoding_batches = prefill_batches;
+            d.num_heads = p->num_kv_heads * d.num_kv_repeats;
+            d.num_kv_heads = p->num_kv_heads;
+            d.head_dim = p->head_dim;
+            d.cache_mode = p->cache_mode;
+            d.num_token_ranges = plan.num_token_ranges;
+            d.workspace = p->workspace;
+            d.workspace_size = p->workspace_size;
+            d.kernel_request = PMXHIP_DECODE_KERNEL_MFMA32;
+            pmxhip::DecodeLaunch c;
+            if (int rc = decode_prepare("prefill_attention", &d, d.workspace, d.workspace_size, &c)) return rc;
+            c.seqstarts = p->seqstarts + p->decoding_batches;
+            c.chunk_q_heads = (int32_t)g;
+            c.chunk_causal = p->is_causal ? 1 : 0;
+            return launch_result("prefill_attention", pmxhip::launch_decode(c, 0, stream));
+        }
+    }
 
     pmxhip::PrefillLaunch a{};
     a.query = p->query;

@@ -216,6 +216,13 @@ ppl::common::RetCode dynamic_batching_multi_head_cache_attention::heuristic_prep
     cfg.decoding_multi_block_partial_log_sum_exp_size = plan.partial_ml_size;
     cfg.decoding_multi_block_counter_size = 0;
     cfg.workspace_size = plan.workspace_size;
+    // short prefill chunks run on the decode step's kernel and keep their split-KV pieces in the same workspace (the
+    // two stages follow each other on the stream)
+    if (enable_cache_prefill && prefill_batches > 0 && !attn_mask && !alibi_slopes) {
+        const int64_t chunk_ws = pmxhip_prefill_workspace_size(batch, decoding_batches, max_seqlen, max_kvlen, num_heads,
+                                                               num_kv_heads, head_dim, device_prop.multiProcessorCount);
+        if (chunk_ws > cfg.workspace_size) cfg.workspace_size = chunk_ws;
+    }
     cfg.enable_cache_prefill = enable_cache_prefill;
     return ppl::common::RC_SUCCESS;
 }
@@ -332,6 +339,8 @@ ppl::common::RetCode dynamic_batching_multi_head_cache_attention::forward_prefil
     p.mask_stride_h = cfg.mask_stride_h;
     p.alibi_slopes = static_cast<const float*>(cfg.alibi_slopes);
     p.prefill_query_rows = cfg.prefill_query_rows;
+    p.workspace = cfg.workspace;
+    p.workspace_size = cfg.workspace_size;
     if (!cfg.enable_cache_prefill) { // kernel.cu:2181-2212: the step's own fp16 K/V only, no cache read
         p.current_key = cfg.current_key;
         p.current_value = cfg.current_value;

@@ -493,7 +493,17 @@ __global__ __launch_bounds__(64 * NW) void decode_combine_kernel(const DecodeLau
     const int64_t total = stream_length(a.kvstarts[a.decoding_batches] - kv_base, a.decoding_batches);
     const int64_t s_beg = sequence_origin(a.kvstarts[b] - kv_base, b);
     const int64_t s_end = s_beg + (a.kvstarts[b + 1] - a.kvstarts[b]);
-    half_t* out = (half_t*)a.output + (int64_t)b * a.output_stride_s + (int64_t)h * D;
+    int64_t out_row = b;
+    int out_head = h;
+    if (a.seqstarts != nullptr) { // chunks of query tokens: h is a (query position, query head) column of a kv head
+        const int gv = (int)a.num_kv_repeats, gr = a.chunk_q_heads;
+        const int gq = h % gv, cpos = gq / gr;
+        out_row = a.seqstarts[b];
+        if (cpos >= (int)(a.seqstarts[b + 1] - out_row)) return; // the sequence's chunk is shorter
+        out_row += cpos;
+        out_head = (h / gv) * gr + (gq - cpos * gr);
+    }
+    half_t* out = (half_t*)a.output + out_row * a.output_stride_s + (int64_t)out_head * D;
     if (s_end <= s_beg) { // empty sequence: the reference yields 0/(0+1e-6) = 0 (kernel.cu:516)
         for (int c = tid; c < D; c += 64 * NW) out[c] = (half_t)0.f;
         return;

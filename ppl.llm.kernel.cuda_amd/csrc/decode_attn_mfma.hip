@@ -60,10 +60,16 @@ __device__ __forceinline__ int vt_index(int row /* from vt_row */, int pos /* 0.
 
 // D: head_dim 128 or 64 (half the k-steps, channel blocks and V units).  blockIdx.z: which 32 query heads of the
 // kv head's group are this launch's columns (more than 32 query heads per kv head take several passes over the cache).
-template <int NW, bool PAGED, bool MASK, int D>
+// CHUNK: the sequences have a few query tokens each instead of one (short prefill chunks, the candidate tokens of
+// speculative decoding: a.seqstarts gives their query rows).  The columns of a kv head are then (query position,
+// query head) pairs, column = position * (query heads per kv head) + head, a.num_kv_repeats counts those columns and
+// a.num_heads the columns of all kv heads; a column attends the tokens below its own causal limit.  Everything else
+// -- ranges, pieces, workspace -- is the decode step's, with columns in place of query heads.
+template <int NW, bool PAGED, bool MASK, int D, bool CHUNK = false>
 __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(const DecodeLaunch a)
 {
     static_assert(D == 128 || D == 64, "head_dim");
+    static_assert(!(CHUNK && MASK), "no attn_mask form for chunks");
     constexpr int HALF = D / 2; // channels of a token that a half-wave's lanes hold as K bytes
     constexpr int KW = D / 32;  // 16-byte words of those bytes
     constexpr int KS = D / 16;  // k-steps of S^T
@@ -79,6 +85,9 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
     const int hh = lane >> 5;
     const int G = (int)a.num_kv_repeats;
     const int gq = blockIdx.z * kMfmaBlock + l32; // this lane's column: query head gq of the kv head's group
+    const int GR = CHUNK ? (int)a.chunk_q_heads : G;       // query heads per kv head
+    const int cpos = CHUNK ? gq / GR : 0;                  // the column's query position within its sequence's chunk
+    const int cg = CHUNK ? gq - cpos * GR : gq;            // ... and its query head within the kv head's group
     const int kvh = blockIdx.y * NW + wave;
     half_t* const sV = s_vt[wave][0];
     half_t* const sVlo = s_vt[wave][1];
@@ -128,10 +137,19 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
 
         // ---- Q fragments (B operand of S^T): column = query head l32; k-step s of half-wave hh covers the
         // channels [HALF hh + 16 (s / 2) + 8 (s % 2), + 8), so that a lane's K bytes are HALF consecutive ones ----
+        int64_t q_row = b; // row of the query and output tensors
+        int qlen = 1;
+        if (CHUNK) {
+            q_row = a.seqstarts[b];
+            qlen = (int)(a.seqstarts[b + 1] - q_row);
+        }
+        const bool on = gq < G && cpos < qlen;
+        // tokens this column attends: all of the sequence, or (causal chunk) those up to its own position
+        const int col_lim = CHUNK && a.chunk_causal ? (int)len - qlen + cpos + 1 : (int)len;
+        const int first_cut = CHUNK && a.chunk_causal ? (int)len - qlen + 1 : (int)len; // the smallest limit of any column
         f16x8 qf[KS];
         {
-            const bool on = gq < G;
-            const half_t* qp = (const half_t*)a.query + (int64_t)b * a.query_stride_s + (int64_t)(kvh * G + (on ? gq : 0)) * D + HALF * hh;
+            const half_t* qp = (const half_t*)a.query + (q_row + (on ? cpos : 0)) * a.query_stride_s + (int64_t)(kvh * GR + (on ? cg : 0)) * D + HALF * hh;
 #pragma unroll
             for (int s = 0; s < KS; ++s) {
                 qf[s] = *(const f16x8*)(qp + 8 * s);
@@ -269,11 +287,12 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
                     s_acc[e] += (float)mask_row[t < pe32 ? t : pe32 - 1] * (kLog2e / sm_scale);
                 }
             }
-            if (pos + kMfmaBlock > pe32) { // only the last block of a piece (wave-uniform)
+            if (pos + kMfmaBlock > pe32 || (CHUNK && pos + kMfmaBlock > first_cut)) { // a piece's last block, or one that reaches a column's causal limit (wave-uniform)
+                const int lim = CHUNK ? (col_lim < pe32 ? col_lim : pe32) : pe32;
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int t = pos + 8 * (e >> 2) + 4 * hh + (e & 3);
-                    if (t >= pe32) s_acc[e] = -INFINITY;
+                    if (t >= lim) s_acc[e] = -INFINITY;
                 }
             }
             // maximum of the raw dot products; the (positive) logit scale is applied to it afterwards
@@ -326,11 +345,11 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
         // ---- end of the piece: element e of block cb <-> channel 32 cb + 8 (e / 4) + 4 hh + e % 4 ----
         const float l_tot = l_run + __shfl_xor(l_run, 32);
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-        if (gq < G) {
-            const int h = kvh * G + gq;
+        if (on) {
+            const int h = kvh * G + gq; // the column among all columns: its slot in the pieces' workspace
             const bool whole = (pa == 0) && (pe == len);
             if (whole) {
-                half_t* op = (half_t*)a.output + (int64_t)b * a.output_stride_s + (int64_t)h * D;
+                half_t* op = (half_t*)a.output + (q_row + cpos) * a.output_stride_s + (int64_t)(kvh * GR + cg) * D;
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
@@ -715,6 +734,11 @@ template <int NW, int D>
 static void launch_decode_mfma32(const DecodeLaunch& a, dim3 grid, dim3 block, hipStream_t stream)
 {
     const bool paged = a.cache_mode == 1, mask = a.attn_mask != nullptr;
+    if (a.seqstarts != nullptr) { // chunks of query tokens (no mask form: the caller checks)
+        if (paged) hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, true, false, D, true>), grid, block, 0, stream, a);
+        else hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, false, false, D, true>), grid, block, 0, stream, a);
+        return;
+    }
     if (paged) {
         if (mask) hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, true, true, D>), grid, block, 0, stream, a);
         else hipLaunchKernelGGL((decode_attention_mfma_kernel<NW, true, false, D>), grid, block, 0, stream, a);

@@ -36,7 +36,6 @@ namespace {
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
-constexpr int kQuadMaxHeads = 8; // kv heads per workgroup (two per wave): eight, or four or two when the kv heads do not come in eights
 constexpr int kQuadBlock = 16;  // tokens per block
 constexpr int kDppRor8 = 0x128; // row_ror:8 = lane ^ 8 inside a row of 16
 

@@ -68,6 +68,12 @@ struct DecodeLaunch {
                                   // of the kernel named by `kernel` (the combine kernel derives the same cuts from it)
     int32_t min_tokens_per_range;
     int32_t kernel;               // DecodeKernel that runs the token ranges; never kDecodeKernelAuto at launch
+    // Chunks of a few query tokens per sequence on the 32-column kernel (nullptr = one query token per sequence, row =
+    // sequence index): rows of sequence b are seqstarts[b] .. seqstarts[b + 1]; num_kv_repeats and num_heads then count
+    // (query position, query head) columns, chunk_q_heads the query heads per kv head.
+    const int64_t* seqstarts;
+    int32_t chunk_q_heads;
+    int32_t chunk_causal;
 };
 
 struct PrefillLaunch {

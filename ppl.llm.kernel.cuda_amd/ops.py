@@ -168,11 +168,12 @@ def prefill_attention(query, output, cache, scale, seqstarts, kvstarts, cachesta
                       batch, decoding_batches, max_seqlen, max_kvlen, layer_idx, num_heads, num_kv_heads,
                       head_dim, cache_mode, page_size, cache_stride_s, cache_stride_l, cache_stride_h,
                       cache_stride_kv, cachestarts_stride_b, attn_mask=None, mask_stride_s=0, mask_stride_h=0,
-                      alibi_slopes=None, current_key=None, current_value=None, prefill_query_rows=None, stream=None,
-                      check=True):
+                      alibi_slopes=None, current_key=None, current_value=None, prefill_query_rows=None, workspace=None,
+                      stream=None, check=True):
     """Multi-query-token attention of the prefill sequences.  Optional: additive half `attn_mask` with its
-    strides, float32 `alibi_slopes` [Hq], and `current_key`/`current_value` [rows, KVH, D] to attend over
-    the step's own fp16 rows instead of the cache."""
+    strides, float32 `alibi_slopes` [Hq], `current_key`/`current_value` [rows, KVH, D] to attend over
+    the step's own fp16 rows instead of the cache, and a `workspace` of prefill_workspace_size() bytes with which a
+    batch of short chunks runs on the decode step's kernel."""
     p = PrefillParams()
     p.query = _ptr(query)
     p.output = _ptr(output)
@@ -211,10 +212,20 @@ def prefill_attention(query, output, cache, scale, seqstarts, kvstarts, cachesta
         p.value_stride_s = num_kv_heads * head_dim
     # the rows of the prefill sequences follow from the query tensor (decode sequences have one row each)
     p.prefill_query_rows = (int(query.shape[0]) - decoding_batches) if prefill_query_rows is None else prefill_query_rows
+    if workspace is not None:
+        p.workspace = _ptr(workspace)
+        p.workspace_size = int(workspace.numel() * workspace.element_size())
     rc = _lib.lib().pmxhip_prefill_attention(ctypes.byref(p), _stream(stream))
     if check and rc != RC_SUCCESS:
         raise PmxError(rc, "prefill_attention")
     return rc
+
+
+def prefill_workspace_size(batch, decoding_batches, max_seqlen, max_kvlen, num_heads, num_kv_heads, head_dim, cus=0):
+    """Bytes of the workspace with which a batch of short chunks runs on the decode step's kernel; 0 for every
+    other batch (cus = 0: the compute units of the current device)."""
+    return int(_lib.lib().pmxhip_prefill_workspace_size(batch, decoding_batches, max_seqlen, max_kvlen, num_heads,
+                                                        num_kv_heads, head_dim, cus))
 
 
 def _rope_params(query, key, start_pos, seqstarts, rotated_query, rotated_key, *, theta, rotary_dim, batch, max_seqlen,

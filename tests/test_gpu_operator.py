@@ -61,6 +61,18 @@ def test_mixed_batch_at_the_other_head_dims(pkg, oracle, heads):
     full_step(pkg, oracle, bt, rng)
 
 
+@pytest.mark.parametrize("heads,q_lens", [((32, 8, 128), [4, 8, 1, 5]), ((8, 8, 64), [32, 2, 17, 9]), ((16, 2, 128), [3, 4, 2, 1])])
+def test_mixed_batch_with_short_chunks(pkg, oracle, heads, q_lens):
+    """Decode sequences plus chunks of a few query tokens (speculative decoding's candidates): the operator's workspace
+    covers the prefill stage's pieces too, and forward() runs those chunks on the decode step's kernel."""
+    hq, hkv, d = heads
+    bt, rng = pkg.workloads.custom_batch(430 + hq + d, num_heads=hq, num_kv_heads=hkv, head_dim=d, cache_mode=1,
+                                         dec_kv_lens=[300, 33, 1700, 1], prefill_q_lens=q_lens,
+                                         prefill_prior=[1500, 0, 640, 2047], outliers=True, num_layer=2, layer_idx=1)
+    assert pkg.ops.prefill_workspace_size(bt.batch, bt.decoding_batches, bt.max_seqlen, bt.max_kvlen, hq, hkv, d) > 0
+    full_step(pkg, oracle, bt, rng)
+
+
 def test_scaled_c5_through_the_operator(pkg, oracle):
     bt, rng = pkg.workloads.make_batch("C5", scale=0.06)
     full_step(pkg, oracle, bt, rng)

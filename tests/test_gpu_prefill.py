@@ -67,6 +67,47 @@ def test_prefill_short_chunks_over_long_histories(pkg, oracle, shape):
     assert_attention_close(got, ref, "short chunks %s" % (shape,))
 
 
+@pytest.mark.parametrize("is_causal", [True, False])
+@pytest.mark.parametrize("cache_mode", [0, 1])
+@pytest.mark.parametrize("shape,q_lens", [((32, 8, 128), [4, 1, 8, 3, 2, 8, 5]), ((8, 8, 64), [16, 5, 32, 1, 31, 2, 9]),
+                                          ((8, 1, 128), [4, 2, 1, 3, 4, 1, 2]), ((16, 2, 64), [3, 4, 1, 2, 4, 4, 1]),
+                                          ((4, 4, 128), [32, 7, 20, 1, 2, 30, 16]), ((12, 3, 128), [8, 2, 1, 7, 3, 8, 4])])
+def test_prefill_short_chunks_on_the_decode_kernel(pkg, oracle, shape, q_lens, cache_mode, is_causal):
+    """With the workspace of prefill_workspace_size() a batch whose (query position, query head) pairs per kv head fit
+    32 columns runs on the decode step's MFMA kernel over token ranges: same results as the oracle and as the tile
+    kernel, pieces in the workspace, rows of the decode sequences untouched."""
+    hq, hkv, d = shape
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 360 + hq + d, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                         cache_mode=cache_mode, dec_kv_lens=[33, 140],
+                                         prefill_q_lens=q_lens, prefill_prior=[1500, 0, 900, 33, 2047, 126, 640],
+                                         outliers=True)
+    bt.is_causal = is_causal
+    ref = oracle_prefill(oracle, bt, q, cache, scale)
+    ws_bytes = pkg.ops.prefill_workspace_size(bt.batch, bt.decoding_batches, bt.max_seqlen, bt.max_kvlen, hq, hkv, d)
+    assert ws_bytes > 0
+    ws = torch.full((ws_bytes // 4,), float("nan"), dtype=torch.float32, device="cuda")
+    got = run_prefill(pkg, dev, is_causal=is_causal, workspace=ws)
+    assert_attention_close(got[bt.decoding_batches:], ref[bt.decoding_batches:], "chunks on the decode kernel %s" % (shape,))
+    assert np.isnan(got[:bt.decoding_batches]).all()       # the decode sequences' rows are not this stage's
+    assert not torch.isnan(ws).all()                       # pieces were written: the decode kernel ran
+    tile = run_prefill(pkg, dev, is_causal=is_causal)      # no workspace: the tile kernel
+    assert_attention_close(tile[bt.decoding_batches:], ref[bt.decoding_batches:], "tile kernel %s" % (shape,))
+    # a workspace that is too small is not an error: the tile kernel runs
+    small = torch.full((16,), float("nan"), dtype=torch.float32, device="cuda")
+    got2 = run_prefill(pkg, dev, is_causal=is_causal, workspace=small)
+    assert_attention_close(got2[bt.decoding_batches:], ref[bt.decoding_batches:], "small workspace %s" % (shape,))
+    assert torch.isnan(small).all()
+
+
+def test_prefill_workspace_size_is_zero_for_other_batches(pkg, hip_lib):
+    f = pkg.ops.prefill_workspace_size
+    assert f(8, 2, 8, 4096, 32, 8, 128, 256) > 0            # 8 positions x 4 query heads per kv head = 32 columns
+    assert f(8, 2, 9, 4096, 32, 8, 128, 256) == 0           # 36 columns
+    assert f(8, 8, 8, 4096, 32, 8, 128, 256) == 0           # no prefill sequence
+    assert f(8, 2, 8, 4096, 32, 8, 96, 256) == 0 and f(8, 2, 8, 4096, 32, 8, 256, 256) == 0
+    assert f(8, 2, 32, 4096, 8, 8, 64, 256) > 0
+
+
 @pytest.mark.parametrize("n_seq,is_causal", [(150, True), (150, False), (1100, True)])
 def test_prefill_many_sequences_every_tile_once(pkg, oracle, n_seq, is_causal):
     """The kernel numbers the batch's query tiles in the order of falling cost and every workgroup looks its own
