@@ -265,7 +265,7 @@ typedef struct pmxhip_prefill_params {
     /* Optional workspace, NULL = none.  No counterpart in the reference's call (its flash_attn2 split-KV path keeps
      * its partial results inside the kernel's own allocation, flash_api.cu:169-178).  With at least
      * pmxhip_prefill_workspace_size() bytes (16-byte aligned) a batch of short chunks -- max_seqlen * (Hq / KVH)
-     * <= 32, head_dim 64 or 128, no attn_mask, alibi or current_key -- runs on the decode step's MFMA kernel over
+     * <= 32, head_dim 64 or 128, no attn_mask, alibi or current_key -- runs on the decode step's MFMA kernels over
      * token ranges, with (query position, query head) pairs as its columns and the split-KV pieces in this
      * workspace; without it, or for any other batch, the tile kernel runs.  Results are the same within the tolerance. */
     void* workspace;

@@ -433,13 +433,19 @@ bool prefill_chunk_shape(int64_t max_seqlen, int64_t num_heads, int64_t num_kv_h
     return max_seqlen * (num_heads / num_kv_heads) <= kPrefillChunkColumns;
 }
 
+// the kernel of that path: the 16-column form where the columns fit it (head_dim 128 only), else the 32-column form
+int32_t prefill_chunk_kernel(int64_t columns, int64_t head_dim)
+{
+    return columns <= 16 && head_dim == 128 ? PMXHIP_DECODE_KERNEL_MFMA16 : PMXHIP_DECODE_KERNEL_MFMA32;
+}
+
 // the plan of that path: a decode step of `prefill_batches` sequences whose kv heads have max_seqlen * G columns each
 int prefill_chunk_plan(int64_t prefill_batches, int64_t max_seqlen, int64_t max_kvlen, int64_t num_heads, int64_t num_kv_heads,
                        int64_t head_dim, int32_t compute_units, pmxhip_decode_plan* plan)
 {
     const int64_t columns = max_seqlen * (num_heads / num_kv_heads);
     return pmxhip_decode_plan_make_kernel(prefill_batches, num_kv_heads * columns, num_kv_heads, head_dim, max_kvlen,
-                                          compute_units, 0, PMXHIP_DECODE_KERNEL_MFMA32, plan);
+                                          compute_units, 0, prefill_chunk_kernel(columns, head_dim), plan);
 }
 
 } // namespace
@@ -526,7 +532,7 @@ int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t str
             d.num_token_ranges = plan.num_token_ranges;
             d.workspace = p->workspace;
             d.workspace_size = p->workspace_size;
-            d.kernel_request = PMXHIP_DECODE_KERNEL_MFMA32;
+            d.kernel_request = prefill_chunk_kernel(d.num_kv_repeats, p->head_dim);
             pmxhip::DecodeLaunch c;
             if (int rc = decode_prepare("prefill_attention", &d, d.workspace, d.workspace_size, &c)) return rc;
             c.seqstarts = p->seqstarts + p->decoding_batches;

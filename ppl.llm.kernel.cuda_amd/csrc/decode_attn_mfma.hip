@@ -389,9 +389,11 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
 //   O^T tile (16 channels x 16 columns, eight per block): A = row `channel 16 cb + r` of the V^T tile,
 //     16-byte block qq, whose eight positions are the tokens of the lane's two S^T accumulators in order:
 //     position 8 qq + 4 tile + i <-> token 16 tile + 4 qq + i; the accumulator holds channels 16 cb + 4 qq + i
-template <int NW, bool PAGED, bool MASK>
+// CHUNK: as in the 32-column kernel (columns = (query position, query head) pairs of short chunks).
+template <int NW, bool PAGED, bool MASK, bool CHUNK = false>
 __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(const DecodeLaunch a)
 {
+    static_assert(!(CHUNK && MASK), "no attn_mask form for chunks");
     constexpr int D = kMfmaD;
     __shared__ __attribute__((aligned(16))) half_t s_vt[NW][2][D * kMfmaBlock]; // [wave][hi, lo]
     // a block's raw K rows, on their way from whole-line loads to the lanes that hold them as MFMA operands:
@@ -404,6 +406,9 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
     const int r16 = lane & 15;
     const int qq = lane >> 4;
     const int G = (int)a.num_kv_repeats;
+    const int GR = CHUNK ? (int)a.chunk_q_heads : G;       // query heads per kv head
+    const int cpos = CHUNK ? r16 / GR : 0;                 // the column's query position within its sequence's chunk
+    const int cg = CHUNK ? r16 - cpos * GR : r16;          // ... and its query head within the kv head's group
     const int kvh = blockIdx.y * NW + wave;
     half_t* const sV = s_vt[wave][0];
     half_t* const sVlo = s_vt[wave][1];
@@ -455,10 +460,19 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
         };
 
         // ---- Q fragments (B operand of S^T): column = query head r16 ----
+        int64_t q_row = b; // row of the query and output tensors
+        int qlen = 1;
+        if (CHUNK) {
+            q_row = a.seqstarts[b];
+            qlen = (int)(a.seqstarts[b + 1] - q_row);
+        }
+        const bool on = r16 < G && cpos < qlen;
+        // tokens this column attends: all of the sequence, or (causal chunk) those up to its own position
+        const int col_lim = CHUNK && a.chunk_causal ? (int)len - qlen + cpos + 1 : (int)len;
+        const int first_cut = CHUNK && a.chunk_causal ? (int)len - qlen + 1 : (int)len; // the smallest limit of any column
         f16x8 qf[4];
         {
-            const bool on = r16 < G;
-            const half_t* qp = (const half_t*)a.query + (int64_t)b * a.query_stride_s + (int64_t)(kvh * G + (on ? r16 : 0)) * D + 16 * qq;
+            const half_t* qp = (const half_t*)a.query + (q_row + (on ? cpos : 0)) * a.query_stride_s + (int64_t)(kvh * GR + (on ? cg : 0)) * D + 16 * qq;
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 qf[s] = *(const f16x8*)(qp + 64 * (s >> 1) + 8 * (s & 1));
@@ -639,13 +653,14 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
                         s_acc[t][e] += (float)mask_row[tk < pe32 ? tk : pe32 - 1] * (kLog2e / sm_scale);
                     }
             }
-            if (pos + kMfmaBlock > pe32) { // only the last block of a piece (wave-uniform)
+            if (pos + kMfmaBlock > pe32 || (CHUNK && pos + kMfmaBlock > first_cut)) { // a piece's last block, or one that reaches a column's causal limit (wave-uniform)
+                const int lim = CHUNK ? (col_lim < pe32 ? col_lim : pe32) : pe32;
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         const int tk = pos + 16 * t + 4 * qq + e;
-                        if (tk >= pe32) s_acc[t][e] = -INFINITY;
+                        if (tk >= lim) s_acc[t][e] = -INFINITY;
                     }
             }
             // maximum of the raw dot products; the (positive) logit scale is applied to it afterwards
@@ -702,11 +717,11 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
         float l_tot = l_run + __shfl_xor(l_run, 16);
         l_tot += __shfl_xor(l_tot, 32);
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-        if (r16 < G) {
-            const int h = kvh * G + r16;
+        if (on) {
+            const int h = kvh * G + r16; // the column among all columns: its slot in the pieces' workspace
             const bool whole = (pa == 0) && (pe == len);
             if (whole) {
-                half_t* op = (half_t*)a.output + (int64_t)b * a.output_stride_s + (int64_t)h * D;
+                half_t* op = (half_t*)a.output + (q_row + cpos) * a.output_stride_s + (int64_t)(kvh * GR + cg) * D;
 #pragma unroll
                 for (int cb = 0; cb < 8; ++cb) {
                     f16x4 w;
@@ -755,6 +770,11 @@ static void launch_decode_mfma_nw(const DecodeLaunch& a, hipStream_t stream)
     const dim3 block(NW * kWave);
     const bool paged = a.cache_mode == 1, mask = a.attn_mask != nullptr;
     if (a.kernel == kDecodeKernelMfma16) {
+        if (a.seqstarts != nullptr) { // chunks of query tokens (no mask form: the caller checks)
+            if (paged) hipLaunchKernelGGL((decode_attention_mfma16_kernel<NW, true, false, true>), grid, block, 0, stream, a);
+            else hipLaunchKernelGGL((decode_attention_mfma16_kernel<NW, false, false, true>), grid, block, 0, stream, a);
+            return;
+        }
         if (paged) {
             if (mask) hipLaunchKernelGGL((decode_attention_mfma16_kernel<NW, true, true>), grid, block, 0, stream, a);
             else hipLaunchKernelGGL((decode_attention_mfma16_kernel<NW, true, false>), grid, block, 0, stream, a);

@@ -61,7 +61,8 @@ def test_mixed_batch_at_the_other_head_dims(pkg, oracle, heads):
     full_step(pkg, oracle, bt, rng)
 
 
-@pytest.mark.parametrize("heads,q_lens", [((32, 8, 128), [4, 8, 1, 5]), ((8, 8, 64), [32, 2, 17, 9]), ((16, 2, 128), [3, 4, 2, 1])])
+@pytest.mark.parametrize("heads,q_lens", [((32, 8, 128), [4, 8, 1, 5]), ((8, 8, 64), [32, 2, 17, 9]), ((16, 2, 128), [3, 4, 2, 1]),
+                                          ((32, 8, 128), [4, 2, 1, 3])])
 def test_mixed_batch_with_short_chunks(pkg, oracle, heads, q_lens):
     """Decode sequences plus chunks of a few query tokens (speculative decoding's candidates): the operator's workspace
     covers the prefill stage's pieces too, and forward() runs those chunks on the decode step's kernel."""

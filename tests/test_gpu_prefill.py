@@ -71,7 +71,10 @@ def test_prefill_short_chunks_over_long_histories(pkg, oracle, shape):
 @pytest.mark.parametrize("cache_mode", [0, 1])
 @pytest.mark.parametrize("shape,q_lens", [((32, 8, 128), [4, 1, 8, 3, 2, 8, 5]), ((8, 8, 64), [16, 5, 32, 1, 31, 2, 9]),
                                           ((8, 1, 128), [4, 2, 1, 3, 4, 1, 2]), ((16, 2, 64), [3, 4, 1, 2, 4, 4, 1]),
-                                          ((4, 4, 128), [32, 7, 20, 1, 2, 30, 16]), ((12, 3, 128), [8, 2, 1, 7, 3, 8, 4])])
+                                          ((4, 4, 128), [32, 7, 20, 1, 2, 30, 16]), ((12, 3, 128), [8, 2, 1, 7, 3, 8, 4]),
+                                          # up to 16 columns at head_dim 128: the 16-column form of the kernel
+                                          ((32, 8, 128), [4, 1, 2, 3, 4, 4, 1]), ((8, 8, 128), [16, 3, 1, 9, 15, 2, 16]),
+                                          ((16, 2, 128), [2, 1, 2, 2, 1, 2, 2])])
 def test_prefill_short_chunks_on_the_decode_kernel(pkg, oracle, shape, q_lens, cache_mode, is_causal):
     """With the workspace of prefill_workspace_size() a batch whose (query position, query head) pairs per kv head fit
     32 columns runs on the decode step's MFMA kernel over token ranges: same results as the oracle and as the tile
