@@ -95,11 +95,13 @@ def test_cache_beyond_4_gib(pkg, oracle, heads):
     full_step(pkg, oracle, bt, rng)
 
 
-def test_forward_in_a_hip_graph(pkg, oracle):
+@pytest.mark.parametrize("q_lens,prior", [([70], [300]), ([4, 7, 1], [1300, 40, 2000])])
+def test_forward_in_a_hip_graph(pkg, oracle, q_lens, prior):
     """forward() records no memory-set node and allocates nothing, so a caller can capture it: every replay,
-    with eager calls between the replays, gives the rows of the eager call bit for bit."""
+    with eager calls between the replays, gives the rows of the eager call bit for bit.  With a prefill chunk on the
+    tile kernel, and with short chunks on the decode step's kernel."""
     bt, rng = pkg.workloads.custom_batch(404, num_heads=32, num_kv_heads=8, head_dim=128, cache_mode=1,
-                                         dec_kv_lens=[700, 2, 1900, 130, 1], prefill_q_lens=[70], prefill_prior=[300],
+                                         dec_kv_lens=[700, 2, 1900, 130, 1], prefill_q_lens=q_lens, prefill_prior=prior,
                                          outliers=True)
     cache, scale = host_cache(bt)
     dev = pkg.harness.DeviceBatch(bt)
