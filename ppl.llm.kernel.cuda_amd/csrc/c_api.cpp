@@ -503,7 +503,10 @@ int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t str
         pmxhip_decode_plan plan;
         if (prefill_chunk_plan(prefill_batches, p->max_seqlen, p->max_kvlen, p->num_heads, p->num_kv_heads, p->head_dim, 0, &plan) ==
                 PMXHIP_SUCCESS &&
-            plan.workspace_size <= p->workspace_size && aligned16(p->cache) && !(reinterpret_cast<uintptr_t>(p->scale) & 3u)) {
+            plan.workspace_size <= p->workspace_size && aligned16(p->cache) && !(reinterpret_cast<uintptr_t>(p->scale) & 3u) &&
+            // what the decode kernels ask of the layout beyond this stage's own checks (else: the tile kernel)
+            p->cache_stride_s % 16 == 0 && p->cache_stride_l % 16 == 0 && p->cache_stride_h % 16 == 0 && p->cache_stride_kv % 16 == 0 &&
+            p->cache_stride_h >= 0 && 32.0 * (double)p->cache_stride_s + 4.0 * (double)p->cache_stride_h < 2147483648.0) {
             const int64_t g = p->num_heads / p->num_kv_heads;
             pmxhip_decode_params d;
             memset(&d, 0, sizeof(d));
