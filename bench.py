@@ -131,6 +131,64 @@ def extras(torch, ops, dev, bt, replay_times):
     return res
 
 
+def chunk_bench(torch, pkg, spec, steps, replays):
+    """--chunks: the prefill stage on a batch of short chunks (a few query tokens per sequence over a long history, no
+    decode sequences), once on the tile kernel (no workspace) and once with the workspace that routes it to the decode
+    step's MFMA kernel.  A graph of `steps` stage calls replayed `replays` times back to back, median replay."""
+    wl, harness, ops = pkg.workloads, pkg.harness, pkg.ops
+    c = dict(hq=32, hkv=8, d=128, seqs=64, qmin=2, qmax=8, prior=2048, mode=1)
+    c.update({k: int(v) for k, v in (kv.split("=") for kv in spec.split(","))})
+    q_lens = np.random.default_rng(5).integers(c["qmin"], c["qmax"] + 1, c["seqs"]).tolist()
+    bt, rng = wl.custom_batch(11, num_heads=c["hq"], num_kv_heads=c["hkv"], head_dim=c["d"], cache_mode=c["mode"],
+                              dec_kv_lens=[], prefill_q_lens=q_lens, prefill_prior=[c["prior"]] * c["seqs"], outliers=True)
+    dev = harness.DeviceBatch(bt)
+    dev.fill_history(rng, max_rows=1 << 15)
+    q, k, v = wl.step_inputs(bt, rng)
+    dev.set_step_inputs(q, k, v)
+    kw = dict(attn_scale=bt.attn_scale, is_causal=True, batch=bt.batch, decoding_batches=0, max_seqlen=bt.max_seqlen,
+              max_kvlen=bt.max_kvlen, layer_idx=bt.layer_idx, num_heads=c["hq"], num_kv_heads=c["hkv"], head_dim=c["d"],
+              **dev.layout_kwargs())
+    ws_bytes = ops.prefill_workspace_size(bt.batch, 0, bt.max_seqlen, bt.max_kvlen, c["hq"], c["hkv"], c["d"])
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev.device)
+    stream, side = torch.cuda.current_stream(), torch.cuda.Stream()
+
+    def timed(workspace):
+        def call(st):
+            ops.prefill_attention(dev.query, dev.output, dev.cache, dev.scale, dev.seqstarts, dev.kvstarts, dev.cachestarts,
+                                  workspace=workspace, stream=st, **kw)
+        call(stream)
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(steps):
+                    call(side)
+            graph.replay()
+            side.synchronize()
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(replays + 1)]
+            evs[0].record(side)
+            for r in range(replays):
+                graph.replay()
+                evs[r + 1].record(side)
+            side.synchronize()
+        return float(np.median([evs[r].elapsed_time(evs[r + 1]) * 1e3 / steps for r in range(replays)]))
+
+    tile_us = timed(None)
+    tile_out = dev.output.clone()
+    chunk_us = timed(ws) if ws_bytes else None
+    diff = float((dev.output.float() - tile_out.float()).abs().max()) if ws_bytes else None
+    cache_bytes = int(sum(int(x) for x in bt.kv_lens)) * c["hkv"] * (2 * c["d"] + c["d"] // 2)
+    print(json.dumps({
+        "metric": "prefill stage on short chunks, microseconds per call", "unit": "us", "higher_is_better": False,
+        "n_gpus": 1, "steps": steps, "data": "synthetic", "dtype": "int8 KV cache, fp16 in/out, fp32 accumulate",
+        "config": {"workload": "chunks(%s)" % spec, "sequences": c["seqs"], "query_tokens": [c["qmin"], c["qmax"]],
+                   "prior_tokens": c["prior"], "columns_per_kv_head": int(bt.max_seqlen) * (c["hq"] // c["hkv"]),
+                   "cache_bytes": cache_bytes},
+        "tile_kernel_us": tile_us, "decode_kernel_path_us": chunk_us, "value": chunk_us if chunk_us else tile_us,
+        "decode_kernel_path_gbs": cache_bytes / (chunk_us * 1e-6) / 1e9 if chunk_us else None,
+        "workspace_bytes": ws_bytes, "max_abs_difference_between_the_two": diff}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -144,6 +202,9 @@ def main():
     ap.add_argument("--custom", default="",
                     help="a decode-only batch instead of --workload, e.g. 'hq=8,hkv=1,d=128,batch=64,kvmin=1024,"
                          "kvmax=4096,mode=1' (kv lengths uniform in [kvmin, kvmax], seed 7, outlier channels)")
+    ap.add_argument("--chunks", default="",
+                    help="instead of a layer call: the prefill stage on a batch of short chunks, e.g. 'hq=32,hkv=8,d=128,"
+                         "seqs=64,qmin=2,qmax=8,prior=2048', on the tile kernel and on the decode step's kernel")
     ap.add_argument("--extras", action="store_true",
                     help="also time the kernels either side of the layer call on this batch's new tokens (RoPE alone, "
                          "RoPE fused with the append) and a 64-page kv_cache_reorder; reported under `extras`")
@@ -163,6 +224,9 @@ def main():
     wl, harness, ops = pkg.workloads, pkg.harness, pkg.ops
     torch.cuda.set_device(0)
 
+    if args.chunks:
+        chunk_bench(torch, pkg, args.chunks, args.steps, max(10, args.replays))
+        return
     if args.custom:
         c = dict(hq=32, hkv=8, d=128, batch=64, kvmin=1024, kvmax=4096, mode=1)
         c.update({k: int(v) for k, v in (kv.split("=") for kv in args.custom.split(","))})

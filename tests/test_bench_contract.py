@@ -39,3 +39,9 @@ def test_bench_line_has_the_contract_fields():
 def test_bench_custom_shape():
     d = run_bench("--custom", "hq=8,hkv=2,d=64,batch=8,kvmin=200,kvmax=400", "--steps", "3", "--warmup", "1", "--no-cpu-baseline")
     assert d["config"]["workload"].startswith("custom(") and d["roofline"]["traffic"] is None and d["value"] > 0
+
+
+def test_bench_short_chunks():
+    d = run_bench("--chunks", "hq=8,hkv=2,d=128,seqs=8,qmin=2,qmax=4,prior=700", "--steps", "3")
+    assert d["config"]["columns_per_kv_head"] == 16 and d["workspace_bytes"] > 0
+    assert d["tile_kernel_us"] > 0 and d["decode_kernel_path_us"] > 0 and d["max_abs_difference_between_the_two"] < 0.05
