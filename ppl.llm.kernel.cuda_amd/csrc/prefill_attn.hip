@@ -476,16 +476,23 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         auto softmax_max = [&](f32x16& sacc, int mb) -> float {
             float mx = kNegBig;
             if (EXTRA) {
+                // element i is token t0 + o_i, o_i = 8 (i / 4) + i % 4 a constant of the unrolled loop.  The alibi term
+                // is slope2 * (t0 + o_i) (causal) or -slope2 * |d0 - o_i| with d0 the distance of t0 from the column's
+                // own position: one multiply-add per element on a per-block base.  The limit test runs only on the
+                // tiles that reach a column's limit, as in the plain form; mask values are read below the limit only
+                // (the tile may reach beyond the mask's row).
+                const int t0 = t_base + 32 * mb + 4 * hh;
+                const float slope2 = slope * kLog2e;
+                const bool has_alibi = a.alibi_slopes != nullptr, causal = a.is_causal != 0;
+                const float base = causal ? slope2 * (float)t0 : (float)(pos_c + kvlen - qlen - t0);
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const int t = t_base + 32 * mb + 8 * (i >> 2) + 4 * hh + (i & 3);
-                    float v = -INFINITY;
-                    if (t < lim) {
-                        float add = 0.f;
-                        if (mask_row) add = (float)mask_row[t];
-                        if (a.alibi_slopes) add += a.is_causal ? slope * (float)t : -slope * fabsf((float)(pos_c + kvlen - qlen - t));
-                        v = __builtin_fmaf(sacc[i], sm_scale, add * kLog2e);
-                    }
+                    const int o = 8 * (i >> 2) + (i & 3);
+                    float add = 0.f;
+                    if (has_alibi) add = causal ? __builtin_fmaf(slope2, (float)o, base) : -slope2 * fabsf(base - (float)o);
+                    if (mask_row && t0 + o < lim) add = __builtin_fmaf((float)mask_row[t0 + o], kLog2e, add);
+                    float v = __builtin_fmaf(sacc[i], sm_scale, add);
+                    if ((limit || mask_row) && t0 + o >= lim) v = -INFINITY;
                     sacc[i] = v;
                     mx = fmaxf(mx, v);
                 }
