@@ -232,7 +232,7 @@ int pmxhip_decode_plan_make_kernel(int64_t decoding_batches, int64_t num_heads, 
         return fail(PMXHIP_UNSUPPORTED, "decode_plan: kernel %d (%s) does not serve %lld query / %lld kv heads of %lld channels",
                     kernel_request, pmxhip::decode_kernel_name(kernel_request), (long long)num_heads, (long long)num_kv_heads,
                     (long long)head_dim);
-    const int min_tokens = c.wg_tokens > 128 ? c.wg_tokens : 128;
+    const int min_tokens = pmxhip::decode_min_tokens_per_range(c.wg_tokens);
 
     int64_t ranges = num_token_ranges_hint;
     if (ranges == 0) {
@@ -333,7 +333,7 @@ int decode_prepare(const char* who, const pmxhip_decode_params* p, void* workspa
     a.q_heads_per_pass = c.q_heads_per_pass;
     a.num_passes = c.num_passes;
     a.wg_tokens = c.wg_tokens;
-    a.min_tokens_per_range = c.wg_tokens > 128 ? c.wg_tokens : 128;
+    a.min_tokens_per_range = pmxhip::decode_min_tokens_per_range(c.wg_tokens);
 
     if (a.ranges > 1) {
         const int64_t pieces = (int64_t)a.ranges + p->decoding_batches;
