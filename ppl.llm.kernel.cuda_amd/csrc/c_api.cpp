@@ -241,10 +241,21 @@ int pmxhip_decode_plan_make_kernel(int64_t decoding_batches, int64_t num_heads, 
         if (cus <= 0) return fail(PMXHIP_INVALID_VALUE, "decode_plan: compute_units not given and no current device");
         // as many ranges as fill the workgroup slots of the chip: two workgroups of four waves per CU, or as many as
         // eight waves make where a kernel with smaller workgroups serves the shape (a wave per kv head, or per two)
-        ranges = ((int64_t)cus * c.wgs_per_cu + groups - 1) / groups;
+        const int64_t slots = (int64_t)cus * c.wgs_per_cu;
+        ranges = (slots + groups - 1) / groups;
+        // A short batch: ranges of about 128 tokens (twice the smallest) where those still fill half of the slots,
+        // shorter ones -- down to the smallest -- only to get that far: a piece has a fixed cost, and an idle CU costs more.
         const int64_t max_tokens = decoding_batches * (max_kvlen > 0 ? max_kvlen : 1);
-        const int64_t useful = (max_tokens + min_tokens - 1) / min_tokens;
-        if (ranges > useful) ranges = useful;
+        const int64_t comfortable = 2 * (int64_t)min_tokens;
+        const int64_t useful = (max_tokens + comfortable - 1) / comfortable;
+        if (ranges > useful) {
+            ranges = useful;
+            const int64_t half = slots / 2 / groups > 1 ? slots / 2 / groups : 1;
+            if (ranges < half) {
+                const int64_t finest = (max_tokens + min_tokens - 1) / min_tokens;
+                ranges = half < finest ? half : finest;
+            }
+        }
         if (ranges < 1) ranges = 1;
     }
     plan->num_token_ranges = (int32_t)ranges;

@@ -228,9 +228,11 @@ enum DecodeKernel : int32_t {
     kDecodeKernelMfma32 = 4,  // decode_attn_mfma.hip: 32 query-head columns per pass, head_dim 128 or 64
 };
 // Fewest tokens a range is given: with fewer, the start of a piece (lookups, query rows, first rows of the cache) and
-// its slot in the workspace cost more than the parallelism buys.  64 against 128 measured 26.4 -> 22.1 us per layer
-// call on 32 sequences of 200-600 tokens and 19.1 -> 17.3 us for the kernel on 8 query / 1 kv head, 64 sequences of
-// 1024-4096; 32 was slower again.  Batches that fill the chip are cut by the number of workgroup slots, not by this.
+// its slot in the workspace cost more than the parallelism buys.  On batches far smaller than the chip 64 beats 128
+// (one sequence of 4096 tokens: 12.7 against 18.1 us for the kernel; 32 sequences of 200-600 tokens: 22.1 against
+// 26.4 us per layer call) and 32 is slower again; where ranges of 128 already fill half of the workgroup slots they
+// are the better cut (one sequence of 32768 tokens: 21.9 against 24.5 us), which is how the plan chooses its number
+// of ranges.  Batches that fill the chip are cut by the number of workgroup slots, not by this.
 constexpr int decode_min_tokens_per_range(int wg_tokens) { return wg_tokens > 64 ? wg_tokens : 64; }
 
 struct DecodeChoice {
