@@ -252,8 +252,15 @@ int pmxhip_decode_plan_make_kernel(int64_t decoding_batches, int64_t num_heads, 
             ranges = useful;
             const int64_t half = slots / 2 / groups > 1 ? slots / 2 / groups : 1;
             if (ranges < half) {
-                const int64_t finest = (max_tokens + min_tokens - 1) / min_tokens;
-                ranges = half < finest ? half : finest;
+                const int64_t finer = (max_tokens + min_tokens - 1) / min_tokens;
+                ranges = half < finer ? half : finer;
+            }
+            // a step of a few sequences: below a workgroup per two CUs the ranges go down to the kernel's floor
+            const int64_t sparse = cus / 2 / groups > 1 ? cus / 2 / groups : 1;
+            if (ranges < sparse) {
+                const int floor_tokens = pmxhip::decode_floor_tokens_per_range(c.wg_tokens);
+                const int64_t finest = (max_tokens + floor_tokens - 1) / floor_tokens;
+                ranges = sparse < finest ? sparse : finest;
             }
         }
         if (ranges < 1) ranges = 1;
@@ -344,7 +351,7 @@ int decode_prepare(const char* who, const pmxhip_decode_params* p, void* workspa
     a.q_heads_per_pass = c.q_heads_per_pass;
     a.num_passes = c.num_passes;
     a.wg_tokens = c.wg_tokens;
-    a.min_tokens_per_range = pmxhip::decode_min_tokens_per_range(c.wg_tokens);
+    a.min_tokens_per_range = pmxhip::decode_floor_tokens_per_range(c.wg_tokens);
 
     if (a.ranges > 1) {
         const int64_t pieces = (int64_t)a.ranges + p->decoding_batches;

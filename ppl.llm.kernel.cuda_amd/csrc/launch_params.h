@@ -234,6 +234,10 @@ enum DecodeKernel : int32_t {
 // are the better cut (one sequence of 32768 tokens: 21.9 against 24.5 us), which is how the plan chooses its number
 // of ranges.  Batches that fill the chip are cut by the number of workgroup slots, not by this.
 constexpr int decode_min_tokens_per_range(int wg_tokens) { return wg_tokens > 64 ? wg_tokens : 64; }
+// ... and the floor that the kernels apply to whatever number of ranges they are given: a step of a few sequences
+// that leaves most CUs without a workgroup is cut down to this (one sequence of 4096 tokens: 12.7 us for the kernel
+// with 64 ranges of 64 tokens, 10.2 us with 128 of 32).
+constexpr int decode_floor_tokens_per_range(int wg_tokens) { return wg_tokens > 32 ? wg_tokens : 32; }
 
 struct DecodeChoice {
     int32_t kernel;             // never kDecodeKernelAuto

@@ -141,7 +141,7 @@ def test_decode_plan(pkg, hip_lib):
     assert plan.q_heads_per_pass == 32 and plan.num_passes == 1 and plan.kv_heads_per_group == 1
     plan = pkg.ops.decode_plan(4, 48, 3, 64, 512, cus=256, kernel=pkg._lib.DECODE_KERNEL_GENERAL)  # -> two passes of 8
     assert plan.q_heads_per_pass == 8 and plan.num_passes == 2 and plan.kv_heads_per_group == 1
-    plan = pkg.ops.decode_plan(1, 8, 8, 64, 60, cus=256)    # tiny: one range, no workspace
+    plan = pkg.ops.decode_plan(1, 8, 8, 64, 30, cus=256)    # tiny: one range, no workspace
     assert plan.num_token_ranges == 1 and plan.workspace_size == 0
     plan = pkg.ops.decode_plan(4, 8, 8, 64, 512, cus=256, ranges_hint=7)
     assert plan.num_token_ranges == 7
