@@ -267,7 +267,9 @@ typedef struct pmxhip_prefill_params {
      * pmxhip_prefill_workspace_size() bytes (16-byte aligned) a batch of short chunks -- max_seqlen * (Hq / KVH)
      * <= 32, head_dim 64 or 128, no attn_mask, alibi or current_key -- runs on the decode step's MFMA kernels over
      * token ranges, with (query position, query head) pairs as its columns and the split-KV pieces in this
-     * workspace; without it, or for any other batch, the tile kernel runs.  Results are the same within the tolerance. */
+     * workspace; without it, or for any other batch, the tile kernel runs.  Results are the same within the tolerance.
+     * On that path max_seqlen must bound the query rows of every prefill sequence, as it does in the reference's
+     * call (kernel.cu:2143): rows of a sequence beyond it would not be computed. */
     void* workspace;
     int64_t workspace_size;
 } pmxhip_prefill_params;
