@@ -346,6 +346,13 @@ int decode_prepare(const char* who, const pmxhip_decode_params* p, void* workspa
                                             "most four query heads per kv head", who);
         pmxhip::decode_choose(p->head_dim, p->num_heads, p->num_kv_heads, pmxhip::kDecodeKernelGeneral, &c);
     }
+    // ... and by the cache layout: 32-bit lane offsets against a 64-bit base per wave (decode_fit_cache_strides)
+    if (!pmxhip::decode_fit_cache_strides(p->head_dim, p->num_heads, p->num_kv_heads, p->kernel_request, p->cache_stride_s,
+                                          p->cache_stride_h, &c))
+        return fail(PMXHIP_UNSUPPORTED,
+                    "%s: cache_stride_s %lld / cache_stride_h %lld: the rows of one block of %d tokens%s must lie within 2 GiB",
+                    who, (long long)p->cache_stride_s, (long long)p->cache_stride_h, c.wg_tokens,
+                    c.kernel == pmxhip::kDecodeKernelQuad ? " of the two kv heads of a wave (requested quad kernel)" : "");
     a.kernel = c.kernel;
     a.kv_heads_per_group = c.kv_heads_per_group;
     a.q_heads_per_pass = c.q_heads_per_pass;
@@ -365,11 +372,6 @@ int decode_prepare(const char* who, const pmxhip_decode_params* p, void* workspa
         a.partial_ml = reinterpret_cast<float*>(static_cast<char*>(workspace) + out_bytes);
     }
 
-    {   // per-lane cache offsets are 32-bit: (tokens of one wave block) * stride_s + (kv heads of a group) * stride_h
-        const double span = (double)c.wg_tokens * (double)p->cache_stride_s + (double)c.kv_heads_per_group * (double)p->cache_stride_h;
-        if (p->cache_stride_s < 0 || p->cache_stride_h < 0 || span >= 2147483648.0)
-            return fail(PMXHIP_UNSUPPORTED, "%s: cache_stride_s/cache_stride_h too large for 32-bit lane offsets", who);
-    }
     *out = a;
     return PMXHIP_SUCCESS;
 }
@@ -524,7 +526,7 @@ int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t str
             plan.workspace_size <= p->workspace_size && aligned16(p->cache) && !(reinterpret_cast<uintptr_t>(p->scale) & 3u) &&
             // what the decode kernels ask of the layout beyond this stage's own checks (else: the tile kernel)
             p->cache_stride_s % 16 == 0 && p->cache_stride_l % 16 == 0 && p->cache_stride_h % 16 == 0 && p->cache_stride_kv % 16 == 0 &&
-            p->cache_stride_h >= 0 && 32.0 * (double)p->cache_stride_s + 4.0 * (double)p->cache_stride_h < 2147483648.0) {
+            p->cache_stride_h >= 0 && p->cache_stride_s >= 0 && 32.0 * (double)p->cache_stride_s + 256.0 < 2147483648.0) {
             const int64_t g = p->num_heads / p->num_kv_heads;
             pmxhip_decode_params d;
             memset(&d, 0, sizeof(d));

@@ -145,9 +145,13 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
     if (r0 >= total) return;
     const int64_t r1 = (r0 + per < total) ? r0 + per : total;
 
-    const int64_t group_off = a.layer_idx * a.cache_stride_l + (int64_t)(blockIdx.y * (KPW * WP)) * a.cache_stride_h;
+    // Addressing: a 64-bit base per wave (scalar registers) that carries the layer and the wave's first kv head, and
+    // a 32-bit offset per lane: (token in block) * stride_s + (second kv head of the wave ? stride_h : 0) + channel.
+    // Only one stride_h is left in the lane offset, so a layout that keeps the heads far apart (L, KVH, S, 2, D)
+    // is addressed like any other.
+    const int64_t group_off = a.layer_idx * a.cache_stride_l + (int64_t)(blockIdx.y * (KPW * WP) + wave * KPW) * a.cache_stride_h;
     const uint32_t stride_s32 = (uint32_t)a.cache_stride_s; // the host checks that a block's span fits 32 bits
-    const uint32_t lane_base = (uint32_t)((int64_t)head_slot * a.cache_stride_h + ch0);
+    const uint32_t lane_base = (uint32_t)((int64_t)(head_slot - wave * KPW) * a.cache_stride_h + ch0);
     const char* const cache_k = (const char*)a.cache + group_off;
     const char* const cache_v = cache_k + a.cache_stride_kv;
     const char* const scale_k = (const char*)a.scale + (group_off >> 3) * 2;

@@ -106,6 +106,57 @@ bool decode_choose(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, in
     return true;
 }
 
+namespace {
+
+// Bytes that the 32-bit lane offsets of a kernel span: the tokens of one wave block times the row stride, the kv
+// heads that share a wave's 64-bit base times the head stride, and a row.
+double lane_offset_span(const DecodeChoice& c, int64_t head_dim, int64_t stride_s, int64_t stride_h)
+{
+    int64_t tokens = c.wg_tokens, heads_apart = 0;
+    switch (c.kernel) {
+        case kDecodeKernelGeneral:
+            tokens = c.wg_tokens / 4;               // a wave's block; the four waves have bases of their own
+            heads_apart = c.kv_heads_per_group - 1; // every wave spans the group's kv heads
+            break;
+        case kDecodeKernelQuad:
+            heads_apart = head_dim == 256 ? 0 : 1;  // the wave's second kv head; the first is in the wave's base
+            break;
+        default: break;                             // a wave per kv head: the head is in the base
+    }
+    return (double)tokens * (double)stride_s + (double)heads_apart * (double)stride_h + (double)head_dim;
+}
+
+} // namespace
+
+bool decode_fit_cache_strides(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, int32_t requested,
+                              int64_t stride_s, int64_t stride_h, DecodeChoice* c)
+{
+    constexpr double kLimit = 2147483648.0;
+    if (stride_s < 0 || stride_h < 0) return false;
+    if (lane_offset_span(*c, head_dim, stride_s, stride_h) < kLimit) return true;
+    if (c->kernel == kDecodeKernelGeneral) {
+        // fewer kv heads per wave (more tokens instead) until the heads' distance fits; one kv head per workgroup
+        // has no head term at all
+        while (c->kv_heads_per_group > 1) {
+            c->kv_heads_per_group /= 2;
+            c->wg_tokens = decode_wg_tokens((int)head_dim, c->kv_heads_per_group);
+            if (lane_offset_span(*c, head_dim, stride_s, stride_h) < kLimit) return true;
+        }
+        return false;
+    }
+    if (c->kernel == kDecodeKernelQuad && requested == kDecodeKernelAuto) {
+        // two kv heads further apart than a lane offset reaches: a kernel with a wave per kv head takes the step
+        DecodeChoice alt;
+        const int64_t g = num_heads / num_kv_heads;
+        const int32_t other = head_dim == 128 && g <= kDecodeMfma16Columns ? kDecodeKernelMfma16
+                              : (head_dim == 128 || head_dim == 64 ? kDecodeKernelMfma32 : kDecodeKernelGeneral);
+        if (!decode_choose(head_dim, num_heads, num_kv_heads, other, &alt)) return false;
+        *c = alt;
+        return decode_fit_cache_strides(head_dim, num_heads, num_kv_heads, other, stride_s, stride_h, c);
+    }
+    return false;
+}
+
 bool decode_quad_launch_ok(const DecodeLaunch& a)
 {
     if (a.output_stride_s % 8 != 0 || (reinterpret_cast<uintptr_t>(a.output) & 15u) != 0) return false;

@@ -250,6 +250,14 @@ struct DecodeChoice {
 // The kernel that serves a shape, and the grouping it implies.  `requested` kDecodeKernelAuto picks by shape;
 // any other value insists on that kernel and the call fails (false) when it cannot serve the shape.
 bool decode_choose(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, int32_t requested, DecodeChoice* out);
+// Makes the choice fit a cache layout: the kernels address a row as a 64-bit base per wave plus a 32-bit offset per
+// lane, and where the kv heads of a wave lie further apart than such an offset reaches (cache_stride_h of a layout
+// that keeps the heads outermost) the general kernel takes fewer kv heads per workgroup and, unless the quad kernel
+// was requested, a kernel with a wave per kv head takes its steps.  The number of ranges of a plan stays valid: it
+// does not depend on the grouping.  False: no kernel serves the strides (a block of tokens alone spans 2 GiB, or a
+// stride is negative).
+bool decode_fit_cache_strides(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, int32_t requested,
+                              int64_t stride_s, int64_t stride_h, DecodeChoice* c);
 // What the quad kernel needs of a launch beyond the C ABI's own checks: 16-byte aligned output rows and,
 // with attn_mask, one set of waves and mask offsets within 32 bits.
 bool decode_quad_launch_ok(const DecodeLaunch& a);

@@ -15,39 +15,69 @@ import numpy as np
 PAGE = 128
 
 
+LAYOUTS = ("l2shd", "sl2hd", "lhs2d")
+
+
 @dataclass
 class CacheLayout:
-    """int8 cache [L, 2, T, KVH, D] and fp16 scale [L, 2, T, KVH, D/8]."""
+    """int8 cache and fp16 scale (one scale per 8 channels: the same shape with D/8 last) in one of three orders
+    of (layer L, K/V plane 2, token S, kv head H, channel D); the operator only sees the four strides.
+
+    "l2shd"  [L, 2, S, H, D]  the order the benchmark configurations name
+    "sl2hd"  [S, L, 2, H, D]  a token's rows of every layer together
+    "lhs2d"  [L, H, S, 2, D]  a kv head's tokens together, K and V rows of a token side by side
+    (the second and third are the two the reference's header documents, multi_head_cache_attention.h:145-146)."""
     num_layer: int
     pool_tokens: int
     num_kv_heads: int
     head_dim: int
+    kind: str = "l2shd"
+
+    def _dims(self):
+        return dict(L=self.num_layer, K=2, S=self.pool_tokens, H=self.num_kv_heads, D=self.head_dim)
+
+    def _order(self):
+        return {"l2shd": "LKSHD", "sl2hd": "SLKHD", "lhs2d": "LHSKD"}[self.kind]
+
+    def _stride(self, axis):
+        dims, order = self._dims(), self._order()
+        n = 1
+        for ax in order[order.index(axis) + 1:]:
+            n *= dims[ax]
+        return n
 
     @property
     def stride_s(self):
-        return self.num_kv_heads * self.head_dim
+        return self._stride("S")
 
     @property
     def stride_h(self):
-        return self.head_dim
+        return self._stride("H")
 
     @property
     def stride_kv(self):
-        return self.pool_tokens * self.stride_s
+        return self._stride("K")
 
     @property
     def stride_l(self):
-        return 2 * self.stride_kv
+        return self._stride("L")
 
     @property
     def cache_elems(self):
-        return self.num_layer * self.stride_l
+        return self.num_layer * 2 * self.pool_tokens * self.num_kv_heads * self.head_dim
 
     def cache_shape(self):
-        return (self.num_layer, 2, self.pool_tokens, self.num_kv_heads, self.head_dim)
+        dims = self._dims()
+        return tuple(dims[ax] for ax in self._order())
 
     def scale_shape(self):
-        return (self.num_layer, 2, self.pool_tokens, self.num_kv_heads, self.head_dim // 8)
+        return self.cache_shape()[:-1] + (self.head_dim // 8,)
+
+    def canonical(self, arr):
+        """A view of a cache or scale array (numpy or torch) of this layout with its axes as [L, 2, S, H, D]."""
+        order = self._order()
+        axes = tuple(order.index(ax) for ax in "LKSHD")
+        return np.transpose(arr, axes) if isinstance(arr, np.ndarray) else arr.permute(axes)
 
 
 @dataclass
@@ -71,6 +101,7 @@ class Batch:
     start_pos: np.ndarray = field(default=None, repr=False)
     cachestarts: np.ndarray = field(default=None, repr=False)
     cachestarts_stride_b: int = 0
+    layout_kind: str = "l2shd"
     layout: CacheLayout = field(default=None, repr=False)
     outlier_channels: np.ndarray = field(default=None, repr=False)  # [KVH, n_out]
 
@@ -118,7 +149,7 @@ class Batch:
         return 4 * self.num_heads * self.head_dim * tot
 
 
-def finalize(bt: Batch, rng: np.random.Generator):
+def finalize(bt: Batch, rng: np.random.Generator, pool_tokens_at_least: int = 0):
     """Derives the index arrays and places the sequences in a token pool."""
     B = bt.batch
     bt.seqstarts = np.concatenate([[0], np.cumsum(bt.q_lens)]).astype(np.int64)
@@ -127,7 +158,7 @@ def finalize(bt: Batch, rng: np.random.Generator):
     if bt.cache_mode == 1:
         pages = (bt.kv_lens + PAGE - 1) // PAGE
         n_pages = int(pages.sum())
-        pool_pages = n_pages + 3  # a few pages nobody owns (canaries)
+        pool_pages = max(n_pages + 3, -(-pool_tokens_at_least // PAGE))  # a few pages nobody owns (canaries)
         perm = rng.permutation(pool_pages)[:n_pages]
         max_p = int(pages.max()) if B else 1
         table = np.zeros((B, max_p), dtype=np.int64)
@@ -149,8 +180,8 @@ def finalize(bt: Batch, rng: np.random.Generator):
             cur += int(bt.kv_lens[b]) + int(rng.integers(0, 4))
         bt.cachestarts = starts
         bt.cachestarts_stride_b = 1
-        pool_tokens = cur + 3
-    bt.layout = CacheLayout(bt.num_layer, int(pool_tokens), bt.num_kv_heads, bt.head_dim)
+        pool_tokens = max(cur + 3, pool_tokens_at_least)
+    bt.layout = CacheLayout(bt.num_layer, int(pool_tokens), bt.num_kv_heads, bt.head_dim, bt.layout_kind)
     n_out = int(math.ceil(0.02 * bt.head_dim)) if bt.outliers else 0
     if n_out:
         bt.outlier_channels = np.stack(
@@ -175,7 +206,7 @@ def _loguniform_int(rng, lo, hi, n):
     return np.floor(np.exp(rng.uniform(np.log(lo), np.log(hi), n))).astype(np.int64)
 
 
-def make_batch(name: str, scale: float = 1.0) -> Batch:
+def make_batch(name: str, scale: float = 1.0, layout: str = "l2shd", num_layer: int = 1) -> Batch:
     """The five benchmark configurations; `scale` < 1 shrinks sequence lengths
     (and keeps every other property) so that CPU checks finish quickly."""
     def sc(v):
@@ -213,11 +244,14 @@ def make_batch(name: str, scale: float = 1.0) -> Batch:
         bt = Batch(name, seed, 32, 8, 128, 1, 240, q_lens, kv_lens, outliers=True)
     else:
         raise KeyError(name)
+    bt.layout_kind = layout
+    bt.num_layer = num_layer
     return finalize(bt, rng), rng
 
 
 def custom_batch(seed, num_heads, num_kv_heads, head_dim, cache_mode, dec_kv_lens, prefill_q_lens=(),
-                 prefill_prior=(), outliers=False, num_layer=1, layer_idx=0, is_causal=True):
+                 prefill_prior=(), outliers=False, num_layer=1, layer_idx=0, is_causal=True, layout="l2shd",
+                 pool_tokens_at_least=0):
     """Arbitrary ragged batch for tests."""
     rng = np.random.default_rng(seed)
     dec_kv = np.asarray(dec_kv_lens, dtype=np.int64)
@@ -226,8 +260,8 @@ def custom_batch(seed, num_heads, num_kv_heads, head_dim, cache_mode, dec_kv_len
     q_lens = np.concatenate([np.ones(len(dec_kv), np.int64), pq]).astype(np.int64)
     kv_lens = np.concatenate([dec_kv, pp + pq]).astype(np.int64)
     bt = Batch("custom", seed, num_heads, num_kv_heads, head_dim, cache_mode, len(dec_kv), q_lens, kv_lens,
-               outliers=outliers, num_layer=num_layer, layer_idx=layer_idx, is_causal=is_causal)
-    return finalize(bt, rng), rng
+               outliers=outliers, num_layer=num_layer, layer_idx=layer_idx, is_causal=is_causal, layout_kind=layout)
+    return finalize(bt, rng, pool_tokens_at_least), rng
 
 
 def history_chunks(bt: Batch, rng, max_rows=1 << 16):
