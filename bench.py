@@ -17,7 +17,12 @@ reported as `us_per_layer_eager`).  `roofline` prices the dominant kernel alone 
 token-range decode kernel, named by the library) in the same regime: a graph of K launches
 of that kernel, replayed and timed the same way on the stream it is launched on; the
 figure of an event-separated launch loop is given beside it (`stages_us`).
-`cpu_baseline` is the CPU oracle on a bounded sample of the same batch.
+`cpu_baseline` is the CPU oracle (quantise/append + decode attention) on a bounded sample of the same batch.
+
+The cache has `--layers` layers (default 8) and timed call i works on layer i mod layers, as the layers of a model
+follow each other: two calls on the same layer are then separated by the cache bytes of all the other layers (gigabytes),
+so nothing of a layer's cache is left in the 256 MB memory-side cache when its turn comes again.  `same_layer` gives
+the figure of the regime in which every call re-reads one layer, for comparison.
 """
 import argparse
 import json
@@ -50,9 +55,10 @@ def read_traffic(workload, kernel):
     return None
 
 
-def cpu_baseline(oracle, bt, q, cache_host, scale_host, budget_s=2.0):
-    """The oracle's decode attention over the first sequences of the batch, sized to the time budget."""
-    lay = bt.layout
+def cpu_baseline(oracle, bt, lay, q, k, v, cache_host, scale_host, budget_s=2.0):
+    """The oracle's step -- quantise/append of the new K/V rows, then decode attention -- over the first sequences of
+    the batch (decode sequences, one new row each), sized to the time budget.  `cache_host` / `scale_host`: a cache of
+    one layer in the layout `lay`."""
     kw = dict(cache_stride_s=lay.stride_s, cache_stride_l=lay.stride_l, cache_stride_h=lay.stride_h,
               cache_stride_kv=lay.stride_kv, cachestarts_stride_b=bt.cachestarts_stride_b)
     d = bt.head_dim
@@ -60,30 +66,36 @@ def cpu_baseline(oracle, bt, q, cache_host, scale_host, budget_s=2.0):
 
     def run(nseq):
         kvstarts = bt.kvstarts[:nseq + 1]
+        rows = int(bt.seqstarts[nseq])
         t0 = time.perf_counter()
+        oracle.kv_cache_quantize(k[:rows], v[:rows], bt.seqstarts[:nseq + 1], bt.cachestarts, bt.start_pos[:nseq], 0,
+                                 bt.num_kv_heads, d, bt.page_size, cache=cache_host, scale=scale_host, **kw)
+        t1 = time.perf_counter()
         oracle.decode_attention(q, cache_host, scale_host, bt.cachestarts, kvstarts, nseq, bt.num_heads,
-                                bt.num_kv_heads, d, bt.attn_scale, bt.layer_idx, bt.page_size, **kw)
-        dt = time.perf_counter() - t0
+                                bt.num_kv_heads, d, bt.attn_scale, 0, bt.page_size, **kw)
+        t2 = time.perf_counter()
         tokens = int(bt.kv_lens[:nseq].sum())
-        return dt, tokens * per_tok + 2 * nseq * bt.num_heads * d * 2, tokens
+        return t2 - t0, t1 - t0, tokens * per_tok + 2 * nseq * bt.num_heads * d * 2, tokens
 
     n0 = max(1, min(bt.decoding_batches, 4))
-    dt, nbytes, tokens = run(n0)  # also warms the pages
+    dt, _, nbytes, tokens = run(n0)  # also warms the pages
     rate = tokens / max(dt, 1e-6)
     cum = np.cumsum(bt.kv_lens[:bt.decoding_batches])
     # as many sequences as one pass of about a second covers, then passes until the budget is spent
     nseq = int(min(bt.decoding_batches, max(n0, np.searchsorted(cum, rate * 1.0) + 1)))
-    times = []
+    times, appends = [], []
     t_all = time.perf_counter()
     while not times or (time.perf_counter() - t_all < budget_s and len(times) < 50):
-        dt, nbytes, tokens = run(nseq)
+        dt, dt_append, nbytes, tokens = run(nseq)
         times.append(dt)
+        appends.append(dt_append)
     dt = float(np.median(times))
     cores = oracle.num_threads()
     return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": "decode attention of the first %d of %d sequences (%d kv tokens): median of %d passes of %.2f s "
-                      "(%.0f core-seconds in all)" % (nseq, bt.decoding_batches, tokens, len(times), dt,
-                                                      sum(times) * cores),
+            "sample": "quantise/append of the new rows + decode attention of the first %d of %d sequences (%d kv tokens): "
+                      "median of %d passes of %.2f s, of which the append %.1f ms (%.0f core-seconds in all)" % (
+                          nseq, bt.decoding_batches, tokens, len(times), dt, float(np.median(appends)) * 1e3,
+                          sum(times) * cores),
             "us_per_layer_extrapolated": dt * 1e6 * bt.decode_kv_tokens / max(tokens, 1)}
 
 
@@ -199,6 +211,10 @@ def main():
     ap.add_argument("--eager", action="store_true", help="time host-launched kernels only (no HIP graph)")
     ap.add_argument("--ranges", type=int, default=0, help="token ranges for decode (0 = planned)")
     ap.add_argument("--replays", type=int, default=12, help="timed replays of the K-step graph (at least 10)")
+    ap.add_argument("--layers", type=int, default=8,
+                    help="layers of the cache; timed call i works on layer i mod layers (1 = every call re-reads one layer)")
+    ap.add_argument("--layout", default="l2shd", choices=["l2shd", "sl2hd", "lhs2d"],
+                    help="order of the cache tensor: (L,2,S,H,D), (S,L,2,H,D) or (L,H,S,2,D)")
     ap.add_argument("--custom", default="",
                     help="a decode-only batch instead of --workload, e.g. 'hq=8,hkv=1,d=128,batch=64,kvmin=1024,"
                          "kvmax=4096,mode=1' (kv lengths uniform in [kvmin, kvmax], seed 7, outlier channels)")
@@ -231,16 +247,31 @@ def main():
         c = dict(hq=32, hkv=8, d=128, batch=64, kvmin=1024, kvmax=4096, mode=1)
         c.update({k: int(v) for k, v in (kv.split("=") for kv in args.custom.split(","))})
         lens = np.random.default_rng(7).integers(c["kvmin"], c["kvmax"] + 1, c["batch"])
-        bt, rng = wl.custom_batch(7, c["hq"], c["hkv"], c["d"], c["mode"], lens.tolist(), outliers=True)
+        bt, rng = wl.custom_batch(7, c["hq"], c["hkv"], c["d"], c["mode"], lens.tolist(), outliers=True,
+                                  num_layer=max(1, args.layers), layout=args.layout)
         bt.name = "custom(%s)" % args.custom
     else:
-        bt, rng = wl.make_batch(args.workload)
+        bt, rng = wl.make_batch(args.workload, layout=args.layout, num_layer=max(1, args.layers))
+    n_layers = bt.num_layer
     dev = harness.DeviceBatch(bt)
-    # context already in the cache: quantised from seeded fp16 rows by the HIP append kernel
+    # context already in the cache: quantised from seeded fp16 rows by the HIP append kernel into layer 0; the other
+    # layers hold copies of it at their own addresses
     dev.fill_history(rng, max_rows=1 << 15)
+    for layer in range(1, n_layers):
+        dev.copy_layer(0, layer)
     q, k, v = wl.step_inputs(bt, rng)
     dev.set_step_inputs(q, k, v)
-    op = dev.make_operator(specify_decoding_multi_block=1)
+    layer_ops = [dev.make_operator(specify_decoding_multi_block=1, layer_idx=layer) for layer in range(n_layers)]
+    op = layer_ops[0]
+    for other in layer_ops[1:]:
+        other.set_workspace(op.workspace)
+    calls = {"n": 0}
+
+    def next_layer():
+        """Layer of the next call: 0, 1, ..., layers - 1, 0, ... in the order the calls are issued or recorded."""
+        layer = calls["n"] % n_layers
+        calls["n"] += 1
+        return layer
     if args.ranges:
         plan = ops.decode_plan(bt.decoding_batches, bt.num_heads, bt.num_kv_heads, bt.head_dim, bt.max_kvlen,
                                ranges_hint=args.ranges)
@@ -249,7 +280,7 @@ def main():
     stream = torch.cuda.current_stream()
 
     def step():
-        rc = op.forward(stream)
+        rc = layer_ops[next_layer()].forward(stream)
         if rc != 0:
             raise RuntimeError("forward() returned %d" % rc)
 
@@ -294,11 +325,15 @@ def main():
         return {"median": float(np.median(ts)), "min": float(np.min(ts)), "first": float(ts[0]), "max": float(np.max(ts))}
 
     def forward_on(st):
-        rc = op.forward(st)
+        rc = layer_ops[next_layer()].forward(st)
         if rc != 0:
             raise RuntimeError("forward() returned %d during capture" % rc)
 
-    layer_replays = kernel_replays = prefill_replays = None
+    def forward_same_layer(st):
+        if op.forward(st) != 0:
+            raise RuntimeError("forward() failed during capture")
+
+    layer_replays = kernel_replays = prefill_replays = same_layer_replays = same_kernel_replays = None
     if not args.eager:
         # The K layer calls recorded once into a HIP graph and replayed: the way a serving loop runs a decode step
         # (all layers in one graph).  Every kernel runs on every replay; the replays follow each other without a
@@ -308,10 +343,14 @@ def main():
             step_s = float(np.median(layer_replays)) * 1e-6
             launch = "HIP graph of %d layer calls, %d replays back to back, median replay" % (args.steps, replays)
             kernel_replays = replay_times(lambda st: dev.decode_only(num_token_ranges=plan.num_token_ranges, workspace=ws,
-                                                                      stage=1, stream=st))
+                                                                      stage=1, stream=st, layer_idx=next_layer()))
+            if n_layers > 1:  # the regime in which every call re-reads the same layer, for comparison
+                same_layer_replays = replay_times(forward_same_layer)
+                same_kernel_replays = replay_times(lambda st: dev.decode_only(num_token_ranges=plan.num_token_ranges,
+                                                                               workspace=ws, stage=1, stream=st, layer_idx=0))
             if bt.batch > bt.decoding_batches:
                 def prefill_on(st):
-                    if op.forward_prefill(st) != 0:
+                    if layer_ops[next_layer()].forward_prefill(st) != 0:
                         raise RuntimeError("forward_prefill() failed during capture")
                 prefill_replays = replay_times(prefill_on)
         except Exception as exc:  # the eager timing above stands
@@ -332,12 +371,13 @@ def main():
         return {"avg_us": float(np.mean(ts)), "median_us": float(ts[len(ts) // 2]), "min_us": float(ts[0])}
 
     n_ev = max(20, args.steps)
-    t_ranges = time_stage(lambda: dev.decode_only(num_token_ranges=plan.num_token_ranges, workspace=ws, stage=1), n_ev)
+    t_ranges = time_stage(lambda: dev.decode_only(num_token_ranges=plan.num_token_ranges, workspace=ws, stage=1,
+                                                  layer_idx=next_layer()), n_ev)
     t_combine = time_stage(lambda: dev.decode_only(num_token_ranges=plan.num_token_ranges, workspace=ws, stage=2), n_ev)
-    t_append = time_stage(lambda: op.forward_kvstore(stream), n_ev)
+    t_append = time_stage(lambda: layer_ops[next_layer()].forward_kvstore(stream), n_ev)
     stages = {"decode_ranges": t_ranges, "decode_combine": t_combine, "append": t_append}
     if bt.batch > bt.decoding_batches:
-        stages["prefill"] = time_stage(lambda: op.forward_prefill(stream), n_ev)
+        stages["prefill"] = time_stage(lambda: layer_ops[next_layer()].forward_prefill(stream), n_ev)
 
     # the projection behind the attention (single-rank row_parallel_linear) on this step's decode rows: a square
     # weight of (heads * head_dim)^2 halves, streamed once per call
@@ -384,12 +424,17 @@ def main():
         "dtype": "int8 cache, fp16 in/out, fp32 accumulate",
         "data": "synthetic (numpy default_rng(%d); cache filled through the HIP quantise/append kernel)" % bt.seed,
         "config": {
-            "workload": "%s: %d decode seqs, %d q / %d kv heads, D=%d, %d kv tokens (max %d), cache_mode %d%s" % (
+            "workload": "%s: %d decode seqs, %d q / %d kv heads, D=%d, %d kv tokens (max %d), cache_mode %d%s; %s" % (
                 bt.name, bt.decoding_batches, bt.num_heads, bt.num_kv_heads, bt.head_dim, bt.decode_kv_tokens,
                 bt.max_kvlen, bt.cache_mode,
                 ", + %d prefill seqs (%d query rows)" % (bt.batch - bt.decoding_batches,
                                                          int(bt.q_lens[bt.decoding_batches:].sum()))
-                if bt.batch > bt.decoding_batches else ""),
+                if bt.batch > bt.decoding_batches else "",
+                "call i on layer i mod %d of a %.1f GB cache (%s)" % (
+                    n_layers, (dev.cache.numel() + 2 * dev.scale.numel()) / 1e9, bt.layout.kind)
+                if n_layers > 1 else "every call on the one layer of the cache (%s)" % bt.layout.kind),
+            "layers": n_layers,
+            "cache_layout": bt.layout.kind,
             "algorithmic_bytes": dec_bytes,
             "token_ranges": int(plan.num_token_ranges),
             "kv_heads_per_group": int(plan.kv_heads_per_group),
@@ -415,6 +460,12 @@ def main():
             "frac_launch_loop": dec_bytes / (t_ranges["avg_us"] * 1e-6) / 1e9 / HBM_PEAK_GBS,
         },
     }
+    if same_layer_replays:
+        same_us = float(np.median(same_layer_replays))
+        same_k = float(np.mean(same_kernel_replays))
+        out["same_layer"] = {"note": "every call on layer 0 (a re-read of the same bytes may hit the memory-side cache); "
+                                     "not the headline", "us_per_layer": same_us, "value": dec_bytes / same_us / 1e3,
+                             "kernel_us": same_k, "kernel_frac": dec_bytes / same_k / 1e3 / HBM_PEAK_GBS}
     proj_us = float(np.mean(proj_replays)) if proj_replays else stages["o_proj"]["avg_us"]
     proj_bytes = hidden * hidden * 2
     out["o_proj"] = {"kernel": "wavek_linear_kernel + linear_reduce_kernel" if proj_ws_bytes else "wavek_linear_kernel", "rows": int(bt.decoding_batches), "in_features": hidden,
@@ -434,7 +485,13 @@ def main():
         out["extras"] = extras(torch, ops, dev, bt, replay_times)
     if not args.no_cpu_baseline:
         oracle = entry.load_oracle()
-        out["cpu_baseline"] = cpu_baseline(oracle, bt, q, dev.cache.cpu().numpy(), dev.scale.cpu().numpy())
+        # layer 0 as a cache of one layer in the same order of axes
+        lay, lay1 = bt.layout, wl.CacheLayout(1, bt.layout.pool_tokens, bt.num_kv_heads, bt.head_dim, bt.layout.kind)
+        cache0 = torch.empty(lay1.cache_shape(), dtype=torch.int8, device=dev.device)
+        scale0 = torch.empty(lay1.scale_shape(), dtype=torch.float16, device=dev.device)
+        lay1.canonical(cache0)[0].copy_(lay.canonical(dev.cache)[0])
+        lay1.canonical(scale0)[0].copy_(lay.canonical(dev.scale)[0])
+        out["cpu_baseline"] = cpu_baseline(oracle, bt, lay1, q, k, v, cache0.cpu().numpy(), scale0.cpu().numpy())
     print(json.dumps(out))
 
 

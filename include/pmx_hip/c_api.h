@@ -91,7 +91,19 @@ PMXHIP_API int pmxhip_kv_cache_quantize(const pmxhip_kvstore_params* p, pmxhip_s
  * split-KV partials and their combine (kernel.cu:600-678).  The split is not a
  * fixed block count: the kv tokens of all decode sequences form one stream that
  * is cut into `num_token_ranges` equal ranges, one workgroup each, and a second
- * kernel merges the pieces of every sequence that spans more than one range. */
+ * kernel merges the pieces of every sequence that spans more than one range.
+ * Zero the struct before filling it in (memset, `= {0}`): fields added behind the
+ * reference's, such as kernel_request, mean "as before" only when they are zero.
+ *
+ * Cache layout: the four strides are free (any order of layer, K/V plane, token and
+ * kv head, multiples of 16 bytes).  A kernel addresses a row as a 64-bit base per
+ * wave plus a 32-bit offset per lane, so what must lie within 2 GiB is one block of
+ * tokens of one kv head: 32 * cache_stride_s + head_dim < 2^31 always suffices
+ * (prefill: 64 * cache_stride_s + head_dim).  cache_stride_h may be anything: where
+ * two neighbouring kv heads lie 2 GiB or more apart (a (L, KVH, S, 2, D) pool of
+ * more than 2^23 tokens at head_dim 128) a kernel with a wave per kv head runs the
+ * step instead of the quad kernel, and only an explicit kernel_request for the quad
+ * kernel is refused (PMXHIP_UNSUPPORTED). */
 typedef struct pmxhip_decode_params {
     const void* query;     /* half (B_dec, Hq, D); row = sequence index */
     const void* attn_mask; /* half, optional (NULL = none) */
@@ -269,7 +281,11 @@ typedef struct pmxhip_prefill_params {
      * token ranges, with (query position, query head) pairs as its columns and the split-KV pieces in this
      * workspace; without it, or for any other batch, the tile kernel runs.  Results are the same within the tolerance.
      * On that path max_seqlen must bound the query rows of every prefill sequence, as it does in the reference's
-     * call (kernel.cu:2143): rows of a sequence beyond it would not be computed. */
+     * call (kernel.cu:2143), because the step has max_seqlen query positions per sequence.  A max_seqlen that
+     * prefill_query_rows proves too small (more rows than prefill sequences * max_seqlen) keeps the batch on the tile
+     * kernel, which walks every row whatever the hint; otherwise the rows of a sequence beyond max_seqlen are not
+     * computed and are filled with NaN, so that an understated hint shows in the output.  A layout or alignment that
+     * the decode kernels refuse also keeps the batch on the tile kernel. */
     void* workspace;
     int64_t workspace_size;
 } pmxhip_prefill_params;
@@ -466,24 +482,37 @@ PMXHIP_API int pmxhip_rope_kv_cache_quantize(const pmxhip_rope_params* rope, con
  * place.  bias may be NULL.  Strides are in halves per row.  Needs N % 16 == 0, K % 32 == 0, 16-byte aligned
  * rows of input and weight and 8-byte aligned rows of output and bias; anything else returns
  * PMXHIP_UNSUPPORTED.  The kernels of this library are written for the decode step (M up to a few hundred rows:
- * bound by streaming the K * N * 2 weight bytes).  From 384 rows on the problem is a compute-bound GEMM and goes to
- * hipBLASLt, as the reference's goes to cublasLt, if libhipblaslt.so can be loaded at that moment (dlopen; there is
- * no link-time dependency); without it, or when it declines the problem, the same kernels serve M 128 rows at a
- * time.  The first such call of a process on a device creates the library's handle and must not come under stream
- * capture (pmxhip_init makes it).
+ * bound by streaming the K * N * 2 weight bytes); they serve any M, 128 rows at a time, allocate nothing and add
+ * their partial sums in a fixed order, so a call's result does not depend on timing.
  * workspace: at decode sizes there are fewer blocks of 64 output columns than CUs, so the k range is split over
  * several workgroups whose float32 partial tiles pass through `workspace` (the role of the reference's
  * cublas_workspace argument) and are added in a fixed order by a second kernel.
  * pmxhip_row_parallel_linear_workspace_size gives the bytes that serve (M, in_features, out_features) on the
  * current device (0 = none needed); with a NULL or smaller workspace the call still computes the same function,
- * one k range per column block (slower at decode sizes).  For M from 384 rows on the figure is what the vendor
- * library is offered as its own workspace (64 MiB; it picks an algorithm that fits what it is given).  The workspace
- * needs 16-byte alignment and no clearing. */
+ * one k range per column block (slower at decode sizes).  The workspace needs 16-byte alignment and no clearing.
+ *
+ * The _ex forms take flags.  PMXHIP_LINEAR_VENDOR_GEMM: from 384 rows on (a prefill chunk's query rows: a
+ * compute-bound GEMM) the problem goes to hipBLASLt, as the reference's goes to cublasLt, if libhipblaslt.so can be
+ * loaded (dlopen; there is no link-time dependency); where it cannot, or declines the problem, and below 384 rows,
+ * this library's kernels run as without the flag.  That route is outside the rest of this header's contract: the
+ * vendor library allocates on the host (its handle per device, descriptors per call), chooses its own summation
+ * order, and is offered the caller's workspace (the _ex size query then asks for 64 MiB).  Its handle is created by
+ * pmxhip_init_vendor_gemm() or by the first flagged call on a device, which must not come under stream capture. */
+#define PMXHIP_LINEAR_VENDOR_GEMM 1
 PMXHIP_API int64_t pmxhip_row_parallel_linear_workspace_size(int64_t m, int64_t in_features, int64_t out_features);
 PMXHIP_API int pmxhip_row_parallel_linear(pmxhip_stream_t stream, const void* input, const void* weight, const void* bias,
                                           int64_t m, int64_t in_features, int64_t out_features, int64_t input_stride,
                                           int64_t weight_stride, int64_t output_stride, int64_t workspace_size,
                                           void* workspace, void* output);
+PMXHIP_API int64_t pmxhip_row_parallel_linear_workspace_size_ex(int64_t m, int64_t in_features, int64_t out_features,
+                                                                int32_t flags);
+PMXHIP_API int pmxhip_row_parallel_linear_ex(pmxhip_stream_t stream, const void* input, const void* weight, const void* bias,
+                                             int64_t m, int64_t in_features, int64_t out_features, int64_t input_stride,
+                                             int64_t weight_stride, int64_t output_stride, int64_t workspace_size,
+                                             void* workspace, void* output, int32_t flags);
+/* Loads hipBLASLt and creates its handle on the current device (PMXHIP_LINEAR_VENDOR_GEMM); PMXHIP_UNSUPPORTED when
+ * the library cannot be loaded.  Host only; allocates. */
+PMXHIP_API int pmxhip_init_vendor_gemm(void);
 
 /* One-time set-up on the current device, for callers that record their first step under stream capture: the
  * attribute calls of the kernels with large dynamic LDS (otherwise made at each kernel's first launch, which a

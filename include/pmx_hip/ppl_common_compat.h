@@ -5,7 +5,9 @@
  * include/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention.h and
  * src/ppl/kernel/llm/cuda/pmx/multi_head_cache_attention/utils.cu:68-131,269
  * touch is provided: RetCode, datatype_t, and TensorShape's GetDim /
- * GetDimCount / GetDataType / CalcElementsExcludingPadding.
+ * GetDimCount / GetDataType / CalcElementsExcludingPadding; and, for the argument list of
+ * include/ppl/kernel/llm/cuda/pmx/row_parallel_linear.h:28-46, ppl::common::NcclParam (rank, size, communicator)
+ * and the two cuBLASLt types it names as opaque stand-ins (PMX_HIP_HAVE_BLASLT_TYPES: the call site brings its own).
  * When building inside a tree that has the real ppl.common, define
  * PMX_HIP_USE_PPL_COMMON and these are taken from there instead.
  */
@@ -84,7 +86,24 @@ private:
     int64_t dims_[kMaxDims];
 };
 
+// ppl/common/cuda/nccl_utils.h: what row_parallel_linear reads of it is `size` (row_parallel_linear.cu:83)
+struct NcclParam {
+    int rank = 0;
+    int size = 1;
+    void* nccl_comm = nullptr;
+};
+
 }} // namespace ppl::common
 
 #endif // PMX_HIP_USE_PPL_COMMON
+
+/* The GEMM handle and algorithm of the reference's row_parallel_linear: this build takes and ignores them (its
+ * own kernels, or hipBLASLt through a handle of its own), so that a call site keeps its argument list. */
+#ifndef PMX_HIP_HAVE_BLASLT_TYPES
+struct pmxhip_opaque_blaslt_context;
+typedef pmxhip_opaque_blaslt_context* cublasLtHandle_t;
+struct cublasLtMatmulAlgo_t {
+    uint64_t data[8];
+};
+#endif
 #endif // PMX_HIP_PPL_COMMON_COMPAT_H_

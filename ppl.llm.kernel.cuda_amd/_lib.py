@@ -35,6 +35,7 @@ EXPORTED_SYMBOLS = (
     "pmxhip_kv_cache_reorder", "pmxhip_kv_cache_invert_reorder",
     "pmxhip_rotary_position_embedding", "pmxhip_rope_kv_cache_quantize",
     "pmxhip_row_parallel_linear", "pmxhip_row_parallel_linear_workspace_size",
+    "pmxhip_row_parallel_linear_ex", "pmxhip_row_parallel_linear_workspace_size_ex", "pmxhip_init_vendor_gemm",
 )
 
 
@@ -215,6 +216,12 @@ def lib():
     L.pmxhip_row_parallel_linear.argtypes = [c_vp] * 4 + [c_i64] * 7 + [c_vp, c_vp]
     L.pmxhip_row_parallel_linear_workspace_size.restype = c_i64
     L.pmxhip_row_parallel_linear_workspace_size.argtypes = [c_i64] * 3
+    L.pmxhip_row_parallel_linear_ex.restype = ctypes.c_int
+    L.pmxhip_row_parallel_linear_ex.argtypes = [c_vp] * 4 + [c_i64] * 7 + [c_vp, c_vp, ctypes.c_int32]
+    L.pmxhip_row_parallel_linear_workspace_size_ex.restype = c_i64
+    L.pmxhip_row_parallel_linear_workspace_size_ex.argtypes = [c_i64] * 3 + [ctypes.c_int32]
+    L.pmxhip_init_vendor_gemm.restype = ctypes.c_int
+    L.pmxhip_init_vendor_gemm.argtypes = []
     L.pmxhip_init.restype = ctypes.c_int
     L.pmxhip_init.argtypes = []
     L.pmxhip_decode_plan_make_kernel.restype = ctypes.c_int

@@ -1,6 +1,7 @@
 // Host side of the C ABI: argument checks, the split plan, and kernel launches.
 // No allocation, no synchronisation; errors are reported by return code plus a
-// thread-local message (pmxhip_last_error).
+// thread-local message (pmxhip_last_error).  The one exception is opt-in: the vendor GEMM route of
+// pmxhip_row_parallel_linear_ex (PMXHIP_LINEAR_VENDOR_GEMM), whose library allocates on the host.
 #include "pmx_hip/c_api.h"
 
 #include <hip/hip_runtime.h>
@@ -23,6 +24,7 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 namespace {
 
 thread_local char g_last_error[512] = "";
+thread_local bool g_quiet = false; // a check whose failure only selects another route: no message on stderr
 
 int fail(int code, const char* fmt, ...)
 {
@@ -30,7 +32,7 @@ int fail(int code, const char* fmt, ...)
     va_start(ap, fmt);
     vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
     va_end(ap);
-    fprintf(stderr, "[pmx_hip] error: %s\n", g_last_error);
+    if (!g_quiet) fprintf(stderr, "[pmx_hip] error: %s\n", g_last_error);
     return code;
 }
 
@@ -123,8 +125,15 @@ int pmxhip_init(void)
     void* ptr = nullptr;
     if (int rc = static_scratch("init", nullptr, &ptr)) return rc;
     (void)current_compute_units();
+    return PMXHIP_SUCCESS;
+}
+
+int pmxhip_init_vendor_gemm(void)
+{
     int device = 0;
-    if (hipGetDevice(&device) == hipSuccess) (void)pmxhip::init_linear_library(device);
+    if (hipGetDevice(&device) != hipSuccess) return fail(PMXHIP_OTHER_ERROR, "init_vendor_gemm: no current device");
+    if (!pmxhip::linear_library_available() || pmxhip::init_linear_library(device) != 0)
+        return fail(PMXHIP_UNSUPPORTED, "init_vendor_gemm: hipBLASLt could not be loaded or gave no handle");
     return PMXHIP_SUCCESS;
 }
 
@@ -376,6 +385,15 @@ int decode_prepare(const char* who, const pmxhip_decode_params* p, void* workspa
     return PMXHIP_SUCCESS;
 }
 
+int decode_prepare_quiet(const char* who, const pmxhip_decode_params* p, void* workspace, int64_t workspace_size,
+                         pmxhip::DecodeLaunch* out)
+{
+    g_quiet = true;
+    const int rc = decode_prepare(who, p, workspace, workspace_size, out);
+    g_quiet = false;
+    return rc;
+}
+
 } // namespace
 
 int pmxhip_decode_attention(const pmxhip_decode_params* p, pmxhip_stream_t stream)
@@ -408,10 +426,11 @@ int pmxhip_decode_attention_static(const pmxhip_decode_params* p, pmxhip_stream_
                         "holds %lld; use fewer token ranges or pmxhip_decode_attention with a workspace of your own",
                         need, (long long)kStaticScratchBytes);
     }
-    void* ws = nullptr;
-    if (int rc = static_scratch("decode_attention_static", stream, &ws)) return rc;
+    void* ws = nullptr; // one range: every sequence is written as final output and no piece passes through memory
+    if (p->num_token_ranges > 1)
+        if (int rc = static_scratch("decode_attention_static", stream, &ws)) return rc;
     pmxhip::DecodeLaunch a;
-    if (int rc = decode_prepare("decode_attention_static", p, ws, kStaticScratchBytes, &a)) return rc;
+    if (int rc = decode_prepare("decode_attention_static", p, ws, ws ? kStaticScratchBytes : 0, &a)) return rc;
     return launch_result("decode_attention_static", pmxhip::launch_decode(a, 0, stream));
 }
 
@@ -421,7 +440,7 @@ const char* pmxhip_decode_kernel_name(const pmxhip_decode_params* p)
     pmxhip::DecodeLaunch a;
     // the workspace plays no part in the choice; a dummy satisfies the size check
     alignas(16) static char dummy[16];
-    if (decode_prepare("decode_kernel_name", p, p->workspace ? p->workspace : dummy, INT64_MAX, &a) != PMXHIP_SUCCESS) return "";
+    if (decode_prepare_quiet("decode_kernel_name", p, p->workspace ? p->workspace : dummy, INT64_MAX, &a) != PMXHIP_SUCCESS) return "";
     return pmxhip::decode_kernel_name(a.kernel);
 }
 
@@ -517,8 +536,12 @@ int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t str
     if ((reinterpret_cast<uintptr_t>(p->output) & 7u) || p->output_stride_s % 4 != 0)
         return fail(PMXHIP_UNSUPPORTED, "prefill_attention: output must be 8-byte aligned with a row stride that is a multiple of 4");
 
-    // short chunks on the decode step's kernels, where the shape, the inputs and the caller's workspace allow
-    if (!from_current && !p->attn_mask && !p->alibi_slopes && p->workspace && aligned16(p->workspace) &&
+    // short chunks on the decode step's kernels, where the shape, the inputs and the caller's workspace allow.  That
+    // route computes max_seqlen query positions per sequence, so a max_seqlen that the row count of the prefill
+    // sequences proves too small (more rows than sequences * max_seqlen) keeps the batch on the tile kernel, which
+    // walks every row whatever the hint.
+    const bool hint_covers_rows = p->prefill_query_rows <= 0 || p->prefill_query_rows <= prefill_batches * p->max_seqlen;
+    if (!from_current && !p->attn_mask && !p->alibi_slopes && p->workspace && aligned16(p->workspace) && hint_covers_rows &&
         prefill_chunk_shape(p->max_seqlen, p->num_heads, p->num_kv_heads, p->head_dim)) {
         pmxhip_decode_plan plan;
         if (prefill_chunk_plan(prefill_batches, p->max_seqlen, p->max_kvlen, p->num_heads, p->num_kv_heads, p->head_dim, 0, &plan) ==
@@ -557,11 +580,13 @@ int pmxhip_prefill_attention(const pmxhip_prefill_params* p, pmxhip_stream_t str
             d.workspace_size = p->workspace_size;
             d.kernel_request = prefill_chunk_kernel(d.num_kv_repeats, p->head_dim);
             pmxhip::DecodeLaunch c;
-            if (int rc = decode_prepare("prefill_attention", &d, d.workspace, d.workspace_size, &c)) return rc;
-            c.seqstarts = p->seqstarts + p->decoding_batches;
-            c.chunk_q_heads = (int32_t)g;
-            c.chunk_causal = p->is_causal ? 1 : 0;
-            return launch_result("prefill_attention", pmxhip::launch_decode(c, 0, stream));
+            // what the decode kernels refuse (an alignment, a stride) the tile kernel may still serve
+            if (decode_prepare_quiet("prefill_attention", &d, d.workspace, d.workspace_size, &c) == PMXHIP_SUCCESS) {
+                c.seqstarts = p->seqstarts + p->decoding_batches;
+                c.chunk_q_heads = (int32_t)g;
+                c.chunk_causal = p->is_causal ? 1 : 0;
+                return launch_result("prefill_attention", pmxhip::launch_decode(c, 0, stream));
+            }
         }
     }
 
@@ -755,9 +780,15 @@ int pmxhip_rope_kv_cache_quantize(const pmxhip_rope_params* rope, const pmxhip_k
 
 int64_t pmxhip_row_parallel_linear_workspace_size(int64_t m, int64_t in_features, int64_t out_features)
 {
+    return pmxhip_row_parallel_linear_workspace_size_ex(m, in_features, out_features, 0);
+}
+
+int64_t pmxhip_row_parallel_linear_workspace_size_ex(int64_t m, int64_t in_features, int64_t out_features, int32_t flags)
+{
     if (m <= 0 || in_features <= 0 || out_features <= 0) return 0;
     const int64_t own = pmxhip::linear_workspace_bytes(m, out_features, in_features, current_compute_units());
-    if (m >= pmxhip::kLinearLibraryRows && pmxhip::linear_library_available() && own < pmxhip::kLinearLibraryWorkspace)
+    if ((flags & PMXHIP_LINEAR_VENDOR_GEMM) && m >= pmxhip::kLinearLibraryRows && pmxhip::linear_library_available() &&
+        own < pmxhip::kLinearLibraryWorkspace)
         return pmxhip::kLinearLibraryWorkspace;
     return own;
 }
@@ -766,6 +797,15 @@ int pmxhip_row_parallel_linear(pmxhip_stream_t stream, const void* input, const 
                                int64_t in_features, int64_t out_features, int64_t input_stride, int64_t weight_stride,
                                int64_t output_stride, int64_t workspace_size, void* workspace, void* output)
 {
+    return pmxhip_row_parallel_linear_ex(stream, input, weight, bias, m, in_features, out_features, input_stride, weight_stride,
+                                         output_stride, workspace_size, workspace, output, 0);
+}
+
+int pmxhip_row_parallel_linear_ex(pmxhip_stream_t stream, const void* input, const void* weight, const void* bias, int64_t m,
+                                  int64_t in_features, int64_t out_features, int64_t input_stride, int64_t weight_stride,
+                                  int64_t output_stride, int64_t workspace_size, void* workspace, void* output, int32_t flags)
+{
+    if (flags & ~PMXHIP_LINEAR_VENDOR_GEMM) return fail(PMXHIP_INVALID_VALUE, "row_parallel_linear: unknown flags %d", flags);
     if (m < 0 || in_features <= 0 || out_features <= 0) return fail(PMXHIP_INVALID_VALUE, "row_parallel_linear: bad sizes");
     if (m == 0) return PMXHIP_SUCCESS;
     if (!input || !weight || !output) return fail(PMXHIP_INVALID_VALUE, "row_parallel_linear: null device pointer");
@@ -788,8 +828,8 @@ int pmxhip_row_parallel_linear(pmxhip_stream_t stream, const void* input, const 
     a.input_stride = input_stride;
     a.weight_stride = weight_stride;
     a.output_stride = output_stride;
-    // many rows: a compute-bound GEMM for the vendor library, when it can be loaded and takes the problem
-    if (m >= pmxhip::kLinearLibraryRows && pmxhip::linear_library_available()) {
+    // on request, many rows: a compute-bound GEMM for the vendor library, when it can be loaded and takes the problem
+    if ((flags & PMXHIP_LINEAR_VENDOR_GEMM) && m >= pmxhip::kLinearLibraryRows && pmxhip::linear_library_available()) {
         int device = 0;
         if (hipGetDevice(&device) != hipSuccess) return fail(PMXHIP_OTHER_ERROR, "row_parallel_linear: no current device");
         const int rc = pmxhip::launch_linear_library(a, device, workspace, workspace ? workspace_size : 0, stream);

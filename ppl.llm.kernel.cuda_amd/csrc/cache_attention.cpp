@@ -559,13 +559,18 @@ ppl::common::RetCode row_parallel_linear(
     const int64_t in_features, const int64_t out_features,
     const bool input_is_parallel,
     const int64_t workspace_size, void* workspace,
-    const ppl::common::TensorShape* output_shape, void* output)
+    const ppl::common::TensorShape* output_shape, void* output,
+    const bool use_vendor_gemm)
 {
     (void)bias_shape;
     (void)output_shape;
     if (!input_is_parallel) { // row_parallel_linear.cu:46-49
         PMX_LOG_ERROR("currnetly only support parallel input");
         return ppl::common::RC_UNSUPPORTED;
+    }
+    if (!input_shape || !weight_shape) {
+        PMX_LOG_ERROR("row_parallel_linear: null shape");
+        return ppl::common::RC_INVALID_VALUE;
     }
     if (input_shape->GetDataType() != ppl::common::DATATYPE_FLOAT16 || weight_shape->GetDataType() != ppl::common::DATATYPE_FLOAT16) {
         PMX_LOG_ERROR("row_parallel_linear only supports fp16");
@@ -574,13 +579,39 @@ ppl::common::RetCode row_parallel_linear(
     // M = all dimensions of the input but the last (row_parallel_linear.cu:55)
     int64_t m = 1;
     for (uint32_t i = 0; i + 1 < input_shape->GetDimCount(); ++i) m *= input_shape->GetDim(i);
-    return to_retcode(pmxhip_row_parallel_linear(stream, input, weight, bias, m, in_features, out_features, in_features, in_features,
-                                                 out_features, workspace_size, workspace, output));
+    return to_retcode(pmxhip_row_parallel_linear_ex(stream, input, weight, bias, m, in_features, out_features, in_features, in_features,
+                                                    out_features, workspace_size, workspace, output,
+                                                    use_vendor_gemm ? PMXHIP_LINEAR_VENDOR_GEMM : 0));
 }
 
-int64_t row_parallel_linear_workspace_size(const int64_t m, const int64_t in_features, const int64_t out_features)
+ppl::common::RetCode row_parallel_linear(
+    const hipStream_t stream,
+    const cublasLtHandle_t& cublaslt_handle, const cublasLtMatmulAlgo_t* algo,
+    const ppl::common::TensorShape* input_shape, const void* input,
+    const ppl::common::TensorShape* weight_shape, const void* weight,
+    const ppl::common::TensorShape* bias_shape, const void* bias,
+    const int64_t in_features, const int64_t out_features,
+    const ppl::common::NcclParam* nccl_param, const bool input_is_parallel, void* split_buffer,
+    const int64_t cublas_workspace_size, void* cublas_workspace,
+    const ppl::common::TensorShape* output_shape, void* output,
+    const bool use_vendor_gemm)
 {
-    return pmxhip_row_parallel_linear_workspace_size(m, in_features, out_features);
+    (void)cublaslt_handle; // the GEMM runs on this library's kernels (or on a hipBLASLt handle of its own)
+    (void)algo;
+    (void)split_buffer;    // the reference's scratch for input_is_parallel = false, which it rejects as well
+    if (nccl_param && nccl_param->size > 1) { // row_parallel_linear.cu:83-97: the all-reduce over the ranks
+        PMX_LOG_ERROR("row_parallel_linear: a communicator of %d ranks; this build runs on one GPU and has no all-reduce",
+                      nccl_param->size);
+        return ppl::common::RC_UNSUPPORTED;
+    }
+    return row_parallel_linear(stream, input_shape, input, weight_shape, weight, bias_shape, bias, in_features, out_features,
+                               input_is_parallel, cublas_workspace_size, cublas_workspace, output_shape, output, use_vendor_gemm);
+}
+
+int64_t row_parallel_linear_workspace_size(const int64_t m, const int64_t in_features, const int64_t out_features,
+                                           const bool use_vendor_gemm)
+{
+    return pmxhip_row_parallel_linear_workspace_size_ex(m, in_features, out_features, use_vendor_gemm ? PMXHIP_LINEAR_VENDOR_GEMM : 0);
 }
 
 }}}}} // namespace ppl::kernel::llm::cuda::pmx

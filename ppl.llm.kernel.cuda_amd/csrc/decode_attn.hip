@@ -499,7 +499,17 @@ __global__ __launch_bounds__(64 * NW) void decode_combine_kernel(const DecodeLau
         const int gv = (int)a.num_kv_repeats, gr = a.chunk_q_heads;
         const int gq = h % gv, cpos = gq / gr;
         out_row = a.seqstarts[b];
-        if (cpos >= (int)(a.seqstarts[b + 1] - out_row)) return; // the sequence's chunk is shorter
+        const int64_t chunk_rows = a.seqstarts[b + 1] - out_row;
+        if (h == 0 && chunk_rows > gv / gr) {
+            // The caller's max_seqlen is smaller than this sequence's chunk: the step has no column for the rows
+            // beyond it.  They are filled with NaN rather than left as they were, so that the understated hint shows.
+            const int64_t row_halves = (a.num_heads / gv) * gr * D; // query heads * head_dim
+            for (int64_t r = gv / gr; r < chunk_rows; ++r) {
+                half_t* row = (half_t*)a.output + (out_row + r) * a.output_stride_s;
+                for (int64_t c = tid; c < row_halves; c += 64 * NW) row[c] = bitcast<half_t>((uint16_t)0x7E00);
+            }
+        }
+        if (cpos >= (int)chunk_rows) return; // the sequence's chunk is shorter
         out_row += cpos;
         out_head = (h / gv) * gr + (gq - cpos * gr);
     }
@@ -665,9 +675,9 @@ __global__ __launch_bounds__(64) void splitkv_combine_rows_kernel(
 // ---- host-side launchers (called from the C ABI) -------------------------------
 
 template <int D, int GT, bool PAGED, bool MASK>
-static std::atomic<int>& decode_variant_ready()
+static DeviceMask& decode_variant_ready()
 {
-    static std::atomic<int> ready{0};
+    static DeviceMask ready{0};
     return ready;
 }
 
@@ -743,7 +753,7 @@ template <int D, int GT>
 static int init_decode_dgt()
 {
     int rc = kLaunchOk;
-    auto one = [&](const void* k, std::atomic<int>& ready) {
+    auto one = [&](const void* k, DeviceMask& ready) {
         if (rc == kLaunchOk) rc = set_dynamic_lds_once(k, (int)decode_lds_bytes(D, GT), ready);
     };
     one((const void*)decode_attention_kernel<D, GT, true, true>, decode_variant_ready<D, GT, true, true>());

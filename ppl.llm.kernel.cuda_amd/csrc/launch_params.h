@@ -176,27 +176,29 @@ int launch_linear(const LinearLaunch& a, int compute_units, void* workspace, int
 int64_t linear_workspace_bytes(int64_t m, int64_t n, int64_t k, int compute_units);
 
 // The one-time hipFuncSetAttribute of a kernel whose dynamic LDS exceeds the default limit: once per kernel and
-// device (`ready` holds a bit per device, up to 32 devices in a process).  It runs before the kernel's first launch
-// on the device and never while `stream` is being captured into a graph: a caller that captures first gets
-// kLaunchNeedsWarmup and calls pmxhip_init() or one eager step before.
-inline int current_device_bit()
+// device (`ready` holds a bit per device; devices 0-63, like the other per-device caches of the library -- a
+// device beyond them is refused, not aliased).  It runs before the kernel's first launch on the device and never
+// while `stream` is being captured into a graph: a caller that captures first gets kLaunchNeedsWarmup and calls
+// pmxhip_init() or one eager step before.
+using DeviceMask = std::atomic<uint64_t>;
+inline uint64_t current_device_bit()
 {
     int device = 0;
-    if (hipGetDevice(&device) != hipSuccess) return 0;
-    return 1 << (device & 31);
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 0;
+    return uint64_t(1) << device;
 }
-inline int set_dynamic_lds_once(const void* kernel, int bytes, std::atomic<int>& ready)
+inline int set_dynamic_lds_once(const void* kernel, int bytes, DeviceMask& ready)
 {
-    const int bit = current_device_bit();
+    const uint64_t bit = current_device_bit();
     if (bit == 0) return kLaunchNoKernel;
     if (ready.load(std::memory_order_acquire) & bit) return kLaunchOk;
     if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return kLaunchNoKernel;
     ready.fetch_or(bit, std::memory_order_release);
     return kLaunchOk;
 }
-inline int ensure_dynamic_lds(const void* kernel, int bytes, hipStream_t stream, std::atomic<int>& ready)
+inline int ensure_dynamic_lds(const void* kernel, int bytes, hipStream_t stream, DeviceMask& ready)
 {
-    const int bit = current_device_bit();
+    const uint64_t bit = current_device_bit();
     if (bit != 0 && (ready.load(std::memory_order_acquire) & bit)) return kLaunchOk;
     hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(stream, &st) != hipSuccess || st != hipStreamCaptureStatusNone) {
@@ -206,8 +208,9 @@ inline int ensure_dynamic_lds(const void* kernel, int bytes, hipStream_t stream,
     return set_dynamic_lds_once(kernel, bytes, ready);
 }
 
-// Rows from which the output projection is a compute-bound GEMM and goes to the vendor library when that can be
-// loaded (linear_library.cpp); up to here this build's weight-streaming kernels are as fast or faster.
+// Rows from which the output projection is a compute-bound GEMM and, when the caller asks for it
+// (PMXHIP_LINEAR_VENDOR_GEMM), goes to the vendor library where that can be loaded (linear_library.cpp); up to here
+// this build's weight-streaming kernels are as fast or faster.
 constexpr int64_t kLinearLibraryRows = 384;
 constexpr int64_t kLinearLibraryWorkspace = 64 << 20; // what the library is offered when the caller asks how much to bring
 bool linear_library_available();

@@ -1001,9 +1001,9 @@ constexpr size_t prefill_lds_bytes()
 }
 
 template <int D, int SRC, bool EXTRA>
-static std::atomic<int>& prefill_variant_ready()
+static DeviceMask& prefill_variant_ready()
 {
-    static std::atomic<int> ready{0};
+    static DeviceMask ready{0};
     return ready;
 }
 
@@ -1050,9 +1050,9 @@ constexpr size_t prefill16_lds_bytes()
 }
 
 template <int D, int SRC, bool EXTRA>
-static std::atomic<int>& prefill16_variant_ready()
+static DeviceMask& prefill16_variant_ready()
 {
-    static std::atomic<int> ready{0};
+    static DeviceMask ready{0};
     return ready;
 }
 

@@ -75,6 +75,12 @@ class DeviceBatch:
         self.scale.copy_((torch.rand(self.scale.shape, device=self.device, generator=g) * 0.03 + 0.005).to(torch.float16))
         torch.cuda.synchronize()
 
+    def copy_layer(self, src, dst):
+        """Layer `dst` of the cache becomes a copy of layer `src` (timing runs over several layers)."""
+        lay = self.bt.layout
+        lay.canonical(self.cache)[dst].copy_(lay.canonical(self.cache)[src])
+        lay.canonical(self.scale)[dst].copy_(lay.canonical(self.scale)[src])
+
     def set_step_inputs(self, q, k, v):
         self.query = torch.from_numpy(q).to(self.device)
         self.new_key = torch.from_numpy(k).to(self.device)
@@ -109,7 +115,7 @@ class DeviceBatch:
 
     def decode_only(self, num_token_ranges=0, workspace=None, attn_mask=None, mask_stride_s=0, mask_stride_h=0,
                     output=None, stage=0, kernel=0, static_workspace=False, output_stride_s=None, name_only=False,
-                    stream=None):
+                    stream=None, layer_idx=None):
         """Decode attention through the flat C entry point (no operator object).  `kernel` requests a
         token-range kernel; `static_workspace` uses the entry point that allocates nothing; `name_only`
         launches nothing and returns the name of the kernel the call would run."""
@@ -120,7 +126,7 @@ class DeviceBatch:
             workspace = torch.empty(int(plan.workspace_size), dtype=torch.uint8, device=self.device)
         out = self.output if output is None else output
         r = ops.decode_attention(self.query, out, self.cache, self.scale, self.cachestarts, self.kvstarts,
-                                 attn_scale=bt.attn_scale, layer_idx=bt.layer_idx,
+                                 attn_scale=bt.attn_scale, layer_idx=bt.layer_idx if layer_idx is None else layer_idx,
                                  decoding_batches=bt.decoding_batches, num_heads=bt.num_heads,
                                  num_kv_heads=bt.num_kv_heads, head_dim=bt.head_dim,
                                  num_token_ranges=plan.num_token_ranges, workspace=workspace,

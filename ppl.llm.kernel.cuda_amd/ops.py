@@ -301,15 +301,26 @@ def kv_cache_invert_reorder(outer_mem, page_ids, src_stride, dst_stride, *, laye
     return rc
 
 
-def row_parallel_linear_workspace_size(m, in_features, out_features):
-    """Bytes of workspace that let row_parallel_linear split the k range over the CUs (0 = none needed)."""
-    return int(_lib.lib().pmxhip_row_parallel_linear_workspace_size(m, in_features, out_features))
+LINEAR_VENDOR_GEMM = 1  # PMXHIP_LINEAR_VENDOR_GEMM
 
 
-def row_parallel_linear(input, weight, bias, output, *, workspace=None, stream=None, check=True):
+def row_parallel_linear_workspace_size(m, in_features, out_features, vendor_gemm=False):
+    """Bytes of workspace that let row_parallel_linear split the k range over the CUs (0 = none needed); with
+    `vendor_gemm`, what the vendor library is offered from 384 rows on."""
+    return int(_lib.lib().pmxhip_row_parallel_linear_workspace_size_ex(m, in_features, out_features,
+                                                                        LINEAR_VENDOR_GEMM if vendor_gemm else 0))
+
+
+def vendor_gemm_available():
+    """True when hipBLASLt could be loaded and gave a handle on the current device (allocates; never under capture)."""
+    return _lib.lib().pmxhip_init_vendor_gemm() == RC_SUCCESS
+
+
+def row_parallel_linear(input, weight, bias, output, *, workspace=None, stream=None, check=True, vendor_gemm=False):
     """output (M, N) = input (M, K) @ weight (N, K)^T + bias (N) or None; fp16 tensors, rows contiguous along their
     last dimension (row strides may exceed the row).  The single-rank case of the reference's row_parallel_linear.
-    `workspace`: a uint8 tensor of row_parallel_linear_workspace_size bytes, or None (slower at decode sizes)."""
+    `workspace`: a uint8 tensor of row_parallel_linear_workspace_size bytes, or None (slower at decode sizes).
+    `vendor_gemm`: from 384 rows on, hand the GEMM to hipBLASLt where it loads (off: this library's kernels)."""
     n, k = int(weight.shape[0]), int(weight.shape[1])
     m = input.numel() // k  # a contiguous (B, Hq, D) attention output is the (B, Hq * D) input in place
 
@@ -319,10 +330,10 @@ def row_parallel_linear(input, weight, bias, output, *, workspace=None, stream=N
         if t.dim() != 2 or t.stride(1) != 1:
             raise ValueError("a tensor with padded rows must be 2-d with unit stride along the row")
         return int(t.stride(0))
-    rc = _lib.lib().pmxhip_row_parallel_linear(_stream(stream), _ptr(input), _ptr(weight), _ptr(bias), m, k, n,
-                                               row_stride(input, k), row_stride(weight, k), row_stride(output, n),
-                                               0 if workspace is None else workspace.numel() * workspace.element_size(),
-                                               _ptr(workspace), _ptr(output))
+    rc = _lib.lib().pmxhip_row_parallel_linear_ex(_stream(stream), _ptr(input), _ptr(weight), _ptr(bias), m, k, n,
+                                                  row_stride(input, k), row_stride(weight, k), row_stride(output, n),
+                                                  0 if workspace is None else workspace.numel() * workspace.element_size(),
+                                                  _ptr(workspace), _ptr(output), LINEAR_VENDOR_GEMM if vendor_gemm else 0)
     if check and rc != RC_SUCCESS:
         raise PmxError(rc, "row_parallel_linear")
     return rc

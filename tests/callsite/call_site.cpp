@@ -23,6 +23,11 @@ typedef ppl::common::RetCode (*reorder_fn)(hipStream_t, const void*, const void*
 typedef ppl::common::RetCode (*invert_reorder_fn)(hipStream_t, const void*, const void*, const pmx::Stride&,
                                                   const pmx::Stride&, int64_t, int64_t, int64_t, int64_t, int64_t,
                                                   int64_t, int64_t, int64_t, void*, void*);
+typedef ppl::common::RetCode (*linear_fn)(const hipStream_t, const cublasLtHandle_t&, const cublasLtMatmulAlgo_t*,
+                                          const ppl::common::TensorShape*, const void*, const ppl::common::TensorShape*,
+                                          const void*, const ppl::common::TensorShape*, const void*, const int64_t, const int64_t,
+                                          const ppl::common::NcclParam*, const bool, void*, const int64_t, void*,
+                                          const ppl::common::TensorShape*, void*, const bool);
 typedef ppl::common::RetCode (*rope_fn)(hipStream_t, const ppl::common::TensorShape*, const void*,
                                         const ppl::common::TensorShape*, const void*, const void*, const void*, const float,
                                         const int32_t, const int64_t, const int64_t, const int64_t, const int64_t,
@@ -110,6 +115,8 @@ int main()
     const reorder_fn reorder = &pmx::kv_cache_reorder;
     const invert_reorder_fn invert_reorder = &pmx::kv_cache_invert_reorder;
     const rope_fn rope = &pmx::dynamic_batching_rotary_position_embedding;
+    const linear_fn linear = &pmx::row_parallel_linear; // picks the overload with the reference's argument list
+    (void)linear;
     pmx::Stride stride = {};
     stride.p_stride_cache = 128 * 128;
     stride.p_stride_scale = 128 * 32;
@@ -134,5 +141,18 @@ int main()
                                               num_heads * head_dim, 4096, true, 0, nullptr, &no_rows, query),
            (unsigned)pmx::row_parallel_linear(stream, &no_rows, output, &weight_shape, cache, &bias_shape, nullptr,
                                               num_heads * head_dim, 4096, false, 0, nullptr, &no_rows, query));
+    // ... and with the reference's whole argument list (row_parallel_linear.h:28-46): handle, algorithm, communicator
+    // and split buffer are accepted as a call site passes them; a communicator of two ranks is refused
+    cublasLtHandle_t blas_handle = nullptr;
+    cublasLtMatmulAlgo_t algo = {};
+    ppl::common::NcclParam one_rank, two_ranks;
+    two_ranks.size = 2;
+    printf("linear_ref(no rows)=%u linear_ref(null comm)=%u linear_ref(two ranks)=%u\n",
+           (unsigned)pmx::row_parallel_linear(stream, blas_handle, &algo, &no_rows, output, &weight_shape, cache, &bias_shape, nullptr,
+                                              num_heads * head_dim, 4096, &one_rank, true, nullptr, 0, nullptr, &no_rows, query),
+           (unsigned)pmx::row_parallel_linear(stream, blas_handle, nullptr, &no_rows, output, &weight_shape, cache, &bias_shape,
+                                              nullptr, num_heads * head_dim, 4096, nullptr, true, nullptr, 0, nullptr, &no_rows, query),
+           (unsigned)pmx::row_parallel_linear(stream, blas_handle, &algo, &no_rows, output, &weight_shape, cache, &bias_shape, nullptr,
+                                              num_heads * head_dim, 4096, &two_ranks, true, nullptr, 0, nullptr, &no_rows, query));
     return 0;
 }

@@ -36,4 +36,5 @@ def test_reference_style_call_site_compiles_links_and_runs(pkg, hip_lib, tmp_pat
     assert lines[6] == "rope(empty batch)=0"
     assert lines[7] == "kvcache(empty batch)=0"
     assert lines[8] == "linear(no rows)=0 linear(not parallel)=2"
+    assert lines[9] == "linear_ref(no rows)=0 linear_ref(null comm)=0 linear_ref(two ranks)=2"
     assert out is not None

@@ -102,6 +102,44 @@ def test_prefill_short_chunks_on_the_decode_kernel(pkg, oracle, shape, q_lens, c
     assert torch.isnan(small).all()
 
 
+def test_prefill_short_chunks_with_an_understated_max_seqlen(pkg, oracle):
+    """The short-chunk route computes max_seqlen query positions per sequence.  A max_seqlen that the row count proves
+    too small keeps the batch on the tile kernel (every row right, no piece written); one that the row count cannot
+    expose leaves no row silently unwritten: the rows beyond it come back as NaN, every other row is right."""
+    hq, hkv, d = 32, 8, 128
+
+    def run(q_lens, claimed):
+        bt, dev, q, cache, scale = make_case(pkg, oracle, 377, num_heads=hq, num_kv_heads=hkv, head_dim=d, cache_mode=1,
+                                             dec_kv_lens=[33], prefill_q_lens=q_lens,
+                                             prefill_prior=[1500, 0, 900, 33, 640][:len(q_lens)], outliers=True)
+        ref = oracle_prefill(oracle, bt, q, cache, scale)
+        ws_bytes = pkg.ops.prefill_workspace_size(bt.batch, 1, claimed, bt.max_kvlen, hq, hkv, d)
+        assert ws_bytes > 0
+        ws = torch.full((ws_bytes // 4,), float("nan"), dtype=torch.float32, device="cuda")
+        dev.output.fill_(3.0)
+        pkg.ops.prefill_attention(dev.query, dev.output, dev.cache, dev.scale, dev.seqstarts, dev.kvstarts, dev.cachestarts,
+                                  attn_scale=bt.attn_scale, is_causal=True, batch=bt.batch, decoding_batches=1,
+                                  max_seqlen=claimed, max_kvlen=bt.max_kvlen, layer_idx=0, num_heads=hq, num_kv_heads=hkv,
+                                  head_dim=d, workspace=ws, **dev.layout_kwargs())
+        torch.cuda.synchronize()
+        return bt, dev.output.float().cpu().numpy(), ref, ws
+
+    # 17 rows in 4 sequences: more than 4 * 4, so the hint cannot be right -> the tile kernel
+    bt, got, ref, ws = run([4, 2, 8, 3], claimed=4)
+    assert_attention_close(got[1:], ref[1:], "tile kernel on a provably wrong hint")
+    assert torch.isnan(ws).all()
+    # 16 rows in 5 sequences: 4 per sequence is possible, but the third has 8 -> its rows 4..7 are NaN
+    bt, got, ref, ws = run([4, 2, 8, 1, 1], claimed=4)
+    assert not torch.isnan(ws).all()
+    first = int(bt.seqstarts[3])
+    lost = np.zeros(got.shape[0], dtype=bool)
+    lost[first + 4:first + 8] = True
+    lost[0] = True  # the decode sequence's row is not this stage's
+    assert np.isnan(got[first + 4:first + 8]).all()
+    assert_attention_close(got[~lost], ref[~lost], "rows within the claimed max_seqlen")
+    assert (got[0] == 3.0).all()
+
+
 def test_prefill_workspace_size_is_zero_for_other_batches(pkg, hip_lib):
     f = pkg.ops.prefill_workspace_size
     assert f(8, 2, 8, 4096, 32, 8, 128, 256) > 0            # 8 positions x 4 query heads per kv head = 32 columns

@@ -75,19 +75,19 @@ def test_c_entry_point_rejects_bad_arguments_without_launching(pkg, hip_lib):
                                    (128, 14336 // 8, 4096), (3, 4096, 32), (129, 32, 4064), (17, 64, 64), (128, 128, 3136),
                                    (300, 8192, 1024), (5, 64, 2240), (1, 64, 512), (16, 128, 1024), (17, 64, 1536), (33, 192, 2048),
                                    (65, 64, 512), (130, 192, 2048), (240, 4096, 4096),
-                                   # many rows: the compute-bound form (the vendor library where it loads)
-                                   (384, 256, 512), (1000, 512, 1024), (2500, 1024, 2048)])
-def test_hip_linear_matches_oracle(pkg, oracle, shape):
+                                   # many rows (a prefill chunk's): this library's kernels, 128 rows at a time
+                                   (384, 256, 512), (1000, 512, 1024), (2500, 1024, 2048), (640, 4096, 4096)])
+def test_hip_linear_matches_oracle(pkg, oracle, shape, vendor_gemm=False):
     import torch
     m, n, k = shape
     rng = np.random.default_rng(100 + m + n)
     a, w, b = draw(rng, m, n, k)
     da, dw, db = (torch.from_numpy(x).cuda() for x in (a, w, b))
-    ws_bytes = pkg.ops.row_parallel_linear_workspace_size(m, k, n)
+    ws_bytes = pkg.ops.row_parallel_linear_workspace_size(m, k, n, vendor_gemm=vendor_gemm)
     for bias, with_ws in ((db, True), (None, True), (db, False)):  # with the k-split's workspace and without
         out = torch.full((m, n), float("nan"), dtype=torch.float16, device="cuda")
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda") if with_ws and ws_bytes else None
-        pkg.ops.row_parallel_linear(da, dw, bias, out, workspace=ws)
+        pkg.ops.row_parallel_linear(da, dw, bias, out, workspace=ws, vendor_gemm=vendor_gemm)
         torch.cuda.synchronize()
         got = out.cpu().numpy()
         assert_close(got, a, w, b if bias is not None else None, "hip %s" % (shape,))
@@ -97,11 +97,23 @@ def test_hip_linear_matches_oracle(pkg, oracle, shape):
             ref = oracle.row_parallel_linear(a, w, b if bias is not None else None).astype(np.float64)
             mag = np.abs(a.astype(np.float64)) @ np.abs(w.astype(np.float64)).T
             assert (np.abs(got.astype(np.float64) - ref) <= 2.0 ** -10 * np.abs(ref) + 4e-6 * mag + 1e-7).all()
+    if vendor_gemm:
+        return
     # twice the same call: the partial tiles are added in a fixed order
     out2 = torch.empty_like(out)
     pkg.ops.row_parallel_linear(da, dw, db, out2)
     torch.cuda.synchronize()
     assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(384, 256, 512), (1000, 512, 1024), (2500, 1024, 2048), (200, 256, 512)])
+def test_hip_linear_vendor_gemm_on_request(pkg, oracle, shape):
+    """PMXHIP_LINEAR_VENDOR_GEMM: from 384 rows on the GEMM goes to hipBLASLt where that loads (below, and where it
+    does not, the flag changes nothing); same tolerance against the oracle."""
+    if not pkg.ops.vendor_gemm_available():
+        pytest.skip("hipBLASLt cannot be loaded on this box")
+    test_hip_linear_matches_oracle(pkg, oracle, shape, vendor_gemm=True)
 
 
 @pytest.mark.gpu
