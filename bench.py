@@ -213,6 +213,9 @@ def main():
     ap.add_argument("--replays", type=int, default=12, help="timed replays of the K-step graph (at least 10)")
     ap.add_argument("--layers", type=int, default=8,
                     help="layers of the cache; timed call i works on layer i mod layers (1 = every call re-reads one layer)")
+    ap.add_argument("--no-same-layer", action="store_true",
+                    help="skip the comparison run in which every call re-reads layer 0 (profile runs: every launch of the "
+                         "trace is then one of the rotating regime)")
     ap.add_argument("--layout", default="l2shd", choices=["l2shd", "sl2hd", "lhs2d"],
                     help="order of the cache tensor: (L,2,S,H,D), (S,L,2,H,D) or (L,H,S,2,D)")
     ap.add_argument("--custom", default="",
@@ -344,7 +347,7 @@ def main():
             launch = "HIP graph of %d layer calls, %d replays back to back, median replay" % (args.steps, replays)
             kernel_replays = replay_times(lambda st: dev.decode_only(num_token_ranges=plan.num_token_ranges, workspace=ws,
                                                                       stage=1, stream=st, layer_idx=next_layer()))
-            if n_layers > 1:  # the regime in which every call re-reads the same layer, for comparison
+            if n_layers > 1 and not args.no_same_layer:  # the regime in which every call re-reads the same layer, for comparison
                 same_layer_replays = replay_times(forward_same_layer)
                 same_kernel_replays = replay_times(lambda st: dev.decode_only(num_token_ranges=plan.num_token_ranges,
                                                                                workspace=ws, stage=1, stream=st, layer_idx=0))
