@@ -213,6 +213,9 @@ def main():
     ap.add_argument("--replays", type=int, default=12, help="timed replays of the K-step graph (at least 10)")
     ap.add_argument("--layers", type=int, default=8,
                     help="layers of the cache; timed call i works on layer i mod layers (1 = every call re-reads one layer)")
+    ap.add_argument("--two-streams", action="store_true",
+                    help="mixed steps through forward(stream, side_stream, fork, join): the decode stage on a second "
+                         "stream beside the prefill stage")
     ap.add_argument("--no-same-layer", action="store_true",
                     help="skip the comparison run in which every call re-reads layer 0 (profile runs: every launch of the "
                          "trace is then one of the rotating regime)")
@@ -327,8 +330,18 @@ def main():
     def summary(ts):
         return {"median": float(np.median(ts)), "min": float(np.min(ts)), "first": float(ts[0]), "max": float(np.max(ts))}
 
+    side2 = torch.cuda.Stream() if args.two_streams else None
+    fork_ev, join_ev = torch.cuda.Event(), torch.cuda.Event()
+    if args.two_streams:
+        fork_ev.record(stream)
+        join_ev.record(stream)
+        torch.cuda.synchronize()
+
     def forward_on(st):
-        rc = layer_ops[next_layer()].forward(st)
+        if args.two_streams:
+            rc = layer_ops[next_layer()].forward_streams(st, side2, fork_ev, join_ev)
+        else:
+            rc = layer_ops[next_layer()].forward(st)
         if rc != 0:
             raise RuntimeError("forward() returned %d during capture" % rc)
 
@@ -442,7 +455,8 @@ def main():
             "token_ranges": int(plan.num_token_ranges),
             "kv_heads_per_group": int(plan.kv_heads_per_group),
             "q_heads_per_pass": int(plan.q_heads_per_pass),
-            "step": "append + decode (token-range kernel + combine)" + (" + prefill" if "prefill" in stages else ""),
+            "step": "append + decode (token-range kernel + combine)" + (" + prefill" if "prefill" in stages else "") +
+                    (", decode on a second stream beside the prefill" if args.two_streams and "prefill" in stages else ""),
         },
         "stages_us": stages,
         "roofline": {

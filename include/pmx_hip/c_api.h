@@ -383,6 +383,14 @@ PMXHIP_API int pmxhip_mhca_forward_kvstore(pmxhip_mhca_t op, pmxhip_stream_t str
 PMXHIP_API int pmxhip_mhca_forward_decode(pmxhip_mhca_t op, pmxhip_stream_t stream);
 PMXHIP_API int pmxhip_mhca_forward_prefill(pmxhip_mhca_t op, pmxhip_stream_t stream);
 PMXHIP_API int pmxhip_mhca_forward(pmxhip_mhca_t op, pmxhip_stream_t stream);
+/* forward() of a mixed step with the decode stage on `side_stream`, beside the prefill stage on `stream` (they are
+ * independent once the append has run): forked behind the append with `fork_event`, joined into `stream` with
+ * `join_event` before the call returns.  No counterpart in the reference (multi_head_cache_attention.h:152-158 runs
+ * the stages in one stream order).  Streams and events (hipEvent_t) are the caller's, of the default priority; the
+ * library creates none, so the call can be captured from `stream`.  Steps that are not mixed, and steps whose two
+ * attention stages share the workspace (short prefill chunks on the decode kernels), run as pmxhip_mhca_forward. */
+PMXHIP_API int pmxhip_mhca_forward_streams(pmxhip_mhca_t op, pmxhip_stream_t stream, pmxhip_stream_t side_stream,
+                                           void* fork_event, void* join_event);
 
 /* ---- key_value_cache -------------------------------------------------------
  * The append step under the operator name the serving stack uses for it

@@ -109,6 +109,18 @@ public:
     ppl::common::RetCode forward_decode(const hipStream_t stream);
     ppl::common::RetCode forward_prefill(const hipStream_t stream);
     ppl::common::RetCode forward(const hipStream_t stream);
+    // forward() of a mixed step with its two attention stages side by side (no counterpart in the reference, whose
+    // forward runs the three stages in one stream order, kernel.cu:2219-2240): once the new rows are in the cache
+    // the decode stage and the prefill stage touch disjoint sequences and output rows, so the decode stage goes to
+    // `side_stream` -- forked from `stream` behind the append with `fork_event`, joined back into `stream` with
+    // `join_event` -- and its workgroups fill the compute units that the prefill kernel's tail leaves idle.  Streams
+    // and events are the caller's (both streams of the default priority; the events may be created without
+    // timing); the library creates nothing, so the call can be recorded into a HIP graph from `stream`.  When the
+    // call returns, everything it enqueued is ordered before later work on `stream`.  A step that is not mixed, a
+    // side stream equal to `stream`, and a step whose prefill stage shares the workspace with the decode stage
+    // (short chunks on the decode kernels) run exactly like forward(stream).
+    ppl::common::RetCode forward(const hipStream_t stream, const hipStream_t side_stream, const hipEvent_t fork_event,
+                                 const hipEvent_t join_event);
 };
 
 }}}}} // namespace ppl::kernel::llm::cuda::pmx

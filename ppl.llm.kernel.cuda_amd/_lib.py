@@ -31,7 +31,7 @@ EXPORTED_SYMBOLS = (
     "pmxhip_mhca_create", "pmxhip_mhca_destroy", "pmxhip_mhca_heuristic_prepare",
     "pmxhip_mhca_get_derived", "pmxhip_mhca_set_workspace",
     "pmxhip_mhca_forward_kvstore", "pmxhip_mhca_forward_decode", "pmxhip_mhca_forward_prefill",
-    "pmxhip_mhca_forward",
+    "pmxhip_mhca_forward", "pmxhip_mhca_forward_streams",
     "pmxhip_kv_cache_reorder", "pmxhip_kv_cache_invert_reorder",
     "pmxhip_rotary_position_embedding", "pmxhip_rope_kv_cache_quantize",
     "pmxhip_row_parallel_linear", "pmxhip_row_parallel_linear_workspace_size",
@@ -255,6 +255,8 @@ def lib():
         fn = getattr(L, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [c_vp, c_vp]
+    L.pmxhip_mhca_forward_streams.restype = ctypes.c_int
+    L.pmxhip_mhca_forward_streams.argtypes = [c_vp] * 5
     _lib = L
     return L
 

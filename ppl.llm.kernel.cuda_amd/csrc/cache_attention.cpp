@@ -368,6 +368,44 @@ ppl::common::RetCode dynamic_batching_multi_head_cache_attention::forward(const 
     return ret;
 }
 
+ppl::common::RetCode dynamic_batching_multi_head_cache_attention::forward(const hipStream_t stream, const hipStream_t side_stream,
+                                                                          const hipEvent_t fork_event, const hipEvent_t join_event)
+{
+    // the prefill stage on the short-chunk route writes its pieces into the workspace that the decode stage is using
+    const bool shared_workspace =
+        cfg.workspace != nullptr && cfg.decoding_multi_block_size > 1 && cfg.enable_cache_prefill && !cfg.attn_mask && !cfg.alibi_slopes &&
+        pmxhip_prefill_workspace_size(cfg.batch, cfg.decoding_batches, cfg.max_seqlen, cfg.max_kvlen, cfg.num_heads, cfg.num_kv_heads,
+                                      cfg.head_dim, cfg.device_prop ? cfg.device_prop->multiProcessorCount : 0) > 0;
+    if (cfg.decoding_batches <= 0 || cfg.prefill_batches <= 0 || side_stream == stream || shared_workspace) return forward(stream);
+    if (!fork_event || !join_event) {
+        PMX_LOG_ERROR("forward on two streams needs a fork and a join event");
+        return ppl::common::RC_INVALID_VALUE;
+    }
+    ppl::common::RetCode ret = forward_kvstore(stream);
+    if (ret != ppl::common::RC_SUCCESS) {
+        PMX_LOG_ERROR("kv_store stage failed.");
+        return ret;
+    }
+    if (hipEventRecord(fork_event, stream) != hipSuccess || hipStreamWaitEvent(side_stream, fork_event, 0) != hipSuccess) {
+        PMX_LOG_ERROR("forward on two streams: the fork failed: %s", hipGetErrorString(hipGetLastError()));
+        return ppl::common::RC_OTHER_ERROR;
+    }
+    // from here the side stream is part of the step (and of a capture): it is joined whatever the stages return
+    const ppl::common::RetCode ret_decode = forward_decode(side_stream);
+    const bool joined_side = hipEventRecord(join_event, side_stream) == hipSuccess;
+    const ppl::common::RetCode ret_prefill = forward_prefill(stream);
+    if (!joined_side || hipStreamWaitEvent(stream, join_event, 0) != hipSuccess) {
+        PMX_LOG_ERROR("forward on two streams: the join failed: %s", hipGetErrorString(hipGetLastError()));
+        return ppl::common::RC_OTHER_ERROR;
+    }
+    if (ret_decode != ppl::common::RC_SUCCESS) {
+        PMX_LOG_ERROR("decode stage failed.");
+        return ret_decode;
+    }
+    if (ret_prefill != ppl::common::RC_SUCCESS) PMX_LOG_ERROR("prefill stage failed.");
+    return ret_prefill;
+}
+
 ppl::common::RetCode dynamic_batching_key_value_cache(
     const hipStream_t stream,
     const ppl::common::TensorShape* current_key_shape, const void* current_key,
@@ -726,6 +764,13 @@ int pmxhip_mhca_forward(pmxhip_mhca_t h, pmxhip_stream_t stream)
 {
     if (!h || !h->prepared) return PMXHIP_INVALID_VALUE;
     return (int)h->op.forward(stream);
+}
+
+int pmxhip_mhca_forward_streams(pmxhip_mhca_t h, pmxhip_stream_t stream, pmxhip_stream_t side_stream, void* fork_event,
+                                void* join_event)
+{
+    if (!h || !h->prepared) return PMXHIP_INVALID_VALUE;
+    return (int)h->op.forward(stream, side_stream, static_cast<hipEvent_t>(fork_event), static_cast<hipEvent_t>(join_event));
 }
 
 } // extern "C"

@@ -444,3 +444,10 @@ class DynamicBatchingMultiHeadCacheAttention:
 
     def forward(self, stream=None):
         return _lib.lib().pmxhip_mhca_forward(self._h, _stream(stream))
+
+    def forward_streams(self, stream, side_stream, fork_event, join_event):
+        """forward() of a mixed step with the decode stage on `side_stream` beside the prefill stage on `stream`;
+        the two torch.cuda.Event objects are the fork and the join (recorded once before, so that they exist)."""
+        return _lib.lib().pmxhip_mhca_forward_streams(self._h, _stream(stream), _stream(side_stream),
+                                                      ctypes.c_void_p(fork_event.cuda_event),
+                                                      ctypes.c_void_p(join_event.cuda_event))

@@ -132,6 +132,51 @@ def test_forward_in_a_hip_graph(pkg, oracle, q_lens, prior):
     assert_attention_close(eager.float().cpu().numpy(), ref, "eager rows")
 
 
+@pytest.mark.parametrize("q_lens,prior", [([70, 300], [300, 0]), ([4, 7, 1], [1300, 40, 2000])])
+def test_forward_on_two_streams(pkg, oracle, q_lens, prior):
+    """forward(stream, side_stream, fork, join): the decode stage beside the prefill stage.  Same kernels on the same
+    inputs as forward(stream), so the rows are equal bit for bit -- launched from the host and replayed from a HIP
+    graph captured from the main stream -- and the step is ordered before later work on the main stream.  The batch
+    of short chunks shares its workspace between the stages and runs in one stream order."""
+    bt, rng = pkg.workloads.custom_batch(406, num_heads=32, num_kv_heads=8, head_dim=128, cache_mode=1,
+                                         dec_kv_lens=[700, 2, 1900, 130, 1, 3000], prefill_q_lens=q_lens, prefill_prior=prior,
+                                         outliers=True)
+    cache, scale = host_cache(bt)
+    dev = pkg.harness.DeviceBatch(bt)
+    for b, pos, k_rows, v_rows in oracle_fill_history(oracle, pkg, bt, rng, cache, scale):
+        dev.append_rows(b, pos, k_rows, v_rows)
+    q, k, v = pkg.workloads.step_inputs(bt, rng)
+    dev.set_step_inputs(q, k, v)
+    op = dev.make_operator(specify_decoding_multi_block=1)
+    main, side = torch.cuda.Stream(), torch.cuda.Stream()
+    fork, join = torch.cuda.Event(), torch.cuda.Event()
+    fork.record(main)
+    join.record(main)
+    main.synchronize()
+    with torch.cuda.stream(main):
+        assert op.forward(main) == 0
+        main.synchronize()
+        one_stream = dev.output.clone()
+        dev.output.fill_(float("nan"))
+        assert op.forward_streams(main, side, fork, join) == 0
+        after = dev.output.clone()  # ordered behind the join on the main stream
+        main.synchronize()
+        assert torch.equal(after.view(torch.int16), one_stream.view(torch.int16))
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=main):
+            assert op.forward_streams(main, side, fork, join) == 0
+            assert op.forward_streams(main, side, fork, join) == 0
+        for rep in range(3):
+            dev.output.fill_(float("nan"))
+            graph.replay()
+            main.synchronize()
+            assert torch.equal(dev.output.view(torch.int16), one_stream.view(torch.int16)), "replay %d" % rep
+    oracle_append_step(oracle, bt, k, v, cache, scale)
+    ref = oracle_prefill(oracle, bt, q, cache, scale)
+    ref[:bt.decoding_batches] = oracle_decode(oracle, bt, q, cache, scale)
+    assert_attention_close(one_stream.float().cpu().numpy(), ref, "rows")
+
+
 def test_first_step_under_capture():
     """In a fresh process: a first forward() under stream capture is refused with a message that names
     pmxhip_init(), and after that call the capture succeeds (tests/capture_first_child.py)."""
