@@ -223,7 +223,7 @@ def main():
                     help="order of the cache tensor: (L,2,S,H,D), (S,L,2,H,D) or (L,H,S,2,D)")
     ap.add_argument("--custom", default="",
                     help="a decode-only batch instead of --workload, e.g. 'hq=8,hkv=1,d=128,batch=64,kvmin=1024,"
-                         "kvmax=4096,mode=1' (kv lengths uniform in [kvmin, kvmax], seed 7, outlier channels)")
+                         "kvmax=4096,mode=1,layout=lhs2d' (kv lengths uniform in [kvmin, kvmax], seed 7, outlier channels)")
     ap.add_argument("--chunks", default="",
                     help="instead of a layer call: the prefill stage on a batch of short chunks, e.g. 'hq=32,hkv=8,d=128,"
                          "seqs=64,qmin=2,qmax=8,prior=2048', on the tile kernel and on the decode step's kernel")
@@ -250,11 +250,11 @@ def main():
         chunk_bench(torch, pkg, args.chunks, args.steps, max(10, args.replays))
         return
     if args.custom:
-        c = dict(hq=32, hkv=8, d=128, batch=64, kvmin=1024, kvmax=4096, mode=1)
-        c.update({k: int(v) for k, v in (kv.split("=") for kv in args.custom.split(","))})
+        c = dict(hq=32, hkv=8, d=128, batch=64, kvmin=1024, kvmax=4096, mode=1, layout=args.layout)
+        c.update({k: (v if k == "layout" else int(v)) for k, v in (kv.split("=") for kv in args.custom.split(","))})
         lens = np.random.default_rng(7).integers(c["kvmin"], c["kvmax"] + 1, c["batch"])
         bt, rng = wl.custom_batch(7, c["hq"], c["hkv"], c["d"], c["mode"], lens.tolist(), outliers=True,
-                                  num_layer=max(1, args.layers), layout=args.layout)
+                                  num_layer=max(1, args.layers), layout=c["layout"])
         bt.name = "custom(%s)" % args.custom
     else:
         bt, rng = wl.make_batch(args.workload, layout=args.layout, num_layer=max(1, args.layers))
