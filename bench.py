@@ -143,6 +143,63 @@ def extras(torch, ops, dev, bt, replay_times):
     return res
 
 
+def rope_sweep_bench(torch, pkg, steps, replays):
+    """--rope-sweep: RoPE followed by the quantise/append as two kernels against the fused kernel, by the number of
+    new tokens of a step (32 query / 8 kv heads of 128; 128 sequences of one token, then 16 sequences of equal length).
+    A graph of `steps` calls replayed `replays` times back to back, median replay."""
+    wl, harness, ops = pkg.workloads, pkg.harness, pkg.ops
+    hq, hkv, d = 32, 8, 128
+    side = torch.cuda.Stream()
+
+    def timed(call):
+        call(torch.cuda.current_stream())
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(steps):
+                    call(side)
+            graph.replay()
+            side.synchronize()
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(replays + 1)]
+            evs[0].record(side)
+            for r in range(replays):
+                graph.replay()
+                evs[r + 1].record(side)
+            side.synchronize()
+        return float(np.median([evs[r].elapsed_time(evs[r + 1]) * 1e3 / steps for r in range(replays)]))
+
+    rows = []
+    for n_tok, nseq in ((128, 128), (512, 16), (1024, 16), (2048, 16), (4096, 16), (8192, 16), (16384, 16)):
+        bt, rng = wl.custom_batch(3, hq, hkv, d, 1, [], prefill_q_lens=[n_tok // nseq] * nseq, prefill_prior=[64] * nseq)
+        dev = harness.DeviceBatch(bt)
+        q, k, v = wl.step_inputs(bt, rng)
+        dev.set_step_inputs(q, k, v)
+        lk = dev.layout_kwargs()
+        kw = dict(theta=10000.0, rotary_dim=d, batch=bt.batch, max_seqlen=bt.max_seqlen)
+        rq, rk = torch.empty_like(dev.query), torch.empty_like(dev.new_key)
+
+        def rope(st):
+            ops.rotary_position_embedding(dev.query, dev.new_key, dev.start_pos, dev.seqstarts, rq, rk, stream=st, **kw)
+
+        def append(st):
+            ops.key_value_cache(rk, dev.new_value, dev.seqstarts, dev.cachestarts, dev.start_pos, dev.cache, dev.scale,
+                                batch=bt.batch, max_seqlen=bt.max_seqlen, num_layer=1, layer_idx=0, num_kv_heads=hkv,
+                                head_dim=d, stream=st, **lk)
+
+        def fused(st):
+            ops.rope_key_value_cache(dev.query, dev.new_key, dev.new_value, dev.start_pos, dev.seqstarts, dev.cachestarts,
+                                     rq, rk, dev.cache, dev.scale, num_layer=1, layer_idx=0, stream=st, **lk, **kw)
+
+        rows.append({"new_tokens": n_tok, "sequences": nseq, "rope_us": timed(rope), "append_us": timed(append),
+                     "two_kernels_us": timed(lambda st: (rope(st), append(st))), "fused_us": timed(fused)})
+    print(json.dumps({
+        "metric": "RoPE + quantise/append of a step's new rows, microseconds per call", "unit": "us",
+        "higher_is_better": False, "n_gpus": 1, "steps": steps, "data": "synthetic",
+        "dtype": "fp16 rows, int8 cache", "config": {"workload": "rope-sweep: 32 q / 8 kv heads of 128"},
+        "value": rows[0]["fused_us"], "sweep": rows}))
+
+
 def chunk_bench(torch, pkg, spec, steps, replays):
     """--chunks: the prefill stage on a batch of short chunks (a few query tokens per sequence over a long history, no
     decode sequences), once on the tile kernel (no workspace) and once with the workspace that routes it to the decode
@@ -230,6 +287,8 @@ def main():
     ap.add_argument("--extras", action="store_true",
                     help="also time the kernels either side of the layer call on this batch's new tokens (RoPE alone, "
                          "RoPE fused with the append) and a 64-page kv_cache_reorder; reported under `extras`")
+    ap.add_argument("--rope-sweep", action="store_true",
+                    help="instead of a layer call: RoPE + append as two kernels against the fused kernel, by new tokens")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (known traffic, for scaling rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -248,6 +307,9 @@ def main():
 
     if args.chunks:
         chunk_bench(torch, pkg, args.chunks, args.steps, max(10, args.replays))
+        return
+    if args.rope_sweep:
+        rope_sweep_bench(torch, pkg, args.steps, max(10, args.replays))
         return
     if args.custom:
         c = dict(hq=32, hkv=8, d=128, batch=64, kvmin=1024, kvmax=4096, mode=1, layout=args.layout)

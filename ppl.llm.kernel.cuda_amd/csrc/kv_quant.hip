@@ -121,6 +121,21 @@ __device__ __forceinline__ int sequence_of(PTR starts, int n, int64_t v)
     return lo;
 }
 
+// The same index found by the wave's lanes together: the number of sequences that end at or before v (every lane
+// of the wave must be here, with the same v).  Each lane compares one entry per 64, all requested at once: one
+// memory latency where the bisection has log2(n) of them in a row.
+constexpr int kCountedSequences = 1024;
+__device__ __forceinline__ int sequence_by_count(const int64_t* starts, int n, int64_t v, int lane)
+{
+    int count = 0;
+    for (int i0 = 0; i0 < n; i0 += kWave) {
+        const int i = i0 + lane;
+        const bool ends_before = i < n && starts[i + 1] <= v;
+        count += __builtin_popcountll(__builtin_amdgcn_ballot_w64(ends_before));
+    }
+    return count < n ? count : n - 1;
+}
+
 } // namespace
 
 // stride_tokens: tokens between a thread's units, (workgroups * threads) / groups_per_token; the host sizes the launch
@@ -241,44 +256,61 @@ __global__ __launch_bounds__(kQuantThreads) void rope_append_kernel(const RopeLa
         return *(const u32x4*)((const half_t*)a.value + r.in_tok * a.value_stride_s + r.idx);
     };
 
-    // A decode step has a token per workgroup and a few units per thread: the kernel's time is then a chain of
-    // latencies (index arrays -> cos/sin -> rows -> stores).  The rows depend on none of the rest, so they are
-    // requested first and travel while the coefficients are computed.
+    // The rows depend on nothing that follows (index arrays -> sequence -> cos/sin and cache row), so a thread's
+    // first units are requested before all that and travel meanwhile; a decode step, with a token per workgroup
+    // and a few units per thread, has no others.
     constexpr int kEarly = 3;
-    const bool early = work <= kEarly * kQuantThreads;
     u32x4 early_row[kEarly], early_value[kEarly];
-    if (early) {
 #pragma unroll
-        for (int j = 0; j < kEarly; ++j) {
-            const int w = threadIdx.x + j * kQuantThreads;
-            early_row[j] = u32x4{0, 0, 0, 0};
-            early_value[j] = u32x4{0, 0, 0, 0};
-            if (w < work) {
-                const Unit r = unit_of(w);
-                early_row[j] = load_row(r);
-                if (append && !r.is_query) early_value[j] = load_value(r);
-            }
+    for (int j = 0; j < kEarly; ++j) {
+        const int w = threadIdx.x + j * kQuantThreads;
+        early_row[j] = u32x4{0, 0, 0, 0};
+        early_value[j] = u32x4{0, 0, 0, 0};
+        if (w < work) {
+            const Unit r = unit_of(w);
+            early_row[j] = load_row(r);
+            if (append && !r.is_query) early_value[j] = load_value(r);
         }
     }
 
     {
         const int tl = threadIdx.x / pairs, i = threadIdx.x - tl * pairs;
         const int64_t tok = tok0 + tl;
-        if (tl < tokens_per_wg && tok < n_tokens) {
-            const int64_t in_tok = first + tok;
-            // one new token per sequence (a decode step): token i belongs to sequence i, which two independent loads
-            // confirm; otherwise bisection, a chain of dependent loads
-            int b;
-            int64_t pos;
+        const bool active = tl < tokens_per_wg && tok < n_tokens;
+        const int64_t in_tok = first + tok;
+        // The token's sequence.  One new token per sequence (a decode step): token i belongs to sequence i, which two
+        // independent loads confirm.  Otherwise the lanes of the wave count, for each token the wave covers, the
+        // sequences that end before it (one latency); beyond kCountedSequences sequences every thread bisects (a
+        // chain of dependent loads).
+        int b = -1;
+        int64_t pos = 0;
+        const bool count_search = a.batch <= kCountedSequences;
+        if (active && (n_tokens == a.batch || !count_search)) {
             const int64_t ti = tok < a.batch ? tok : 0;
             const int64_t s0 = a.seqstarts[ti], s1 = a.seqstarts[ti + 1], sp = a.start_pos[ti];
             if (tok < a.batch && s0 == in_tok && s1 > in_tok) {
                 b = (int)tok;
                 pos = sp;
-            } else {
-                b = sequence_of(a.seqstarts, (int)a.batch, in_tok);
-                pos = a.start_pos[b] + (in_tok - a.seqstarts[b]);
             }
+        }
+        if (count_search) { // every lane of the wave is here
+            const int wave0 = threadIdx.x & ~(kWave - 1);
+            const int tl_hi = (wave0 + kWave - 1) / pairs;
+            for (int t = wave0 / pairs; t <= tl_hi; ++t) {
+                const int64_t tk = tok0 + t;
+                if (t >= tokens_per_wg || tk >= n_tokens) break;
+                if (__builtin_amdgcn_ballot_w64(tl == t && b < 0) == 0) continue;
+                const int bt = sequence_by_count(a.seqstarts, (int)a.batch, first + tk, threadIdx.x & (kWave - 1));
+                if (tl == t && b < 0) {
+                    b = bt;
+                    pos = a.start_pos[bt] + (first + tk - a.seqstarts[bt]);
+                }
+            }
+        } else if (active && b < 0) {
+            b = sequence_of(a.seqstarts, (int)a.batch, in_tok);
+            pos = a.start_pos[b] + (in_tok - a.seqstarts[b]);
+        }
+        if (active) {
             float c = 1.f, s = 0.f;
             if (i < rd2) {
                 float th = a.theta;
@@ -344,15 +376,12 @@ __global__ __launch_bounds__(kQuantThreads) void rope_append_kernel(const RopeLa
         }
     };
 
-    if (early) {
 #pragma unroll
-        for (int j = 0; j < kEarly; ++j) {
-            const int w = threadIdx.x + j * kQuantThreads;
-            if (w < work) finish(unit_of(w), early_row[j], early_value[j]);
-        }
-        return;
+    for (int j = 0; j < kEarly; ++j) {
+        const int w = threadIdx.x + j * kQuantThreads;
+        if (w < work) finish(unit_of(w), early_row[j], early_value[j]);
     }
-    for (int w = threadIdx.x; w < work; w += kQuantThreads) {
+    for (int w = threadIdx.x + kEarly * kQuantThreads; w < work; w += kQuantThreads) {
         const Unit r = unit_of(w);
         const u32x4 raw = load_row(r);
         u32x4 vraw = {0, 0, 0, 0};

@@ -111,3 +111,42 @@ def test_gpu_rope_and_fused_append_match_oracle(pkg, oracle, shape, rotary_dim, 
     pkg.ops.rotary_position_embedding(dev.query, dev.new_key, dev.start_pos, dev.seqstarts, dev.query, dev.new_key, **kw)
     torch.cuda.synchronize()
     np.testing.assert_array_equal(dev.query.cpu().numpy().view(np.uint16), rq_ref.view(np.uint16))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(8, 2, 128), (4, 4, 64), (2, 1, 256), (6, 2, 96)])
+@pytest.mark.parametrize("n_dec,n_prefill", [(100, 50), (0, 130), (1000, 100)])
+def test_gpu_rope_many_sequences(pkg, oracle, shape, n_dec, n_prefill):
+    """Batches of 130 to 1100 sequences, single-token and short multi-token ones mixed: a token's sequence is counted by
+    the lanes of a wave (several entries per lane; one, two or four tokens per wave by head_dim) or, beyond 1024
+    sequences, found by bisection.  RoPE alone and fused with the append, bit for bit against the oracle."""
+    import torch
+    hq, hk, d = shape
+    r = np.random.default_rng(n_dec + n_prefill + d)
+    bt, rng = pkg.workloads.custom_batch(77 + d, num_heads=hq, num_kv_heads=hk, head_dim=d, cache_mode=1,
+                                         dec_kv_lens=r.integers(1, 200, n_dec).tolist(),
+                                         prefill_q_lens=r.integers(1, 6, n_prefill).tolist(),
+                                         prefill_prior=r.integers(0, 300, n_prefill).tolist())
+    dev = pkg.harness.DeviceBatch(bt)
+    q, k, v = pkg.workloads.step_inputs(bt, rng)
+    dev.set_step_inputs(q, k, v)
+    kw = dict(theta=10000.0, rotary_dim=d, batch=bt.batch, max_seqlen=bt.max_seqlen)
+    rq_ref, rk_ref = oracle.rotary_position_embedding(q, k, bt.start_pos, bt.seqstarts, 10000.0, d)
+    cache_ref, scale_ref = host_cache(bt)
+    oracle.kv_cache_quantize(rk_ref, v, bt.seqstarts, bt.cachestarts, bt.start_pos, bt.layer_idx, bt.num_kv_heads,
+                             bt.head_dim, bt.page_size, cache=cache_ref, scale=scale_ref, **oracle_layout_kwargs(bt))
+    d_rq, d_rk = torch.empty_like(dev.query), torch.empty_like(dev.new_key)
+    pkg.ops.rotary_position_embedding(dev.query, dev.new_key, dev.start_pos, dev.seqstarts, d_rq, d_rk, **kw)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(d_rq.cpu().numpy().view(np.uint16), rq_ref.view(np.uint16))
+    np.testing.assert_array_equal(d_rk.cpu().numpy().view(np.uint16), rk_ref.view(np.uint16))
+    d_rq.zero_()
+    d_rk.zero_()
+    pkg.ops.rope_key_value_cache(dev.query, dev.new_key, dev.new_value, dev.start_pos, dev.seqstarts, dev.cachestarts,
+                                 d_rq, d_rk, dev.cache, dev.scale, num_layer=bt.num_layer, layer_idx=bt.layer_idx,
+                                 **dev.layout_kwargs(), **kw)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(d_rq.cpu().numpy().view(np.uint16), rq_ref.view(np.uint16))
+    np.testing.assert_array_equal(d_rk.cpu().numpy().view(np.uint16), rk_ref.view(np.uint16))
+    np.testing.assert_array_equal(dev.cache.cpu().numpy(), cache_ref)
+    np.testing.assert_array_equal(dev.scale.cpu().numpy().view(np.uint16), scale_ref.view(np.uint16))
