@@ -110,11 +110,21 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
     const char* const scale_v = scale_k + (a.cache_stride_kv >> 3) * 2;
     const float logit_scale = a.attn_scale * kLog2e;
 
-    int b = find_sequence(kvstarts, a.kvstarts, (int)a.decoding_batches, r0, (int)(threadIdx.x & 63));
-    for (; b < a.decoding_batches; ++b) {
-        const int64_t first_token = kvstarts[b] - kv_base;
+    // The index entries of a sequence are read one sequence ahead (the first one's come out of the search): a piece
+    // that follows another in the range starts at its sequence's first token, so kvstarts and the first page table
+    // entry (contiguous cache: the sequence's first row) are known when the piece before it begins.
+    int64_t seq_start, seq_end, ahead_end = 0, ahead_row = 0, first_row = 0;
+    bool have_first_row = false;
+    int b = find_sequence(kvstarts, a.kvstarts, (int)a.decoding_batches, r0, (int)(threadIdx.x & 63), seq_start, seq_end);
+    for (; b < a.decoding_batches; ++b, seq_start = seq_end, seq_end = ahead_end, first_row = ahead_row, have_first_row = true) {
+        const int64_t first_token = seq_start - kv_base;
         if (stream_length(first_token, b) >= r1) break; // the sequence's interval starts beyond the range
-        const int64_t len = kvstarts[b + 1] - kv_base - first_token;
+        const int64_t len = seq_end - seq_start;
+        {
+            const int64_t nb1 = b + 1 < a.decoding_batches ? b + 1 : b;
+            ahead_end = kvstarts[nb1 + 1];
+            ahead_row = cachestarts[PAGED ? nb1 * a.cachestarts_stride_b : nb1];
+        }
         const int64_t s_beg = sequence_origin(first_token, b);
         int64_t pa, pe; // this workgroup's piece [pa, pe) of the sequence, in sequence coordinates
         piece_bounds(r0, r1, s_beg, len, wg_tokens, pa, pe);
@@ -129,15 +139,15 @@ __global__ __launch_bounds__(kDecodeThreads, (GT <= 4 ? 2 : 1)) void decode_atte
         const bool tail_partial = nb > 0 && pos0 + ((nb - 1) << wg_shift) + wave_tokens > pe32;
 
         const int64_t table_base = PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b;
-        const int64_t seq_row0 = PAGED ? 0 : cachestarts[b];
+        const int64_t seq_row0 = PAGED ? 0 : (have_first_row ? first_row : cachestarts[b]);
         const half_t* mask_row = nullptr;
-        if (MASK) mask_row = (const half_t*)a.attn_mask + (int64_t)b * a.mask_stride_s + kvstarts[b];
+        if (MASK) mask_row = (const half_t*)a.attn_mask + (int64_t)b * a.mask_stride_s + seq_start;
         const int last_page = (pe32 - 1) >> 7;
 
         // Page table entries are read one page ahead with scalar loads, so that no block waits
         // for its row base: `page_row` belongs to page `page_idx`, `next_row` to the page after it.
-        int page_idx = -2;
-        int64_t page_row = 0, next_row = 0;
+        int page_idx = have_first_row ? -1 : -2; // the row of page 0 read ahead stands in as the "next page" of page -1
+        int64_t page_row = 0, next_row = first_row;
         auto row_base_of = [&](int pos) -> int64_t {
             if (!PAGED) return seq_row0 + pos;
             const int pg = pos >> 7;

@@ -137,6 +137,48 @@ __device__ __forceinline__ int find_sequence(const_i64_ptr starts, const int64_t
     return lo;
 }
 
+// The same search, which also hands out starts[b] and starts[b + 1] of the sequence it finds (undefined when it
+// returns n): in the counted form two lanes hold them already, so the workgroup's first piece does not begin with
+// another pair of dependent loads.
+__device__ __forceinline__ int64_t lane_value(int64_t v, int src_lane)
+{
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(uint64_t)v, src_lane);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)((uint64_t)v >> 32), src_lane);
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ int find_sequence(const_i64_ptr starts, const int64_t* starts_global, int n, int64_t g, int lane,
+                                             int64_t& seq_start, int64_t& seq_end)
+{
+    const int64_t base = starts[0];
+    seq_start = base;
+    seq_end = base;
+    if (n <= kCountedSequences) {
+        int count = 0;
+        bool found = false;
+        int64_t last_of_previous = base; // starts[i0] of the chunk in hand
+        for (int i0 = 0; i0 < n; i0 += kWave) {
+            const int i = i0 + lane;
+            const int64_t end_i = i < n ? starts_global[i + 1] : base;
+            const bool below = i < n && stream_length(end_i - base, i + 1) <= g;
+            const int c = __builtin_popcountll(__builtin_amdgcn_ballot_w64(below)); // the lanes below come first
+            count += c;
+            if (!found && c < kWave) { // the sequence is entry i0 + c of this chunk (or there is none: i0 + c == n)
+                found = true;
+                seq_start = c > 0 ? lane_value(end_i, c - 1) : last_of_previous;
+                seq_end = lane_value(end_i, c);
+            }
+            last_of_previous = lane_value(end_i, kWave - 1);
+        }
+        return count;
+    }
+    const int b = find_sequence(starts, starts_global, n, g, lane);
+    if (b < n) {
+        seq_start = starts[b];
+        seq_end = starts[b + 1];
+    }
+    return b;
+}
+
 
 // One block of kTB tokens for one slot: raw cache bytes as loaded, K and V staged separately.
 struct KBlock {
