@@ -190,10 +190,13 @@ __global__ __launch_bounds__(kQuantThreads) void kv_quantize_kernel(const QuantL
 
         const int64_t k_out = row * a.cache_stride_s + out_idx;
         const int64_t v_out = k_out + a.cache_stride_kv;
-        *(u32x2*)(a.cache + k_out) = kq.q;
-        *(u32x2*)(a.cache + v_out) = vq.q;
-        ((half_t*)a.scale)[k_out >> 3] = kq.scale;
-        ((half_t*)a.scale)[v_out >> 3] = vq.scale;
+        // Non-temporal: a wave writes whole lines (16 lanes x 8 bytes per row of a head, 64 scales), nothing here
+        // reads them again, and lines left dirty in the memory-side cache are written back during the kernel that
+        // runs next: the decode launch behind a prefill step's append (28 MB of rows) then took 17 us longer.
+        __builtin_nontemporal_store(kq.q, (u32x2*)(a.cache + k_out));
+        __builtin_nontemporal_store(vq.q, (u32x2*)(a.cache + v_out));
+        __builtin_nontemporal_store(kq.scale, &((half_t*)a.scale)[k_out >> 3]);
+        __builtin_nontemporal_store(vq.scale, &((half_t*)a.scale)[v_out >> 3]);
     }
 }
 
@@ -369,10 +372,10 @@ __global__ __launch_bounds__(kQuantThreads) void rope_append_kernel(const RopeLa
             const Quantised vq = quantise_group(vraw);
             const int64_t k_out = s_row[r.tl] * a.cache_stride_s + a.layer_idx * a.cache_stride_l + (int64_t)r.h * a.cache_stride_h + r.d0;
             const int64_t v_out = k_out + a.cache_stride_kv;
-            *(u32x2*)(a.cache + k_out) = kq.q;
-            *(u32x2*)(a.cache + v_out) = vq.q;
-            ((half_t*)a.scale)[k_out >> 3] = kq.scale;
-            ((half_t*)a.scale)[v_out >> 3] = vq.scale;
+            __builtin_nontemporal_store(kq.q, (u32x2*)(a.cache + k_out));
+            __builtin_nontemporal_store(vq.q, (u32x2*)(a.cache + v_out));
+            __builtin_nontemporal_store(kq.scale, &((half_t*)a.scale)[k_out >> 3]);
+            __builtin_nontemporal_store(vq.scale, &((half_t*)a.scale)[v_out >> 3]);
         }
     };
 

@@ -51,6 +51,12 @@ struct PrefillTile {
     static constexpr int K_STRIDE = D + 8;
     static constexpr int V_STRIDE = ((D + 32) * 2) % 128 == 64 ? D + 32 : D + 64;
 };
+// first half of the epilogue's staging area: the start of the second tile buffer
+template <int D, int SRC>
+constexpr int kEpilogueBase()
+{
+    return (SRC == 2 ? 1 : 2) * kBN * (PrefillTile<D>::K_STRIDE + PrefillTile<D>::V_STRIDE);
+}
 static_assert((PrefillTile<128>::V_STRIDE * 2) % 256 == 64 && (PrefillTile<64>::V_STRIDE * 2) % 256 == 192 &&
                   (PrefillTile<96>::V_STRIDE * 2) % 256 == 64,
               "V row stride");
@@ -646,10 +652,20 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
     }
 
     // ---- normalise and store: element i of block cb <-> channel 32 cb + 8 (i/4) + 4 hh + i%4 ----
+    // A lane holds 8-byte pieces of one output row; stored as they lie, every store instruction would touch 32 rows
+    // with 16 bytes each, and the partly written lines would wait in the caches to be completed.  The wave turns its
+    // 32 rows round in LDS instead (its own region of the second tile buffer: every wave is past the tile loop's last
+    // barrier, and the next item writes that buffer only after its prologue's barrier, which this wave joins after this)
+    // and writes whole rows, 16 bytes per lane, with the non-temporal hint: the rows are not read again by this
+    // kernel, and lines left dirty in the memory-side cache are written back during whatever runs next (a decode launch
+    // after 89 MB of such rows took 12 us longer).
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    if (col_on) {
-        half_t* op = (half_t*)a.output + (q_row0 + pos) * a.output_stride_s + (int64_t)h * D;
+    {
+        constexpr int EP_STRIDE = D + 8;                  // halves per staged row (rows stay 16-byte aligned)
+        constexpr int EP_WAVE = 32 * EP_STRIDE + 32 * 4;  // 32 rows, then their 64-bit output offsets
+        half_t* const ep = smem + kEpilogueBase<D, SRC>() + wave * EP_WAVE;
+        int64_t* const ep_off = (int64_t*)(ep + 32 * EP_STRIDE);
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb)
 #pragma unroll
@@ -657,8 +673,24 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
                 f16x4 w;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) w[e] = (half_t)(o_acc[cb][4 * r + e] * inv);
-                *(f16x4*)(op + 32 * cb + 8 * r + 4 * hh) = w;
+                *(f16x4*)(ep + l32 * EP_STRIDE + 32 * cb + 8 * r + 4 * hh) = w;
             }
+        if (hh == 0) ep_off[l32] = col_on ? (q_row0 + pos) * a.output_stride_s + (int64_t)h * D : (int64_t)-1;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        constexpr int CH = D / 8;            // 16-byte pieces per row
+        constexpr int RPI = 64 / CH;         // rows per store instruction
+        const int piece = lane % CH, row_in = lane / CH;
+#pragma unroll
+        for (int r0 = 0; r0 < 32; r0 += RPI) {
+            const int row = r0 + row_in;
+            if (row_in < RPI && row < 32) {
+                const int64_t off = ep_off[row];
+                const u32x4 w = *(const u32x4*)(ep + row * EP_STRIDE + 8 * piece);
+                if (off >= 0) __builtin_nontemporal_store(w, (u32x4*)((half_t*)a.output + off + 8 * piece));
+            }
+        }
     }
     } // items
 }
@@ -996,8 +1028,11 @@ template <int D, int SRC>
 constexpr size_t prefill_lds_bytes()
 {
     // int8 source: K hi/lo tiles + V hi/lo tiles (above the 64 KB static limit for D = 128, hence dynamic);
-    // fp16 source: one K tile and one V tile; two buffers of each
-    return 2 * (SRC == 2 ? 1 : 2) * kBN * (PrefillTile<D>::K_STRIDE + PrefillTile<D>::V_STRIDE) * sizeof(half_t);
+    // fp16 source: one K tile and one V tile; two buffers of each.  The epilogue's staging (eight waves x 32 rows and
+    // their offsets) starts where the second buffer starts and may reach beyond it.
+    constexpr size_t tiles = 2 * (SRC == 2 ? 1 : 2) * kBN * (PrefillTile<D>::K_STRIDE + PrefillTile<D>::V_STRIDE) * sizeof(half_t);
+    constexpr size_t with_epilogue = (kEpilogueBase<D, SRC>() + 8 * (32 * (D + 8) + 32 * 4)) * sizeof(half_t);
+    return tiles > with_epilogue ? tiles : with_epilogue;
 }
 
 template <int D, int SRC, bool EXTRA>
