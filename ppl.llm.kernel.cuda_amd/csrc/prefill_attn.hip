@@ -515,19 +515,28 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
                 for (int i = 0; i < 16; i += 2) mx = max3(mx, sacc[i], sacc[i + 1]);
                 mx *= sm_scale;
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            {
+                // the other half-wave's maximum through the vector unit's lane swap: a data-share permute would have
+                // to wait for every fragment read already queued behind it
+                const u32x2 both = __builtin_amdgcn_permlane32_swap(bitcast<uint32_t>(mx), bitcast<uint32_t>(mx), false, false);
+                mx = fmaxf(bitcast<float>(both[0]), bitcast<float>(both[1]));
+            }
             return fmaxf(m_run, mx);
         };
-        // part B: p = 2^(logit - max) as hi + lo halves (hi = p rounded toward zero, two at a time; lo = the exact
-        // remainder), elements [i0, i1) of the block
+        // part B: p = 2^(logit - max) as hi + lo halves (hi = p rounded to nearest, two at a time; lo = the exact
+        // remainder), elements [i0, i1) of the block.  The row sum is taken over the hi halves, one dot-product
+        // instruction per pair instead of two additions: rounded to nearest, their errors are at most 2^-12 of each
+        // term and of either sign, so the sum of a row's hundreds of terms differs from the sum of p by ~1e-5 of itself
+        // (a factor on the whole output row, against a relative tolerance of 1e-2).
         auto softmax_exp = [&](const f32x16& sacc, float bias, int i0, int i1, f16x8* ph, f16x8* pl, float& lsum) {
 #pragma unroll
             for (int i = 0; i < 16; i += 2) {
                 if (i < i0 || i >= i1) continue;
                 const float p0 = __builtin_amdgcn_exp2f(EXTRA ? sacc[i] + bias : __builtin_fmaf(sacc[i], sm_scale, bias));
                 const float p1 = __builtin_amdgcn_exp2f(EXTRA ? sacc[i + 1] + bias : __builtin_fmaf(sacc[i + 1], sm_scale, bias));
-                lsum += p0 + p1;
-                const half2_t h2 = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(p0, p1));
+                typedef float float2_t __attribute__((ext_vector_type(2)));
+                const half2_t h2 = __builtin_convertvector(float2_t{p0, p1}, half2_t);
+                lsum = __builtin_amdgcn_fdot2(h2, half2_t{(half_t)1.f, (half_t)1.f}, lsum, false);
                 const half2_t l2 = bitcast<half2_t>(__builtin_amdgcn_cvt_pkrtz(sub_half_lo(p0, h2), sub_half_hi(p1, h2)));
                 ph[i >> 3][i & 7] = h2.x;
                 ph[i >> 3][(i & 7) + 1] = h2.y;
@@ -959,8 +968,14 @@ __global__ __launch_bounds__(kPrefillThreads, D <= 128 ? 4 : 2) void prefill_att
                 v[e] = x;
                 mx = fmaxf(mx, x);
             }
-            mx = fmaxf(mx, __shfl_xor(mx, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            {
+                // across the four quarters of the wave with the vector unit's lane swaps (no data-share permute, which
+                // would wait for the fragment reads queued behind it)
+                const u32x2 rows = __builtin_amdgcn_permlane16_swap(bitcast<uint32_t>(mx), bitcast<uint32_t>(mx), false, false);
+                mx = fmaxf(bitcast<float>(rows[0]), bitcast<float>(rows[1]));
+                const u32x2 both = __builtin_amdgcn_permlane32_swap(bitcast<uint32_t>(mx), bitcast<uint32_t>(mx), false, false);
+                mx = fmaxf(bitcast<float>(both[0]), bitcast<float>(both[1]));
+            }
             const float m_new = fmaxf(m_run, mx);
             if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) { // rare after the first tiles (wave-uniform)
                 const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
