@@ -115,21 +115,11 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
 #pragma unroll
     for (int u = 0; u < VU; ++u) v_q[u] = (lane + 64 * u) / GPT;
 
-    // The index entries of a sequence are read one sequence ahead (the first one's come out of the search): a piece
-    // that follows another in the range starts at its sequence's first token, so kvstarts and the first page table
-    // entry (contiguous cache: the sequence's first row) are known when the piece before it begins.
-    int64_t seq_start, seq_end, ahead_end = 0, ahead_row = 0, first_row = 0;
-    bool have_first_row = false;
-    int b = find_sequence(kvstarts, a.kvstarts, (int)a.decoding_batches, r0, lane, seq_start, seq_end);
-    for (; b < a.decoding_batches; ++b, seq_start = seq_end, seq_end = ahead_end, first_row = ahead_row, have_first_row = true) {
-        const int64_t first_token = seq_start - kv_base;
+    int b = find_sequence(kvstarts, a.kvstarts, (int)a.decoding_batches, r0, lane);
+    for (; b < a.decoding_batches; ++b) {
+        const int64_t first_token = kvstarts[b] - kv_base;
         if (stream_length(first_token, b) >= r1) break;
-        const int64_t len = seq_end - seq_start;
-        {
-            const int64_t nb1 = b + 1 < a.decoding_batches ? b + 1 : b;
-            ahead_end = kvstarts[nb1 + 1];
-            ahead_row = cachestarts[PAGED ? nb1 * a.cachestarts_stride_b : nb1];
-        }
+        const int64_t len = kvstarts[b + 1] - kv_base - first_token;
         const int64_t s_beg = sequence_origin(first_token, b);
         int64_t pa, pe;
         piece_bounds(r0, r1, s_beg, len, kMfmaBlock, pa, pe);
@@ -138,11 +128,10 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
         const int nb = (pe32 - pa32 + kMfmaBlock - 1) / kMfmaBlock;
 
         const int64_t table_base = PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b;
-        const int64_t seq_row0 = PAGED ? 0 : (have_first_row ? first_row : cachestarts[b]);
+        const int64_t seq_row0 = PAGED ? 0 : cachestarts[b];
         // a block of 32 tokens starts on a multiple of 32 and so lies inside one 128-token page
         auto row_base_of = [&](int pos) -> int64_t {
             if (!PAGED) return seq_row0 + pos;
-            if (have_first_row && pos < kPage) return first_row + pos; // page 0 was read ahead
             return cachestarts[table_base + (pos >> 7)] + (pos & (kPage - 1));
         };
 
@@ -173,7 +162,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma_kernel(co
         const half_t* mask_row = nullptr;
         if (MASK) {
             const int h = kvh * G + (gq < G ? gq : 0);
-            mask_row = (const half_t*)a.attn_mask + (int64_t)h * a.mask_stride_h + (int64_t)b * a.mask_stride_s + seq_start;
+            mask_row = (const half_t*)a.attn_mask + (int64_t)h * a.mask_stride_h + (int64_t)b * a.mask_stride_s + kvstarts[b];
         }
 
         // ---- raw bytes of one block: K as (token l32, channels HALF hh .. + HALF), V as (token quad, group) units ----
@@ -450,21 +439,11 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
     v_q[0] = qq + 4 * (qq & 1);
     v_q[1] = qq + 4 * ((qq & 1) ^ 1);
 
-    // The index entries of a sequence are read one sequence ahead (the first one's come out of the search): a piece
-    // that follows another in the range starts at its sequence's first token, so kvstarts and the first page table
-    // entry (contiguous cache: the sequence's first row) are known when the piece before it begins.
-    int64_t seq_start, seq_end, ahead_end = 0, ahead_row = 0, first_row = 0;
-    bool have_first_row = false;
-    int b = find_sequence(kvstarts, a.kvstarts, (int)a.decoding_batches, r0, lane, seq_start, seq_end);
-    for (; b < a.decoding_batches; ++b, seq_start = seq_end, seq_end = ahead_end, first_row = ahead_row, have_first_row = true) {
-        const int64_t first_token = seq_start - kv_base;
+    int b = find_sequence(kvstarts, a.kvstarts, (int)a.decoding_batches, r0, lane);
+    for (; b < a.decoding_batches; ++b) {
+        const int64_t first_token = kvstarts[b] - kv_base;
         if (stream_length(first_token, b) >= r1) break;
-        const int64_t len = seq_end - seq_start;
-        {
-            const int64_t nb1 = b + 1 < a.decoding_batches ? b + 1 : b;
-            ahead_end = kvstarts[nb1 + 1];
-            ahead_row = cachestarts[PAGED ? nb1 * a.cachestarts_stride_b : nb1];
-        }
+        const int64_t len = kvstarts[b + 1] - kv_base - first_token;
         const int64_t s_beg = sequence_origin(first_token, b);
         int64_t pa, pe;
         piece_bounds(r0, r1, s_beg, len, kMfmaBlock, pa, pe);
@@ -473,11 +452,10 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
         const int nb = (pe32 - pa32 + kMfmaBlock - 1) / kMfmaBlock;
 
         const int64_t table_base = PAGED ? (int64_t)b * a.cachestarts_stride_b : (int64_t)b;
-        const int64_t seq_row0 = PAGED ? 0 : (have_first_row ? first_row : cachestarts[b]);
+        const int64_t seq_row0 = PAGED ? 0 : cachestarts[b];
         // a block of 32 tokens starts on a multiple of 32 and so lies inside one 128-token page
         auto row_base_of = [&](int pos) -> int64_t {
             if (!PAGED) return seq_row0 + pos;
-            if (have_first_row && pos < kPage) return first_row + pos; // page 0 was read ahead
             return cachestarts[table_base + (pos >> 7)] + (pos & (kPage - 1));
         };
 
@@ -507,7 +485,7 @@ __global__ __launch_bounds__(NW * kWave, 2) void decode_attention_mfma16_kernel(
         const half_t* mask_row = nullptr;
         if (MASK) {
             const int h = kvh * G + (r16 < G ? r16 : 0);
-            mask_row = (const half_t*)a.attn_mask + (int64_t)h * a.mask_stride_h + (int64_t)b * a.mask_stride_s + seq_start;
+            mask_row = (const half_t*)a.attn_mask + (int64_t)h * a.mask_stride_h + (int64_t)b * a.mask_stride_s + kvstarts[b];
         }
 
         // ---- raw bytes of one block: K of tokens r16 and 16 + r16, V as two (token quad, group) units ----
