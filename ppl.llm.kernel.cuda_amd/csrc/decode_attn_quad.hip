@@ -313,7 +313,13 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
         // loads in flight when a block's logits start: its own, the V block before it and the next K block;
         // a K block has two more requests with the mask
         constexpr int kMoreK = MASK ? 4 : 0, kMoreV = MASK ? 2 : 0;
-        auto logits_softmax = [&](KBlock& kx, uint32_t (&mk)[2], bool beyond_piece) { // beyond_piece: the block reaches past the piece (wave-uniform)
+        // last: the piece's last block, behind which nothing but its own V block has been requested: one wait for the
+        // whole K block then, since the counts below take a further K block's requests for granted (wave-uniform)
+        auto logits_softmax = [&](KBlock& kx, uint32_t (&mk)[2], bool beyond_piece, bool last) { // beyond_piece: the block reaches past the piece (wave-uniform)
+            if (last) {
+                wait_block<8>(kx.q8, kx.sc);
+                if (MASK) wait_loads<8>(mk[0], mk[1]);
+            }
             float part[4][kTB]; // [head][step], over this lane's 16 channels, log2 units
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
@@ -467,7 +473,8 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
             }
         };
 
-        auto accumulate_pv = [&](VBlock& vx) {
+        auto accumulate_pv = [&](VBlock& vx, bool last) { // last: nothing requested behind this V block
+            if (last) wait_block<0>(vx.q8, vx.sc);
 #pragma unroll
             for (int j = 0; j < kTB; ++j) {
                 if (j == 0) wait_loads<22 + kMoreV>(vx.q8[0], vx.sc[0]);
@@ -516,24 +523,30 @@ __global__ __launch_bounds__(kWave * WP * GP, 2) void decode_attention_quad_kern
             // block of each other, so that the second set's requests find the lines in the cache levels
             // (every wave of the workgroup runs the same number of blocks).
             if (GP > 1) __syncthreads();
+            // The piece's last block requests nothing: what it requested would only be waited for before the merge, a
+            // memory latency per piece for nothing.
+            bool last = i + 1 == nb;
             int npos = npos_first;
-            if (i > 0) {
-                npos = pos + (i + 1 < nb ? BLK : 0);
+            if (i > 0 && !last) {
+                npos = pos + BLK;
                 if (tail_partial && i + 2 == nb) clamp_offsets(npos);
                 request_k(kb, mkb, npos);
             }
-            logits_softmax(ka, mka, tail_partial && i + 1 == nb);
-            request_v(vb, kb.boff);
-            accumulate_pv(va);
+            logits_softmax(ka, mka, tail_partial && last, last);
+            if (!last) request_v(vb, kb.boff);
+            accumulate_pv(va, last);
             pin_acc();
             pos = npos;
             if (++i == nb) break;
-            npos = pos + (i + 1 < nb ? BLK : 0);
-            if (tail_partial && i + 2 == nb) clamp_offsets(npos);
-            request_k(ka, mka, npos);
-            logits_softmax(kb, mkb, tail_partial && i + 1 == nb);
-            request_v(va, ka.boff);
-            accumulate_pv(vb);
+            last = i + 1 == nb;
+            if (!last) {
+                npos = pos + BLK;
+                if (tail_partial && i + 2 == nb) clamp_offsets(npos);
+                request_k(ka, mka, npos);
+            }
+            logits_softmax(kb, mkb, tail_partial && last, last);
+            if (!last) request_v(va, ka.boff);
+            accumulate_pv(vb, last);
             pin_acc();
             pos = npos;
             if (++i == nb) break;

@@ -52,6 +52,14 @@ __device__ __forceinline__ void wait_loads(uint32_t& a, uint32_t& b)
 {
     asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N));
 }
+// waits until at most N vector memory operations are outstanding, for a whole block's staging registers
+template <int N>
+__device__ __forceinline__ void wait_block(u32x4 (&q)[4], uint32_t (&sc)[4])
+{
+    asm volatile("s_waitcnt vmcnt(%8)"
+                 : "+v"(q[0]), "+v"(q[1]), "+v"(q[2]), "+v"(q[3]), "+v"(sc[0]), "+v"(sc[1]), "+v"(sc[2]), "+v"(sc[3])
+                 : "n"(N));
+}
 // one half (an attn_mask value) per lane, zero-extended
 __device__ __forceinline__ void load_u16(uint32_t& dst, uint32_t lane_off, const char* wave_base)
 {
