@@ -13,7 +13,7 @@ the whole step time (GB/s).  The K timed steps are K layer calls recorded once i
 graph; the graph is replayed R >= 10 times back to back with an event between the replays,
 and the step time is the MEDIAN replay divided by K (`replays_us_per_layer` also gives the
 first and the fastest; `--eager` times host-launched kernels instead, which is also
-reported as `us_per_layer_eager`).  `roofline` prices the dominant kernel alone (the
+reported as `us_per_layer_eager` (sustained) and `us_per_layer_eager_from_idle`).  `roofline` prices the dominant kernel alone (the
 token-range decode kernel, named by the library) in the same regime: a graph of K launches
 of that kernel, replayed and timed the same way on the stream it is launched on; the
 figure of an event-separated launch loop is given beside it (`stages_us`).
@@ -355,12 +355,25 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    # Host-launched kernels: K timed calls bracketed by synchronisations (the chip starts them from idle: its first
+    # launches after a synchronisation run slower, about a millisecond in all), and K more calls timed by two events
+    # behind K calls that were enqueued without a synchronisation in between (the sustained rate of a loop that
+    # keeps the queue filled).
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
     torch.cuda.synchronize()
-    eager_s = (time.perf_counter() - t0) / args.steps
-    step_s, launch = eager_s, "one launch per kernel from the host (eager)"
+    eager_from_idle_s = (time.perf_counter() - t0) / args.steps
+    ev_a, ev_b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(args.steps):
+        step()
+    ev_a.record(stream)
+    for _ in range(args.steps):
+        step()
+    ev_b.record(stream)
+    torch.cuda.synchronize()
+    eager_s = ev_a.elapsed_time(ev_b) * 1e-3 / args.steps
+    step_s, launch = eager_from_idle_s, "one launch per kernel from the host (eager), timed from idle"
     replays = max(10, args.replays)
     ws = op.workspace
     if ws is None or ws.numel() < int(plan.workspace_size):  # --ranges asked for more ranges than the operator plans
@@ -494,6 +507,7 @@ def main():
         "ms_per_step": step_s * 1e3,
         "us_per_layer": step_s * 1e6,
         "us_per_layer_eager": eager_s * 1e6,
+        "us_per_layer_eager_from_idle": eager_from_idle_s * 1e6,
         "launch": launch,
         "replays_us_per_layer": summary(layer_replays) if layer_replays else None,
         "higher_is_better": True,
