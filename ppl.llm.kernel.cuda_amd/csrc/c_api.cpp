@@ -248,10 +248,11 @@ int pmxhip_decode_plan_make_kernel(int64_t decoding_batches, int64_t num_heads, 
         const int64_t groups = ((num_kv_heads + c.kv_heads_per_group - 1) / c.kv_heads_per_group) * c.num_passes;
         int cus = compute_units > 0 ? compute_units : current_compute_units();
         if (cus <= 0) return fail(PMXHIP_INVALID_VALUE, "decode_plan: compute_units not given and no current device");
-        // as many ranges as fill the workgroup slots of the chip: two workgroups of four waves per CU, or as many as
-        // eight waves make where a kernel with smaller workgroups serves the shape (a wave per kv head, or per two)
-        const int64_t slots = (int64_t)cus * c.wgs_per_cu;
-        ranges = (slots + groups - 1) / groups;
+        // as many ranges as the kernel wants workgroups per CU for a long stream (decode_select.cpp: the quad kernel
+        // one wave per SIMD, the others two; more, smaller workgroups where a wave serves one or two kv heads)
+        const int64_t long_slots = (int64_t)cus * c.wgs_per_cu;
+        const int64_t slots = (int64_t)cus * c.wgs_per_cu_short; // what the rules for short batches below count with
+        ranges = (long_slots + groups - 1) / groups;
         // A short batch: ranges of about 128 tokens (twice the smallest) where those still fill half of the slots,
         // shorter ones -- down to the smallest -- only to get that far: a piece has a fixed cost, and an idle CU costs more.
         const int64_t max_tokens = decoding_batches * (max_kvlen > 0 ? max_kvlen : 1);

@@ -73,6 +73,7 @@ bool decode_choose(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, in
             c.num_passes = (int32_t)((g + gt - 1) / gt);
             c.wg_tokens = decode_wg_tokens((int)head_dim, c.kv_heads_per_group);
             c.wgs_per_cu = 2;
+            c.wgs_per_cu_short = c.wgs_per_cu;
             break;
         }
         case kDecodeKernelQuad: {
@@ -84,8 +85,18 @@ bool decode_choose(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, in
             c.q_heads_per_pass = g <= 1 ? 1 : (g <= 2 ? 2 : (g <= 4 ? 4 : 8)); // rows of the 4x4x4 products in use
             c.num_passes = 1;
             c.wg_tokens = head_dim == 64 ? 2 * kDecodeQuadTokens : kDecodeQuadTokens; // head_dim 64: blocks of 32 tokens
-            c.wgs_per_cu = (head_dim == 256 ? 8 : 16) / c.kv_heads_per_group;
-            if (head_dim == 256 && g > 4) c.wgs_per_cu = c.wgs_per_cu > 1 ? c.wgs_per_cu / 2 : 1; // twice the waves per workgroup
+            // A CU holds eight of this kernel's waves, two per SIMD.  A long stream is cut for four, one per SIMD: the
+            // second wave adds nothing to what the chip streams (each wave keeps three blocks of rows in flight), and
+            // half as many ranges are half as many pieces to write and to combine.  Short batches, whose ranges are a
+            // few blocks, still spread over all eight (their waves mostly wait), and so do the form with two sets of
+            // waves per workgroup (head_dim 256 with more than four query heads per kv head: 43 against 57 us on 8 / 1
+            // heads) and the workgroups of two waves (four kv heads: two such workgroups per CU ran 22 % slower than
+            // four, 216 against 177 us -- their waves do not end up one per SIMD).
+            const int waves = c.kv_heads_per_group / per_wave; // per set
+            c.wgs_per_cu_short = 8 / waves;
+            if (head_dim == 256 && g > 4) c.wgs_per_cu_short = c.wgs_per_cu_short > 1 ? c.wgs_per_cu_short / 2 : 1; // twice the waves per workgroup
+            const bool one_per_simd = !(head_dim == 256 && g > 4) && waves != 2;
+            c.wgs_per_cu = one_per_simd ? c.wgs_per_cu_short / 2 : c.wgs_per_cu_short;
             break;
         }
         case kDecodeKernelMfma16:
@@ -98,6 +109,7 @@ bool decode_choose(int64_t head_dim, int64_t num_heads, int64_t num_kv_heads, in
             c.num_passes = (int32_t)((g + cols - 1) / cols);
             c.wg_tokens = kDecodeMfmaTokens;
             c.wgs_per_cu = kDecodeMfmaWavesPerCu / c.kv_heads_per_group;
+            c.wgs_per_cu_short = c.wgs_per_cu;
             break;
         }
         default: return false;

@@ -248,7 +248,8 @@ struct DecodeChoice {
     int32_t q_heads_per_pass;   // query heads per kv head served by one pass (general kernel: 1, 2, 4 or 8)
     int32_t num_passes;
     int32_t wg_tokens;          // tokens per workgroup iteration = unit of the range cuts
-    int32_t wgs_per_cu;         // workgroups that a CU holds at once (sizes the number of ranges)
+    int32_t wgs_per_cu;         // workgroups per CU that a long stream is cut for (sizes the number of ranges)
+    int32_t wgs_per_cu_short;   // ... and that a CU can hold: what short batches, whose ranges are a few blocks, are spread over
 };
 // The kernel that serves a shape, and the grouping it implies.  `requested` kDecodeKernelAuto picks by shape;
 // any other value insists on that kernel and the call fails (false) when it cannot serve the shape.

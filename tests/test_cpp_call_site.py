@@ -26,9 +26,9 @@ def test_reference_style_call_site_compiles_links_and_runs(pkg, hip_lib, tmp_pat
     lines = r.stdout.splitlines()
     assert lines[0] == "prepare rc=0"
     scale = float(np.float32(1.0 / np.sqrt(np.float32(128))))
-    pieces = 512 + 128  # two workgroups per CU on 256 CUs, one group of eight kv heads; one more piece per sequence
+    pieces = 256 + 128  # one workgroup of four waves per CU on 256 CUs, one group of eight kv heads; one more piece per sequence
     assert lines[1] == ("prefill_batches=0 q_stride_s=4096 k_stride_s=1024 o_stride_s=4096 num_kv_repeats=4 "
-                        "attn_scale=%.9g decoding_algo=3 multi_block=512 workspace_size=%d" % (scale, pieces * 32 * 130 * 4))
+                        "attn_scale=%.9g decoding_algo=3 multi_block=256 workspace_size=%d" % (scale, pieces * 32 * 130 * 4))
     assert lines[2] == "device_prop kept by pointer: 1"
     assert lines[3] == "bad heads rc=2"
     assert lines[4] == "idle prepare rc=0 kvstore=0 decode=0 prefill=0 forward=0"

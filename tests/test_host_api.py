@@ -123,11 +123,11 @@ def test_forward_before_prepare_is_rejected(pkg, hip_lib):
 def test_decode_plan(pkg, hip_lib):
     plan = pkg.ops.decode_plan(128, 32, 8, 128, 8192, cus=256)
     assert plan.kv_heads_per_group == 8 and plan.q_heads_per_pass == 4 and plan.num_passes == 1
-    assert plan.num_token_ranges == 512
+    assert plan.num_token_ranges == 256  # the quad kernel: a long stream is cut for one wave per SIMD
     pieces = plan.num_token_ranges + 128
     assert plan.partial_out_size == pieces * 32 * 128 * 4 and plan.partial_ml_size == pieces * 32 * 2 * 4
     plan = pkg.ops.decode_plan(64, 32, 32, 128, 4096, cus=256)  # MHA: 4 groups of 8 kv heads
-    assert plan.kv_heads_per_group == 8 and plan.q_heads_per_pass == 1 and plan.num_token_ranges == 128
+    assert plan.kv_heads_per_group == 8 and plan.q_heads_per_pass == 1 and plan.num_token_ranges == 64
     plan = pkg.ops.decode_plan(32, 64, 8, 128, 32768, cus=256)  # G = 8: MFMA kernel, 4 kv heads per workgroup, 16 columns
     assert plan.q_heads_per_pass == 16 and plan.num_passes == 1 and plan.kv_heads_per_group == 4
     assert plan.num_token_ranges == 256
@@ -168,7 +168,7 @@ def test_decode_plan_names_its_kernel(pkg, hip_lib):
         plan = pkg.ops.decode_plan(16, hq, hkv, d, 4096, cus=256)
         assert (plan.kernel, plan.q_heads_per_pass, plan.num_passes) == (L.DECODE_KERNEL_MFMA32, 32, passes), (hq, hkv, d)
     # requests: every kernel on the Llama-3-70B shape (8 query heads per kv head, kv heads in eights)
-    for k, (kvhb, gt, ranges) in {L.DECODE_KERNEL_GENERAL: (8, 8, 512), L.DECODE_KERNEL_QUAD: (8, 8, 512),
+    for k, (kvhb, gt, ranges) in {L.DECODE_KERNEL_GENERAL: (8, 8, 512), L.DECODE_KERNEL_QUAD: (8, 8, 256),
                                   L.DECODE_KERNEL_MFMA16: (4, 16, 256), L.DECODE_KERNEL_MFMA32: (4, 32, 256)}.items():
         plan = pkg.ops.decode_plan(32, 64, 8, 128, 32768, cus=256, kernel=k)
         assert (plan.kernel, plan.kv_heads_per_group, plan.q_heads_per_pass, plan.num_token_ranges) == (k, kvhb, gt, ranges)
