@@ -688,6 +688,8 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // 16-byte stores need rows that start on 16-byte addresses (wave-uniform: a property of the launch)
+        const bool wide_rows = ((uintptr_t)a.output & 15u) == 0 && (a.output_stride_s & 7) == 0;
         constexpr int CH = D / 8;            // 16-byte pieces per row
         constexpr int RPI = 64 / CH;         // rows per store instruction
         const int piece = lane % CH, row_in = lane / CH;
@@ -697,7 +699,15 @@ __global__ __launch_bounds__(kPrefillThreads, 2) void prefill_attention_kernel(c
             if (row_in < RPI && row < 32) {
                 const int64_t off = ep_off[row];
                 const u32x4 w = *(const u32x4*)(ep + row * EP_STRIDE + 8 * piece);
-                if (off >= 0) __builtin_nontemporal_store(w, (u32x4*)((half_t*)a.output + off + 8 * piece));
+                if (off >= 0) {
+                    half_t* const dst = (half_t*)a.output + off + 8 * piece;
+                    if (wide_rows) {
+                        __builtin_nontemporal_store(w, (u32x4*)dst);
+                    } else { // output rows aligned to 8 bytes only
+                        *(u32x2*)dst = u32x2{w[0], w[1]};
+                        *(u32x2*)(dst + 4) = u32x2{w[2], w[3]};
+                    }
+                }
             }
         }
     }

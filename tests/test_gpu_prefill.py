@@ -283,3 +283,25 @@ def test_prefill_from_current_key_value(pkg, oracle, shape):
     assert op.forward_prefill() == 0
     torch.cuda.synchronize()
     assert_attention_close(dev.output.float().cpu().numpy()[n_dec:], ref[n_dec:], "operator, enable_cache_prefill=false")
+
+
+def test_prefill_output_rows_aligned_to_8_bytes_only(pkg, oracle):
+    """The C ABI admits output rows that are 8-byte aligned.  The tile kernel writes whole rows in 16-byte pieces where
+    the rows allow it and in 8-byte pieces otherwise: same values, nothing written outside the rows."""
+    bt, dev, q, cache, scale = make_case(pkg, oracle, 330, num_heads=8, num_kv_heads=2, head_dim=128, cache_mode=1,
+                                         dec_kv_lens=[], prefill_q_lens=[70, 5, 129], prefill_prior=[130, 0, 300])
+    ref = oracle_prefill(oracle, bt, q, cache, scale)
+    got = run_prefill(pkg, dev)
+    assert_attention_close(got, ref, "16-byte rows")
+    n = dev.output.numel()
+    buf = torch.full((n + 8,), float("nan"), dtype=torch.float16, device="cuda")
+    out = buf[4:4 + n].view(dev.output.shape)
+    assert out.data_ptr() % 16 == 8
+    keep = dev.output
+    dev.output = out
+    try:
+        got8 = run_prefill(pkg, dev)
+    finally:
+        dev.output = keep
+    np.testing.assert_array_equal(got8, got)
+    assert torch.isnan(buf[:4]).all() and torch.isnan(buf[4 + n:]).all()
